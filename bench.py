@@ -1,0 +1,205 @@
+"""Headline benchmark: Qwen2.5-VL-7B vision encoder forward, bf16, 8 x 448x448 images (8192 patches), one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+A step is one forward pass of the 32-block encoder over the batch, inputs already resident in HBM as
+bf16 (the reference's `.to(device, dtype)` at qwen2_5_vl.py:415-419 is outside the timed region), ending
+with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
+
+  value / unit          whole-job patches per second (also images_per_s, ms_per_step)
+  roofline              the dominant kernel (gate|up GEMM with the SiLU*mul epilogue, one launch per block):
+                        algorithmic FLOPs per launch / average launch duration, measured with HIP events on
+                        the launch stream inside the timed region, against the bf16 dense MFMA peak
+  breakdown             per-stage device time from a separately instrumented pass, and the MFMA fraction
+                        over GEMM+attention time (the target the build is held to)
+  cpu_baseline          the CPU oracle (a port of the reference's algorithm, plain PyTorch) timed on this
+                        host's cores on a bounded sample of the same workload
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+from collections import defaultdict
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak (2.5 PFLOP/s)
+N_IMAGES = 8
+GRID = (1, 32, 32)          # 448 x 448, patch 14
+
+
+def algorithmic_flops(L: int, n_images: int, depth: int = 32, n_full: int = 4) -> dict:
+    H, I, K0, O = 1280, 3420, 1176, 3584
+    per_img = L // n_images
+    f = {
+        "gemm_qkv": 2.0 * L * H * 3 * H,
+        "gemm_proj": 2.0 * L * H * H,
+        "gemm_gate_up": 2.0 * L * H * 2 * I,
+        "gemm_down": 2.0 * L * I * H,
+        "attn_window": 4.0 * 64 * H * L,
+        "attn_full": 4.0 * per_img * H * L,
+        "patch_embed": 2.0 * L * K0 * H,
+        "gemm_merger": (L / 4) * (2.0 * 5120 * 5120 + 2.0 * 5120 * O),
+    }
+    total = (depth * (f["gemm_qkv"] + f["gemm_proj"] + f["gemm_gate_up"] + f["gemm_down"])
+             + (depth - n_full) * f["attn_window"] + n_full * f["attn_full"] + f["patch_embed"] + f["gemm_merger"])
+    f["total"] = total
+    return f
+
+
+class EventMarks:
+    """Records a HIP event on the current (launch) stream at every mark; durations are mark-to-next-mark."""
+
+    def __init__(self, torch, only: set | None = None):
+        self.torch = torch
+        self.only = only
+        self.events: list = []
+        self.prev_kept = False
+
+    def __call__(self, name: str) -> None:
+        keep = self.only is None or name in self.only
+        if keep or self.prev_kept:
+            ev = self.torch.cuda.Event(enable_timing=True)
+            ev.record()
+            self.events.append((name, ev))
+        self.prev_kept = keep
+
+    def durations_ms(self) -> dict:
+        out = defaultdict(list)
+        for (name, ev), (_, nxt) in zip(self.events[:-1], self.events[1:]):
+            if self.only is None or name in self.only:
+                out[name].append(ev.elapsed_time(nxt))
+        return out
+
+
+def cpu_baseline(sd, n_sample_images: int) -> dict:
+    """Time the CPU oracle (bf16, all host threads) on `n_sample_images` of the batch's 8 images."""
+    import torch
+
+    from cornserve_amd import synth
+    from oracle import qwen2_5_vl as oq
+
+    threads = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    ocfg = oq.QwenVisionConfig()
+    px, grid = synth.qwen_inputs([GRID] * n_sample_images, seed=0)
+    sd16 = {k: v.to(torch.bfloat16) for k, v in sd.items()}
+    warm_cfg = oq.QwenVisionConfig(depth=1, fullatt_block_indexes=[0])
+    oq.forward(sd16, warm_cfg, px[:1], grid[:1], dtype=torch.bfloat16)  # thread pool / allocator warm-up
+    t0 = time.perf_counter()
+    out = oq.forward(sd16, ocfg, px, grid, dtype=torch.bfloat16)
+    dt = time.perf_counter() - t0
+    patches = n_sample_images * GRID[0] * GRID[1] * GRID[2]
+    assert len(out) == n_sample_images
+    return {
+        "value": patches / dt, "unit": "patches/s", "cores": threads, "kind": "port",
+        "sample": f"{n_sample_images} of the 8 images ({patches} patches) through the full 32-block encoder, "
+                  f"bf16 step-wise CPU oracle, 1 iteration, {dt:.1f} s",
+    }
+
+
+def main() -> None:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-sample-images", type=int, default=2)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (every image is independent; more GPUs would each "
+              "take a slice of the batch with a full weight replica); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+
+    from cornserve_amd import lib, synth
+    from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
+
+    lib.load()
+    dev = torch.device("cuda:0")
+    cfg = synth.qwen_vision_config()
+    sd = synth.qwen_state_dict(cfg, seed=0)
+    model = Qwen2_5_VisionTransformer(cfg)
+    model.load_state_dict(sd, strict=False)
+    model = model.to(device=dev, dtype=torch.bfloat16).eval()
+    px, grid = synth.qwen_inputs([GRID] * N_IMAGES, seed=0)
+    pixel_values = torch.cat(px).to(device=dev, dtype=torch.bfloat16)
+    grid_np = torch.cat(grid).numpy().astype(np.int64)
+    L = pixel_values.shape[0]
+    flops = algorithmic_flops(L, N_IMAGES)
+
+    with torch.inference_mode():
+        for _ in range(args.warmup):
+            out = model.forward_device(pixel_values, grid_np)
+        torch.cuda.synchronize()
+        marks = EventMarks(torch, only={"gemm_gate_up"})
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            out = model.forward_device(pixel_values, grid_np, mark=marks)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        assert len(out) == N_IMAGES and out[0].shape == (256, 3584)
+        assert torch.isfinite(out[0].float()).all()
+        gu = marks.durations_ms()["gemm_gate_up"]
+        gu_ms = sum(gu) / len(gu)
+
+        # separately instrumented pass: every stage bracketed by events
+        full = EventMarks(torch)
+        for _ in range(3):
+            model.forward_device(pixel_values, grid_np, mark=full)
+        torch.cuda.synchronize()
+    stage_ms = {k: sum(v) / 3 for k, v in full.durations_ms().items()}
+    mfma_keys = [k for k in stage_ms if k.startswith("gemm_") or k.startswith("attn_") or k == "patch_embed"]
+    mfma_ms = sum(stage_ms[k] for k in mfma_keys)
+    ms_per_step = dt / args.steps * 1e3
+    achieved = flops["gemm_gate_up"] / (gu_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": "ViT patches/sec on 1 MI355X (Qwen2.5-VL-7B encoder, bf16); % MFMA peak",
+        "value": L / (dt / args.steps),
+        "unit": "patches/s",
+        "images_per_s": N_IMAGES / (dt / args.steps),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic (seeded N(0,1) patches, N(0,0.02) random-init weights)",
+        "config": {"workload": "configs[1]: 32-block Qwen2.5-VL-7B ViT, bf16, 8 x 448x448 images = 8192 patches, "
+                               "window attention 8x8 patches, full attention at blocks 7/15/23/31, "
+                               "merger to 2048 x 3584", "patches": L, "images": N_IMAGES},
+        "roofline": {
+            "bound": "mfma", "kernel": "gemm_kernel<256,256,SWIGLU> (gate|up projection, 8192x6912x1280 launched, "
+                                       "8192x6840x1280 algorithmic)",
+            "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
+            "avg_launch_ms": gu_ms, "launches_timed": len(gu), "traffic": None,
+        },
+        "breakdown": {
+            "stage_ms_per_step": {k: round(v, 4) for k, v in sorted(stage_ms.items())},
+            "gemm_attention_ms": mfma_ms,
+            "algorithmic_tflop_per_step": flops["total"] / 1e12,
+            "mfma_frac_over_gemm_attention_time": flops["total"] / (mfma_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "mfma_frac_over_whole_step": flops["total"] / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        },
+    }
+    if not args.no_cpu_baseline:
+        del model
+        torch.cuda.empty_cache()
+        result["cpu_baseline"] = cpu_baseline(sd, args.cpu_sample_images)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

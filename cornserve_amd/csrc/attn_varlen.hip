@@ -1,0 +1,311 @@
+// Variable-length, non-causal flash attention on MFMA for gfx950.
+//
+// Replaces flash_attn_varlen_func (eric/models/qwen2_5_vl.py:110-120: block-diagonal attention over
+// cu_seqlens segments, softmax scale head_dim^-0.5, no dropout, no mask inside a segment) and
+// xformers memory_efficient_attention_forward (eric/models/layers/attention.py:51, one segment per
+// image).  Optionally applies the Qwen2.5-VL rotary embedding (qwen2_5_vl.py:26-33) to q and k while
+// they are staged into LDS, so the rotated tensors never exist in HBM.
+//
+// Decomposition.  A workgroup owns one query block (<= 32*NWAVES rows of one segment) of one head and
+// streams that segment's keys/values through LDS in tiles of 64.  Each wave owns 32 query rows.
+// Both products are computed TRANSPOSED so that a lane owns one query column of every accumulator:
+//     S^T[key][q] = K[key][:] . Q[q][:]      (MFMA A operand = K rows, B operand = Q rows, k = head dim)
+//     O^T[d][q]  += V^T[d][key] . P^T[key][q] (A operand = V^T rows, B operand = P, k = keys)
+// With the 32x32 accumulator layout (lane -> column q = lane%32, 16 rows per lane) the online-softmax
+// max / sum over keys is 32 in-register operations plus one exchange with lane^32, the rescale of O is
+// a per-lane scalar, and P goes from the S accumulators straight into the B operand of the second
+// product without touching LDS: accumulator rows 8kk..8kk+7 of a lane are keys
+// {16kk+4h+0..3, 16kk+8+4h+0..3} (h = lane/32); the V^T fragment is read from LDS with the same key
+// order, which is legal because a dot product does not care about the order of its terms.
+// V is transposed once per tile on its way into LDS (pairs of keys packed into 32-bit writes).
+// Head dims that are not multiples of 16 (SigLIP's 72) are zero-padded in LDS only.
+#include "common.h"
+
+namespace {
+
+constexpr int BKV = 64;        // keys per LDS tile
+constexpr int VT_STRIDE = 68;  // bf16 elements per V^T row (64 keys + 4 pad: conflict-free 8-byte reads)
+
+struct AttnArgs {
+  const bf16_t* q;
+  const bf16_t* k;
+  const bf16_t* v;
+  int64_t ld;
+  bf16_t* out;
+  int64_t ldo;
+  const int32_t* work;
+  const float* cos_sin;
+  float scale_log2e;
+};
+
+template <int D, int NWAVES, bool ROPE>
+__global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
+  constexpr int NT = NWAVES * 64;
+  constexpr int BQ = NWAVES * 32;
+  constexpr int KS = (D + 15) / 16;    // MFMA k-steps over the head dim
+  constexpr int DT = (D + 31) / 32;    // 32-row tiles of O^T
+  constexpr int DC = D / 8;            // real 16-byte chunks per row
+  constexpr int DKC = KS * 2;          // chunks per row after zero padding
+  constexpr int RS = (DKC | 1) * 16;   // LDS row stride in bytes, odd chunk count: conflict-free b128 reads
+  static_assert(D % 8 == 0 && D <= 96, "head dim");
+  static_assert(!ROPE || D % 16 == 0, "rotary needs an even number of chunks per half");
+
+  __shared__ __attribute__((aligned(16))) char q_lds[BQ * RS];
+  __shared__ __attribute__((aligned(16))) char k_lds[BKV * RS];
+  __shared__ __attribute__((aligned(16))) bf16_t vt_lds[DT * 32 * VT_STRIDE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int fr = lane & 31, hf = lane >> 5;
+  const int head = blockIdx.y;
+  const int seg_start = a.work[blockIdx.x * 4 + 0];
+  const int seg_end = a.work[blockIdx.x * 4 + 1];
+  const int q0 = a.work[blockIdx.x * 4 + 2];
+  const int nq = a.work[blockIdx.x * 4 + 3];
+  const int64_t hoff = (int64_t)head * D;
+
+  // Stage `nrows` rows starting at global row g0 (valid rows: < g0 + nvalid) of a [*, ld] tensor into an
+  // LDS tile with row stride RS, zero-filling invalid rows and pad chunks, optionally rotating.
+  auto stage_rows = [&](const bf16_t* src, char* dst, int g0, int nrows, int nvalid) {
+    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (ROPE) {
+      constexpr int HC = DC / 2;  // chunks per half
+      for (int i = tid; i < nrows * HC; i += NT) {
+        const int r = i / HC, jc = i - r * HC;
+        bf16x8_t o1 = zero, o2 = zero;
+        if (r < nvalid) {
+          const int64_t g = g0 + r;
+          const bf16_t* p = src + g * a.ld + hoff + jc * 8;
+          const bf16x8_t x1 = *(const bf16x8_t*)p;
+          const bf16x8_t x2 = *(const bf16x8_t*)(p + D / 2);
+          const float* cs = a.cos_sin + g * D + jc * 8;
+          const f32x4_t c0 = *(const f32x4_t*)cs, c1 = *(const f32x4_t*)(cs + 4);
+          const f32x4_t s0 = *(const f32x4_t*)(cs + D / 2), s1 = *(const f32x4_t*)(cs + D / 2 + 4);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float co = e < 4 ? c0[e] : c1[e - 4];
+            const float si = e < 4 ? s0[e] : s1[e - 4];
+            const float xa = bf2f(x1[e]), xb = bf2f(x2[e]);
+            o1[e] = f2bf(xa * co - xb * si);
+            o2[e] = f2bf(xa * si + xb * co);
+          }
+        }
+        *(bf16x8_t*)(dst + r * RS + jc * 16) = o1;
+        *(bf16x8_t*)(dst + r * RS + (jc + HC) * 16) = o2;
+      }
+    } else {
+      for (int i = tid; i < nrows * DKC; i += NT) {
+        const int r = i / DKC, c = i - r * DKC;
+        bf16x8_t x = zero;
+        if (r < nvalid && c < DC) x = *(const bf16x8_t*)(src + (int64_t)(g0 + r) * a.ld + hoff + c * 8);
+        *(bf16x8_t*)(dst + r * RS + c * 16) = x;
+      }
+    }
+    if (ROPE && DKC > DC) {
+      for (int i = tid; i < nrows * (DKC - DC); i += NT) {
+        const int r = i / (DKC - DC), c = DC + i % (DKC - DC);
+        *(bf16x8_t*)(dst + r * RS + c * 16) = zero;
+      }
+    }
+  };
+
+  // V tile -> V^T in LDS: thread takes a pair of keys and one 8-wide chunk of the head dim.
+  auto stage_v = [&](int g0, int nvalid) {
+    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    for (int i = tid; i < (BKV / 2) * DC; i += NT) {
+      const int kp = i % (BKV / 2), c = i / (BKV / 2);
+      const int r0 = 2 * kp;
+      bf16x8_t x0 = zero, x1 = zero;
+      if (r0 < nvalid) x0 = *(const bf16x8_t*)(a.v + (int64_t)(g0 + r0) * a.ld + hoff + c * 8);
+      if (r0 + 1 < nvalid) x1 = *(const bf16x8_t*)(a.v + (int64_t)(g0 + r0 + 1) * a.ld + hoff + c * 8);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        bf16x2_t pr;
+        pr[0] = x0[e];
+        pr[1] = x1[e];
+        *(bf16x2_t*)(vt_lds + (c * 8 + e) * VT_STRIDE + r0) = pr;
+      }
+    }
+  };
+
+  stage_rows(a.q, q_lds, q0, BQ, nq);
+  __syncthreads();
+  bf16x8_t qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8_t*)(q_lds + (wave * 32 + fr) * RS + (2 * ks + hf) * 16);
+
+  f32x16_t oacc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const bool wave_active = wave * 32 < nq;
+
+  const int seg_len = seg_end - seg_start;
+  for (int kv0 = 0; kv0 < seg_len; kv0 += BKV) {
+    const int nvalid = min(BKV, seg_len - kv0);
+    __syncthreads();  // previous tile fully consumed
+    stage_rows(a.k, k_lds, seg_start + kv0, BKV, nvalid);
+    stage_v(seg_start + kv0, nvalid);
+    __syncthreads();
+    if (!wave_active) continue;
+
+    f32x16_t sacc[2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[kt][r] = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8_t kf = *(const bf16x8_t*)(k_lds + (kt * 32 + fr) * RS + (2 * ks + hf) * 16);
+        sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kt], 0, 0, 0);
+      }
+    }
+    // mask keys past the segment end, running max
+    float mx = -INFINITY;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+        const float s = key < nvalid ? sacc[kt][r] : -INFINITY;
+        sacc[kt][r] = s;
+        mx = fmaxf(mx, s);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = exp2f((m_run - m_new) * a.scale_log2e);
+    const float mb = m_new * a.scale_log2e;
+    float psum = 0.f;
+    bf16x8_t pf[2][2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float pv = exp2f(sacc[kt][r] * a.scale_log2e - mb);
+        psum += pv;
+        pf[kt][r >> 3][r & 7] = f2bf(pv);
+      }
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+#pragma unroll
+    for (int t = 0; t < DT; ++t) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int kk = 0; kk < 2; ++kk) {
+          const bf16_t* vp = vt_lds + (t * 32 + fr) * VT_STRIDE + kt * 32 + 16 * kk + 4 * hf;
+          const bf16x4_t v0 = *(const bf16x4_t*)vp;
+          const bf16x4_t v1 = *(const bf16x4_t*)(vp + 8);
+          bf16x8_t vf;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            vf[e] = v0[e];
+            vf[4 + e] = v1[e];
+          }
+          oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][kk], oacc[t], 0, 0, 0);
+        }
+    }
+  }
+
+  // O^T[d][q] / l -> out[q][head*D + d]; lane owns query wave*32 + fr and 4 consecutive d per group.
+  const int qi = wave * 32 + fr;
+  if (qi < nq) {
+    const float inv = 1.0f / l_run;
+    bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d0 = t * 32 + 8 * g + 4 * hf;
+        if (d0 < D) {
+          bf16x4_t o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
+          *(bf16x4_t*)(orow + d0) = o;
+        }
+      }
+  }
+}
+
+template <int D>
+int launch_attn(const AttnArgs& a, int n_work, int heads, int block_q, bool rope, hipStream_t stream) {
+  const dim3 grid(n_work, heads);
+  if (block_q == 64) {
+    if (rope) {
+      if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_kernel<D, 2, true>), grid, dim3(128), 0, stream, a);
+      else return CS_ERR_UNSUPPORTED;
+    } else {
+      hipLaunchKernelGGL((attn_kernel<D, 2, false>), grid, dim3(128), 0, stream, a);
+    }
+  } else {
+    if (rope) {
+      if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_kernel<D, 4, true>), grid, dim3(256), 0, stream, a);
+      else return CS_ERR_UNSUPPORTED;
+    } else {
+      hipLaunchKernelGGL((attn_kernel<D, 4, false>), grid, dim3(256), 0, stream, a);
+    }
+  }
+  return cs_launch_status();
+}
+
+}  // namespace
+
+// Query rows per workgroup: 64 (2 waves) when no segment is longer than 64 rows (window attention),
+// else 128 (4 waves).
+extern "C" int cs_attn_block_q(int32_t max_seqlen) { return max_seqlen <= 64 ? 64 : 128; }
+
+extern "C" int cs_attn_work_host(const int32_t* cu_seqlens_host, int32_t n_seg, int32_t block_q,
+                                 int32_t* work_host, int32_t cap_items, int32_t* n_work) {
+  if (!cu_seqlens_host || n_seg < 0 || block_q <= 0 || !work_host || !n_work) return CS_ERR_INVALID_ARG;
+  int n = 0;
+  for (int s = 0; s < n_seg; ++s) {
+    const int b = cu_seqlens_host[s], e = cu_seqlens_host[s + 1];
+    if (e < b) return CS_ERR_INVALID_ARG;
+    for (int q = b; q < e; q += block_q) {
+      if (n >= cap_items) return CS_ERR_TOO_LARGE;
+      work_host[4 * n + 0] = b;
+      work_host[4 * n + 1] = e;
+      work_host[4 * n + 2] = q;
+      work_host[4 * n + 3] = e - q < block_q ? e - q : block_q;
+      ++n;
+    }
+  }
+  *n_work = n;
+  return CS_OK;
+}
+
+extern "C" int cs_attn_varlen(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
+                              const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
+                              const float* cos_sin, int32_t max_seqlen, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!q || !k || !v || !out || !work || n_work < 0 || heads <= 0 || heads > 65535 || head_dim <= 0 ||
+      max_seqlen <= 0)
+    return CS_ERR_INVALID_ARG;
+  if (ld % 8 || ldo % 4 || head_dim % 8) return CS_ERR_INVALID_ARG;
+  if (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)cos_sin) & 15) return CS_ERR_INVALID_ARG;
+  if ((uintptr_t)out & 7) return CS_ERR_INVALID_ARG;
+  if (n_work == 0) return CS_OK;
+  AttnArgs a;
+  a.q = (const bf16_t*)q;
+  a.k = (const bf16_t*)k;
+  a.v = (const bf16_t*)v;
+  a.ld = ld;
+  a.out = (bf16_t*)out;
+  a.ldo = ldo;
+  a.work = work;
+  a.cos_sin = cos_sin;
+  a.scale_log2e = scale * 1.4426950408889634f;
+  const int bq = cs_attn_block_q(max_seqlen);
+  const bool rope = cos_sin != nullptr;
+  switch (head_dim) {
+    case 64: return launch_attn<64>(a, n_work, heads, bq, rope, stream);
+    case 72: return launch_attn<72>(a, n_work, heads, bq, rope, stream);
+    case 80: return launch_attn<80>(a, n_work, heads, bq, rope, stream);
+    case 96: return launch_attn<96>(a, n_work, heads, bq, rope, stream);
+    default: return CS_ERR_UNSUPPORTED;
+  }
+}

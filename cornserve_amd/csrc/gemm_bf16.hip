@@ -1,0 +1,323 @@
+// bf16 MFMA GEMM for gfx950:  C[M,N] = epilogue( A[M,K] . W[N,K]^T )
+//
+// This is the F.linear of the Eric encoders (reference: eric/models/layers/linear.py:179-188 and
+// :537-554 at TP=1 are plain F.linear(x, W, b)).  Both operands are K-contiguous, which is the native
+// operand form of v_mfma_f32_32x32x16_bf16 (8 consecutive k per lane), so no transposes are needed.
+//
+// Work decomposition: one 512-thread workgroup (8 waves, 2 per SIMD) owns a BM x BN tile of C and
+// walks K in steps of 64.  Tiles are staged global -> registers -> LDS (XOR-swizzled 16-byte chunks,
+// conflict-free for both the 16 B writes and the MFMA fragment reads), double buffered so the global
+// loads of step k+1 are in flight while step k is on the matrix cores.  W is fed as the MFMA "A"
+// operand and the activations as "B", so that each lane ends up owning one row m of C and groups of 4
+// consecutive columns n: epilogues that pair adjacent columns (SwiGLU on interleaved gate|up) and
+// 8-byte packed stores fall out of that.
+//
+// Epilogues (all optional-bias, fp32 accumulate, rounding points follow the reference's bf16 steps):
+//   EPI_BIAS       y = bf16(acc + b)
+//   EPI_RESIDUAL   y = bf16( bf16(acc + b) + r )                     (qwen2_5_vl.py:175,177)
+//   EPI_SWIGLU     y[j] = bf16( bf16(silu(bf16(acc[2j]+b[2j]))) * bf16(acc[2j+1]+b[2j+1]) )
+//                                                                    (qwen2_5_vl.py:143-148)
+//   EPI_GELU_ERF   y = bf16(gelu_erf(bf16(acc + b)))                 (qwen2_5_vl.py:218-222)
+//   EPI_GELU_TANH  y = bf16(gelu_tanh(bf16(acc + b)))                (siglip.py:155-163)
+// plus an optional fp32 per-output-channel scale applied to acc (fp8-e4m3 weights, W_FP8 = true), an
+// optional gather of A rows (a_rows) and scatter of C rows (c_rows) used to fuse the window permutation
+// (qwen2_5_vl.py:438-440) and its inverse (:478-479) into the neighbouring GEMMs, and an optional second
+// residual-like addend indexed by (row % pos_period) for the SigLIP position embedding (siglip.py:100).
+#include "common.h"
+
+namespace {
+
+constexpr int BK = 64;           // K step (bf16 elements): 128 bytes per tile row = 8 chunks of 16 B
+constexpr int NTHREADS = 512;    // 8 waves
+constexpr int WAVES_M = 2;
+constexpr int WAVES_N = 4;
+
+CS_DEVICE int swz(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
+
+CS_DEVICE float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+CS_DEVICE float gelu_tanh(float x) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  float inner = k0 * (x + k1 * x * x * x);
+  return 0.5f * x * (1.0f + tanhf(inner));
+}
+CS_DEVICE float silu(float x) { return x / (1.0f + __expf(-x)); }
+
+// 16 fp8-e4m3 (OCP) values -> 16 bf16.  Conversion is exact: every e4m3 value is representable in bf16.
+CS_DEVICE void fp8x16_to_bf16(const i32x4_t& in, bf16x8_t& lo, bf16x8_t& hi) {
+  float f[16];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    auto p0 = __builtin_amdgcn_cvt_pk_f32_fp8(in[i], false);
+    auto p1 = __builtin_amdgcn_cvt_pk_f32_fp8(in[i], true);
+    f[4 * i + 0] = p0[0];
+    f[4 * i + 1] = p0[1];
+    f[4 * i + 2] = p1[0];
+    f[4 * i + 3] = p1[1];
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    lo[i] = (bf16_t)f[i];
+    hi[i] = (bf16_t)f[8 + i];
+  }
+}
+
+template <int BM, int BN, int EPI, bool W_FP8>
+__global__ __launch_bounds__(NTHREADS) void gemm_kernel(const CsGemmArgs p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  const bf16_t* const pA = (const bf16_t*)p.A;
+  const bf16_t* const pBias = (const bf16_t*)p.bias;
+  const bf16_t* const pRes = (const bf16_t*)p.residual;
+  const bf16_t* const pPos = (const bf16_t*)p.pos;
+  bf16_t* const pC = (bf16_t*)p.C;
+  constexpr int A_BYTES = BM * BK * 2;
+  constexpr int W_BYTES = BN * BK * 2;
+  constexpr int STAGE = A_BYTES + W_BYTES;
+  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
+  constexpr int MT = WTM / 32, NT = WTN / 32;
+  constexpr int A_ITERS = BM / 64;                    // 16 B chunks per thread per stage (A)
+  constexpr int W_ITERS = W_FP8 ? BN / 128 : BN / 64; // fp8: one 16 B load carries two bf16 chunks
+
+  // ---- tile coordinates: XCD-aware remap, then bands of 8 tile-rows walked column-major so the 32
+  //      workgroups resident on one XCD share 8 A panels and 4 W panels through that XCD's L2.
+  const int nb = gridDim.x;
+  int bid = blockIdx.x;
+  {
+    const int per = nb >> 3;
+    if (bid < per * 8) bid = (bid & 7) * per + (bid >> 3);
+  }
+  constexpr int GM = 8;
+  const int band_sz = GM * p.tiles_n;
+  const int band = bid / band_sz;
+  const int within = bid - band * band_sz;
+  const int rows_in_band = min(GM, p.tiles_m - band * GM);
+  const int tm = band * GM + within % rows_in_band;
+  const int tn = within / rows_in_band;
+  const int m0 = tm * BM, n0 = tn * BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
+
+  // ---- global -> LDS staging assignment: thread -> (row r0 + 64*i, chunk c)
+  const int ld_c = tid & 7;
+  const int ld_r = tid >> 3;
+  const bf16_t* a_ptr[A_ITERS];
+#pragma unroll
+  for (int i = 0; i < A_ITERS; ++i) {
+    int r = min(m0 + ld_r + 64 * i, p.M - 1);
+    if (p.a_rows) r = p.a_rows[r];
+    a_ptr[i] = pA + (int64_t)r * p.lda + ld_c * 8;
+  }
+  const char* w_ptr[W_ITERS];
+  int w_lr[W_ITERS], w_lc[W_ITERS];
+#pragma unroll
+  for (int i = 0; i < W_ITERS; ++i) {
+    if (W_FP8) {
+      // 64 fp8 per row = 4 chunks of 16 B; thread -> row tid/4 + 128*i, 16-element group tid%4
+      w_lr[i] = (tid >> 2) + 128 * i;
+      w_lc[i] = (tid & 3) * 2;
+      int r = min(n0 + w_lr[i], p.N - 1);
+      w_ptr[i] = (const char*)p.W + (int64_t)r * p.ldw + (tid & 3) * 16;
+    } else {
+      w_lr[i] = ld_r + 64 * i;
+      w_lc[i] = ld_c;
+      int r = min(n0 + w_lr[i], p.N - 1);
+      w_ptr[i] = (const char*)p.W + ((int64_t)r * p.ldw + ld_c * 8) * 2;
+    }
+  }
+
+  i32x4_t ga[A_ITERS], gw[W_ITERS];
+  const i32x4_t zero4 = {0, 0, 0, 0};
+
+  auto load_global = [&](int kt) {
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int i = 0; i < A_ITERS; ++i) {
+      ga[i] = (k0 + ld_c * 8 < p.K) ? *(const i32x4_t*)(a_ptr[i] + k0) : zero4;
+    }
+#pragma unroll
+    for (int i = 0; i < W_ITERS; ++i) {
+      if (W_FP8)
+        gw[i] = (k0 + (tid & 3) * 16 < p.K) ? *(const i32x4_t*)(w_ptr[i] + k0) : zero4;
+      else
+        gw[i] = (k0 + ld_c * 8 < p.K) ? *(const i32x4_t*)(w_ptr[i] + (int64_t)k0 * 2) : zero4;
+    }
+  };
+  auto store_lds = [&](int stage) {
+    char* As = smem + stage * STAGE;
+    char* Ws = As + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < A_ITERS; ++i) *(i32x4_t*)(As + swz(ld_r + 64 * i, ld_c)) = ga[i];
+#pragma unroll
+    for (int i = 0; i < W_ITERS; ++i) {
+      if (W_FP8) {
+        bf16x8_t lo, hi;
+        fp8x16_to_bf16(gw[i], lo, hi);
+        *(bf16x8_t*)(Ws + swz(w_lr[i], w_lc[i])) = lo;
+        *(bf16x8_t*)(Ws + swz(w_lr[i], w_lc[i] + 1)) = hi;
+      } else {
+        *(i32x4_t*)(Ws + swz(w_lr[i], w_lc[i])) = gw[i];
+      }
+    }
+  };
+
+  f32x16_t acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; ++i)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int frag_row = lane & 31;
+  const int frag_half = lane >> 5;
+
+  auto compute = [&](int stage) {
+    const char* As = smem + stage * STAGE;
+    const char* Ws = As + A_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      bf16x8_t wf[NT], xf[MT];
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        wf[j] = *(const bf16x8_t*)(Ws + swz(wn * WTN + j * 32 + frag_row, ks * 2 + frag_half));
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+        xf[i] = *(const bf16x8_t*)(As + swz(wm * WTM + i * 32 + frag_row, ks * 2 + frag_half));
+#pragma unroll
+      for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[j], xf[i], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  const int nk = (p.K + BK - 1) / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  for (int kt = 0; kt < nk; ++kt) {
+    const int cur = kt & 1;
+    if (kt + 1 < nk) load_global(kt + 1);
+    compute(cur);
+    if (kt + 1 < nk) store_lds(cur ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue.  acc[i][j][4g+q] = C[m][n], m = m0+wm*WTM+i*32+lane%32,
+  //      n = n0+wn*WTN+j*32+8g+4*(lane/32)+q.
+#pragma unroll
+  for (int i = 0; i < MT; ++i) {
+    const int m = m0 + wm * WTM + i * 32 + frag_row;
+    if (m >= p.M) continue;
+    const int64_t crow = p.c_rows ? (int64_t)p.c_rows[m] : (int64_t)m;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int n = n0 + wn * WTN + j * 32 + 8 * g + 4 * frag_half;
+        if (n >= p.N) continue;
+        float v[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = acc[i][j][4 * g + q];
+        if (p.w_scale) {
+          const f32x4_t s = *(const f32x4_t*)(p.w_scale + n);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] *= s[q];
+        }
+        if (p.bias) {
+          const bf16x4_t b = *(const bf16x4_t*)(pBias + n);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] += bf2f(b[q]);
+        }
+        if (EPI == CS_EPI_SWIGLU) {
+          const float gate0 = rbf(silu(rbf(v[0]))), up0 = rbf(v[1]);
+          const float gate1 = rbf(silu(rbf(v[2]))), up1 = rbf(v[3]);
+          bf16x2_t o;
+          o[0] = f2bf(gate0 * up0);
+          o[1] = f2bf(gate1 * up1);
+          *(bf16x2_t*)(pC + crow * p.ldc + (n >> 1)) = o;
+        } else {
+          if (EPI == CS_EPI_GELU_ERF) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = gelu_erf(rbf(v[q]));
+          } else if (EPI == CS_EPI_GELU_TANH) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = gelu_tanh(rbf(v[q]));
+          } else if (EPI == CS_EPI_RESIDUAL) {
+            const bf16x4_t r = *(const bf16x4_t*)(pRes + (int64_t)m * p.ldr + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = rbf(v[q]) + bf2f(r[q]);
+          }
+          if (p.pos) {
+            const bf16x4_t r = *(const bf16x4_t*)(pPos + (int64_t)(m % p.pos_period) * p.ldpos + n);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = rbf(v[q]) + bf2f(r[q]);
+          }
+          bf16x4_t o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) o[q] = f2bf(v[q]);
+          *(bf16x4_t*)(pC + crow * p.ldc + n) = o;
+        }
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int EPI, bool W_FP8>
+int launch(const CsGemmArgs& a, hipStream_t stream) {
+  CsGemmArgs p = a;
+  p.tiles_m = (p.M + BM - 1) / BM;
+  p.tiles_n = (p.N + BN - 1) / BN;
+  constexpr int lds = 2 * (BM + BN) * BK * 2;
+  static bool attr_set = false;
+  auto kern = gemm_kernel<BM, BN, EPI, W_FP8>;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return CS_ERR_LAUNCH;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(p.tiles_m * p.tiles_n), dim3(NTHREADS), lds, stream, p);
+  return cs_launch_status();
+}
+
+template <int BM, int BN, bool W_FP8>
+int dispatch_epi(const CsGemmArgs& a, hipStream_t s) {
+  switch (a.epilogue) {
+    case CS_EPI_BIAS: return launch<BM, BN, CS_EPI_BIAS, W_FP8>(a, s);
+    case CS_EPI_RESIDUAL: return launch<BM, BN, CS_EPI_RESIDUAL, W_FP8>(a, s);
+    case CS_EPI_SWIGLU: return launch<BM, BN, CS_EPI_SWIGLU, W_FP8>(a, s);
+    case CS_EPI_GELU_ERF: return launch<BM, BN, CS_EPI_GELU_ERF, W_FP8>(a, s);
+    case CS_EPI_GELU_TANH: return launch<BM, BN, CS_EPI_GELU_TANH, W_FP8>(a, s);
+    default: return CS_ERR_INVALID_ARG;
+  }
+}
+
+}  // namespace
+
+extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!args) return CS_ERR_INVALID_ARG;
+  const CsGemmArgs& a = *args;
+  if (a.M < 0 || a.N <= 0 || a.K <= 0) return CS_ERR_INVALID_ARG;
+  if (a.M == 0 && a.W) return CS_OK;  // an empty batch may come with null activation buffers
+  if (!a.A || !a.W || !a.C) return CS_ERR_INVALID_ARG;
+  // 16-byte vector loads along K and 8-byte packed stores along N.
+  if (a.K % 8 || a.lda % 8 || a.N % 4 || a.ldc % 2) return CS_ERR_INVALID_ARG;
+  if (a.w_fp8 ? (a.ldw % 16 || a.K % 16 || !a.w_scale) : (a.ldw % 8)) return CS_ERR_INVALID_ARG;
+  if (a.epilogue == CS_EPI_RESIDUAL && (!a.residual || a.ldr % 4)) return CS_ERR_INVALID_ARG;
+  if (a.epilogue != CS_EPI_SWIGLU && a.ldc % 4) return CS_ERR_INVALID_ARG;
+  if (a.pos && (a.pos_period <= 0 || a.ldpos % 4 || a.epilogue == CS_EPI_SWIGLU)) return CS_ERR_INVALID_ARG;
+  if (((uintptr_t)a.A | (uintptr_t)a.W) & 15) return CS_ERR_INVALID_ARG;
+  if (((uintptr_t)a.C | (uintptr_t)a.bias | (uintptr_t)a.residual | (uintptr_t)a.pos) & 7) return CS_ERR_INVALID_ARG;
+  if ((uintptr_t)a.w_scale & 15) return CS_ERR_INVALID_ARG;
+
+  // Tile choice: 256x256 when that fills the chip's 256 CUs reasonably, else smaller tiles for more workgroups.
+  const int64_t t256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+  const bool small = t256 < 192;
+  if (a.w_fp8) {
+    return small ? dispatch_epi<128, 128, true>(a, stream) : dispatch_epi<256, 256, true>(a, stream);
+  }
+  return small ? dispatch_epi<128, 128, false>(a, stream) : dispatch_epi<256, 256, false>(a, stream);
+}

@@ -1,0 +1,228 @@
+// Integer index routines, row gather and rotary embedding of the Qwen2.5-VL vision encoder (gfx950).
+//
+// The reference builds the window permutation with a Python loop per image, boolean masks and a
+// .tolist() host sync (eric/models/qwen2_5_vl.py:357-386), the position ids with another per-image
+// loop (:325-355), and then gathers hidden states and the rotary table (:438-443).  Here the
+// per-item scalars are computed once on the host (a few integers per image), and one device kernel
+// fills every per-patch array from a closed form, one thread per patch:
+//
+//   a merged unit (frame f, row r, col c) of an item with merged grid gh x gw sits in window
+//   (wr, wc) = (r / win, c / win) of height rh = min(win, gh - wr*win) and width cw = min(win, gw - wc*win);
+//   its position in window order is
+//       base + f*gh*gw + wr*win*gw + rh*wc*win + (r - wr*win)*cw + (c - wc*win)
+//   because the windows of one frame are emitted row-major and each window row-major inside
+//   (permute(0,1,3,2,4) then boolean compaction, :372-379).  Empty pad windows contribute nothing.
+#include <math.h>
+
+#include "common.h"
+
+namespace {
+
+struct ItemMeta {  // matches the int32[8] record documented in cornserve_amd.h
+  int t, gh, gw, unit_base, nwr, nwc, patch_base, reserved;
+};
+
+__global__ __launch_bounds__(256) void vit_index_kernel(const ItemMeta* __restrict__ meta, int merge, int win,
+                                                        const float* __restrict__ inv_freq, int rot_dim,
+                                                        int32_t* __restrict__ window_index,
+                                                        int32_t* __restrict__ reverse_index,
+                                                        int32_t* __restrict__ src_rows,
+                                                        int32_t* __restrict__ pos_ids,
+                                                        float* __restrict__ cos_sin) {
+  const ItemMeta it = meta[blockIdx.y];
+  const int mm = merge * merge;
+  const int frame_units = it.gh * it.gw;
+  const int n_patches = it.t * frame_units * mm;
+  const int pl = blockIdx.x * blockDim.x + threadIdx.x;  // patch within the item, ORIGINAL order
+  if (pl >= n_patches) return;
+  const int ul = pl / mm, s = pl - ul * mm;
+  const int f = ul / frame_units;
+  const int rem = ul - f * frame_units;
+  const int r = rem / it.gw, c = rem - r * it.gw;
+  const int wr = r / win, wc = c / win;
+  const int rh = min(win, it.gh - wr * win);
+  const int cw = min(win, it.gw - wc * win);
+  const int pos = wr * win * it.gw + rh * wc * win + (r - wr * win) * cw + (c - wc * win);
+  const int u = it.unit_base + ul;                     // original unit id
+  const int up = it.unit_base + f * frame_units + pos;  // window-order unit id
+  if (s == 0) {
+    if (window_index) window_index[up] = u;
+    if (reverse_index) reverse_index[u] = up;
+  }
+  const int h = r * merge + s / merge;
+  const int w = c * merge + s % merge;
+  const int64_t row_orig = (int64_t)u * mm + s;
+  const int64_t row_win = (int64_t)up * mm + s;
+  if (src_rows) src_rows[row_win] = (int32_t)row_orig;
+  if (pos_ids) {
+    pos_ids[row_orig * 2 + 0] = h;
+    pos_ids[row_orig * 2 + 1] = w;
+  }
+  if (cos_sin) {
+    const int half = rot_dim / 2;
+    float* out = cos_sin + row_win * (2 * rot_dim);
+    for (int j = 0; j < half; ++j) {
+      const float fr = inv_freq[j];
+      const float ah = (float)h * fr, aw = (float)w * fr;
+      out[j] = cosf(ah);
+      out[half + j] = cosf(aw);
+      out[rot_dim + j] = sinf(ah);
+      out[rot_dim + half + j] = sinf(aw);
+    }
+  }
+}
+
+template <typename V>
+__global__ __launch_bounds__(256) void row_gather_kernel(const char* __restrict__ in, int64_t in_stride,
+                                                         const int32_t* __restrict__ rows,
+                                                         char* __restrict__ out, int64_t out_stride, int n_rows,
+                                                         int n_vec) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= n_rows) return;
+  const V* src = (const V*)(in + (int64_t)rows[row] * in_stride);
+  V* dst = (V*)(out + (int64_t)row * out_stride);
+  for (int i = lane; i < n_vec; i += 64) dst[i] = src[i];
+}
+
+// In-place rotary on the q and k column blocks of a packed [L, 3*heads*d] buffer.  One thread owns
+// 8 consecutive j of one (row, q|k, head): it reads x[j..j+8) and x[d/2+j..), rotates in fp32 and
+// writes both halves back with a single bf16 rounding.
+__global__ __launch_bounds__(256) void rope_qk_kernel(bf16_t* __restrict__ qkv, int64_t ld,
+                                                      const float* __restrict__ cos_sin, int L, int heads, int d) {
+  const int half = d >> 1;
+  const int cpr = half >> 3;  // chunks per (row, head, tensor)
+  const int64_t total = (int64_t)L * 2 * heads * cpr;
+  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const int jc = idx % cpr;
+  idx /= cpr;
+  const int h = idx % heads;
+  idx /= heads;
+  const int which = idx % 2;
+  const int64_t l = idx / 2;
+  bf16_t* base = qkv + l * ld + (int64_t)which * heads * d + h * d + jc * 8;
+  const float* cs = cos_sin + l * d + jc * 8;
+  const bf16x8_t x1 = *(const bf16x8_t*)base;
+  const bf16x8_t x2 = *(const bf16x8_t*)(base + half);
+  const f32x4_t c0 = *(const f32x4_t*)cs, c1 = *(const f32x4_t*)(cs + 4);
+  const f32x4_t s0 = *(const f32x4_t*)(cs + half), s1 = *(const f32x4_t*)(cs + half + 4);
+  bf16x8_t o1, o2;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const float co = e < 4 ? c0[e] : c1[e - 4];
+    const float si = e < 4 ? s0[e] : s1[e - 4];
+    const float a = bf2f(x1[e]), b = bf2f(x2[e]);
+    o1[e] = f2bf(a * co - b * si);
+    o2[e] = f2bf(a * si + b * co);
+  }
+  *(bf16x8_t*)base = o1;
+  *(bf16x8_t*)(base + half) = o2;
+}
+
+}  // namespace
+
+extern "C" int cs_abi_version(void) { return CS_ABI_VERSION; }
+
+extern "C" int cs_vit_seqlens_host(const int64_t* grid_thw_host, int32_t n_items, int32_t merge, int32_t win,
+                                   int32_t* cu_window_host, int32_t cap_window, int32_t* n_cu_window,
+                                   int32_t* cu_full_host, int32_t cap_full, int32_t* n_cu_full,
+                                   int32_t* item_meta_host, int64_t* total_patches) {
+  if (!grid_thw_host || n_items < 0 || merge <= 0 || win <= 0 || !cu_window_host || !cu_full_host ||
+      !n_cu_window || !n_cu_full || !item_meta_host || !total_patches || cap_window < 1 || cap_full < 1)
+    return CS_ERR_INVALID_ARG;
+  const int64_t mm = (int64_t)merge * merge;
+  int nw = 0, nf = 0;
+  cu_window_host[nw++] = 0;
+  cu_full_host[nf++] = 0;
+  int64_t unit_base = 0, cu_w = 0, cu_f = 0;
+  for (int i = 0; i < n_items; ++i) {
+    const int64_t t = grid_thw_host[3 * i], h = grid_thw_host[3 * i + 1], w = grid_thw_host[3 * i + 2];
+    if (t <= 0 || h <= 0 || w <= 0 || h % merge || w % merge) return CS_ERR_INVALID_ARG;
+    const int64_t gh = h / merge, gw = w / merge;
+    if ((unit_base + t * gh * gw) * mm > INT32_MAX) return CS_ERR_TOO_LARGE;
+    // The reference pads by win - n % win, i.e. a full extra (empty) window when n divides evenly
+    // (qwen2_5_vl.py:367-370); empty windows repeat the running total and unique_consecutive (:436)
+    // drops the repeats.  Walk the padded window grid literally and drop repeats the same way.
+    const int64_t nwh = (gh + (win - gh % win)) / win, nww = (gw + (win - gw % win)) / win;
+    for (int64_t f = 0; f < t; ++f) {
+      for (int64_t wr = 0; wr < nwh; ++wr) {
+        const int64_t rh = gh - wr * win < 0 ? 0 : (gh - wr * win < win ? gh - wr * win : win);
+        for (int64_t wc = 0; wc < nww; ++wc) {
+          const int64_t cw = gw - wc * win < 0 ? 0 : (gw - wc * win < win ? gw - wc * win : win);
+          cu_w += rh * cw * mm;
+          if ((int64_t)cu_window_host[nw - 1] != cu_w) {
+            if (nw >= cap_window) return CS_ERR_TOO_LARGE;
+            cu_window_host[nw++] = (int32_t)cu_w;
+          }
+        }
+      }
+      // one full-attention segment per frame (qwen2_5_vl.py:445-448)
+      cu_f += h * w;
+      if (nf >= cap_full) return CS_ERR_TOO_LARGE;
+      cu_full_host[nf++] = (int32_t)cu_f;
+    }
+    int32_t* m = item_meta_host + 8 * i;
+    m[0] = (int32_t)t;
+    m[1] = (int32_t)gh;
+    m[2] = (int32_t)gw;
+    m[3] = (int32_t)unit_base;
+    m[4] = (int32_t)((gh + win - 1) / win);
+    m[5] = (int32_t)((gw + win - 1) / win);
+    m[6] = (int32_t)(unit_base * mm);
+    m[7] = 0;
+    unit_base += t * gh * gw;
+  }
+  *n_cu_window = nw;
+  *n_cu_full = nf;
+  *total_patches = unit_base * mm;
+  return CS_OK;
+}
+
+extern "C" int cs_vit_index(const int32_t* item_meta, int32_t n_items, int32_t max_units_per_item,
+                            int32_t merge, int32_t win, const float* inv_freq, int32_t rot_dim,
+                            int32_t* window_index, int32_t* reverse_index, int32_t* src_rows, int32_t* pos_ids,
+                            float* cos_sin, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!item_meta || n_items < 0 || max_units_per_item < 0 || merge <= 0 || win <= 0) return CS_ERR_INVALID_ARG;
+  if (cos_sin && (!inv_freq || rot_dim <= 0 || rot_dim % 2)) return CS_ERR_INVALID_ARG;
+  if (n_items == 0 || max_units_per_item == 0) return CS_OK;
+  if (n_items > 65535) return CS_ERR_TOO_LARGE;
+  const int64_t max_patches = (int64_t)max_units_per_item * merge * merge;
+  const dim3 grid((unsigned)((max_patches + 255) / 256), n_items), block(256);
+  hipLaunchKernelGGL(vit_index_kernel, grid, block, 0, stream, (const ItemMeta*)item_meta, merge, win, inv_freq,
+                     rot_dim, window_index, reverse_index, src_rows, pos_ids, cos_sin);
+  return cs_launch_status();
+}
+
+extern "C" int cs_row_gather(const void* in, int64_t in_stride_bytes, const int32_t* rows, void* out,
+                             int64_t out_stride_bytes, int32_t n_rows, int32_t row_bytes, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (n_rows < 0 || row_bytes <= 0 || row_bytes % 4 || in_stride_bytes % 4 || out_stride_bytes % 4)
+    return CS_ERR_INVALID_ARG;
+  if (n_rows == 0) return CS_OK;  // an empty gather may come with null buffers
+  if (!in || !rows || !out) return CS_ERR_INVALID_ARG;
+  const dim3 grid((n_rows + 3) / 4), block(256);
+  const bool v16 = !(row_bytes % 16) && !(in_stride_bytes % 16) && !(out_stride_bytes % 16) &&
+                   !(((uintptr_t)in | (uintptr_t)out) & 15);
+  if (v16)
+    hipLaunchKernelGGL(row_gather_kernel<i32x4_t>, grid, block, 0, stream, (const char*)in, in_stride_bytes, rows,
+                       (char*)out, out_stride_bytes, n_rows, row_bytes / 16);
+  else
+    hipLaunchKernelGGL(row_gather_kernel<int>, grid, block, 0, stream, (const char*)in, in_stride_bytes, rows,
+                       (char*)out, out_stride_bytes, n_rows, row_bytes / 4);
+  return cs_launch_status();
+}
+
+extern "C" int cs_rope_qk(void* qkv, int64_t ld, const float* cos_sin, int32_t L, int32_t heads, int32_t head_dim,
+                          void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!qkv || !cos_sin || L < 0 || heads <= 0 || head_dim <= 0 || head_dim % 16 || ld % 8 ||
+      ld < (int64_t)3 * heads * head_dim || (((uintptr_t)qkv | (uintptr_t)cos_sin) & 15))
+    return CS_ERR_INVALID_ARG;
+  if (L == 0) return CS_OK;
+  const int64_t total = (int64_t)L * 2 * heads * (head_dim / 16);
+  hipLaunchKernelGGL(rope_qk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (bf16_t*)qkv, ld,
+                     cos_sin, L, heads, head_dim);
+  return cs_launch_status();
+}

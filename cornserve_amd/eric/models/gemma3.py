@@ -1,0 +1,278 @@
+"""Gemma-3 vision encoder (SigLIP tower + multimodal projector adapters) on hand-written gfx950 kernels.
+
+Drop-in for `Gemma3VisionEncoder` (reference: eric/models/gemma3.py:58-136) with the SigLIP tower of
+eric/models/layers/siglip.py.  Parameter names follow the checkpoint (`vision_tower.vision_model....`,
+separate q/k/v projections, which the reference fuses at load time, eric/models/layers/linear.py:339-371);
+the adapter container and its error behaviour follow eric/models/base.py:57-90.
+
+Forward = one fixed sequence of C-ABI launches:
+
+    strided patch gather -> patch-embed GEMM (+bias, +learned position embedding)  siglip.py:91-101
+    per layer: LayerNorm -> fused QKV GEMM -> full MFMA attention (d=72) -> out GEMM(+residual)
+               LayerNorm -> fc1 GEMM(+GELU-tanh) -> fc2 GEMM(+residual)            siglip.py:166-189
+    post LayerNorm                                                                 siglip.py:275-279
+    AvgPool(4x4)+GemmaRMSNorm -> projection GEMM                                   gemma3.py:33-49
+"""
+
+from __future__ import annotations
+
+from collections.abc import Callable
+from typing import Any
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from cornserve_amd import ops
+from cornserve_amd.eric.api import Modality
+from cornserve_amd.eric.models.base import BaseAdapterModule, BaseModalityProcessor, EricModel
+from cornserve_amd.eric.models.qwen2_5_vl import _Linear, _round_up
+
+
+class _LN(nn.Module):
+    def __init__(self, dim: int) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(dim), requires_grad=False)
+
+
+class _Conv(nn.Module):
+    def __init__(self, cin: int, cout: int, k: int) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(cout, cin, k, k), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(cout), requires_grad=False)
+
+
+class _Embedding(nn.Module):
+    def __init__(self, n: int, dim: int) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(n, dim), requires_grad=False)
+
+
+class _Embeddings(nn.Module):
+    def __init__(self, cfg: Any) -> None:
+        super().__init__()
+        self.patch_embedding = _Conv(cfg.num_channels, cfg.hidden_size, cfg.patch_size)
+        self.position_embedding = _Embedding((cfg.image_size // cfg.patch_size) ** 2, cfg.hidden_size)
+
+
+class _SelfAttn(nn.Module):
+    def __init__(self, dim: int) -> None:
+        super().__init__()
+        self.q_proj = _Linear(dim, dim)
+        self.k_proj = _Linear(dim, dim)
+        self.v_proj = _Linear(dim, dim)
+        self.out_proj = _Linear(dim, dim)
+
+
+class _SiglipMLP(nn.Module):
+    def __init__(self, dim: int, inter: int) -> None:
+        super().__init__()
+        self.fc1 = _Linear(dim, inter)
+        self.fc2 = _Linear(inter, dim)
+
+
+class _EncoderLayer(nn.Module):
+    def __init__(self, dim: int, inter: int) -> None:
+        super().__init__()
+        self.self_attn = _SelfAttn(dim)
+        self.layer_norm1 = _LN(dim)
+        self.mlp = _SiglipMLP(dim, inter)
+        self.layer_norm2 = _LN(dim)
+
+
+class _Encoder(nn.Module):
+    def __init__(self, cfg: Any) -> None:
+        super().__init__()
+        self.layers = nn.ModuleList(
+            [_EncoderLayer(cfg.hidden_size, cfg.intermediate_size) for _ in range(cfg.num_hidden_layers)]
+        )
+
+
+class SiglipVisionTransformer(nn.Module):
+    def __init__(self, cfg: Any) -> None:
+        super().__init__()
+        self.embeddings = _Embeddings(cfg)
+        self.encoder = _Encoder(cfg)
+        self.post_layernorm = _LN(cfg.hidden_size)
+
+
+class SiglipVisionModel(nn.Module):
+    def __init__(self, cfg: Any) -> None:
+        super().__init__()
+        self.vision_model = SiglipVisionTransformer(cfg)
+
+
+class Gemma3MultiModalProjector(nn.Module):
+    """Adapter: AvgPool2d -> GemmaRMSNorm -> projection (reference: gemma3.py:18-49)."""
+
+    def __init__(self, config: Any) -> None:
+        super().__init__()
+        vc = config.vision_config
+        self.mm_input_projection_weight = nn.Parameter(
+            torch.zeros(vc.hidden_size, config.text_config.hidden_size), requires_grad=False
+        )
+        self.mm_soft_emb_norm = nn.Module()
+        self.mm_soft_emb_norm.weight = nn.Parameter(torch.zeros(vc.hidden_size), requires_grad=False)
+        self.eps = vc.layer_norm_eps
+        self.patches_per_image = int(vc.image_size // vc.patch_size)
+        self.tokens_per_side = int(config.mm_tokens_per_image**0.5)
+        self.kernel_size = self.patches_per_image // self.tokens_per_side
+        self._wt: torch.Tensor | None = None
+        self.register_load_state_dict_post_hook(lambda module, incompatible: setattr(module, "_wt", None))
+
+    def _apply(self, fn, recurse=True):
+        self._wt = None
+        return super()._apply(fn, recurse)
+
+    def forward(self, vision_outputs: torch.Tensor) -> torch.Tensor:
+        if self._wt is None:  # GEMM wants the weight as [N=T, K=H]
+            self._wt = self.mm_input_projection_weight.t().contiguous()
+        B = vision_outputs.shape[0]
+        normed = ops.avgpool_gemma_rmsnorm(
+            vision_outputs, self.mm_soft_emb_norm.weight, self.patches_per_image, self.kernel_size, self.eps
+        )
+        out = ops.gemm(normed.view(-1, normed.shape[-1]), self._wt, None)
+        return out.view(B, -1, out.shape[-1])
+
+
+class Gemma3MultiModalProjectorAdapter(BaseAdapterModule):
+    def __init__(self) -> None:
+        super().__init__(adapter_cls=Gemma3MultiModalProjector)
+
+
+class Gemma3VisionEncoder(EricModel):
+    def __init__(self, config: Any) -> None:
+        super().__init__()
+        self.config = config
+        self.vision_tower = SiglipVisionModel(config.vision_config)
+        self.multi_modal_projector = Gemma3MultiModalProjectorAdapter()
+        self._packed: dict | None = None
+        self.register_load_state_dict_post_hook(lambda module, incompatible: setattr(module, "_packed", None))
+
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.vision_tower.vision_model.embeddings.patch_embedding.weight.dtype
+
+    @property
+    def device(self) -> torch.device:
+        return self.vision_tower.vision_model.embeddings.patch_embedding.weight.device
+
+    @property
+    def chunk_shape(self) -> tuple[int, ...]:
+        # Same fixed chunking as the reference (gemma3.py:76-88): 256 divides 2560, 3840 and 5376.
+        return (1, self.config.mm_tokens_per_image, 256)
+
+    def _apply(self, fn, recurse=True):
+        self._packed = None
+        out = super()._apply(fn, recurse)
+        for adapter in self.multi_modal_projector.adapters.values():  # adapters sit outside _modules
+            adapter._apply(fn)
+        return out
+
+    @torch.no_grad()
+    def _pack(self) -> dict:
+        vm = self.vision_tower.vision_model
+        vc = self.config.vision_config
+        H = vc.hidden_size
+        kraw = vc.num_channels * vc.patch_size * vc.patch_size
+        kp = _round_up(kraw, 16)
+        pe_w = torch.zeros((H, kp), dtype=self.dtype, device=self.device)
+        pe_w[:, :kraw] = vm.embeddings.patch_embedding.weight.reshape(H, kraw)
+        layers = []
+        for lyr in vm.encoder.layers:
+            a = lyr.self_attn
+            layers.append(
+                {
+                    "ln1": (lyr.layer_norm1.weight, lyr.layer_norm1.bias),
+                    "ln2": (lyr.layer_norm2.weight, lyr.layer_norm2.bias),
+                    "qkv_w": torch.cat([a.q_proj.weight, a.k_proj.weight, a.v_proj.weight], dim=0).contiguous(),
+                    "qkv_b": torch.cat([a.q_proj.bias, a.k_proj.bias, a.v_proj.bias], dim=0).contiguous(),
+                    "out": (a.out_proj.weight, a.out_proj.bias),
+                    "fc1": (lyr.mlp.fc1.weight, lyr.mlp.fc1.bias),
+                    "fc2": (lyr.mlp.fc2.weight, lyr.mlp.fc2.bias),
+                }
+            )
+        return {"pe_w": pe_w, "pe_b": vm.embeddings.patch_embedding.bias, "kp": kp,
+                "pos": vm.embeddings.position_embedding.weight, "layers": layers,
+                "post": (vm.post_layernorm.weight, vm.post_layernorm.bias)}
+
+    def _ensure_packed(self) -> dict:
+        if self._packed is None:
+            if self.dtype != torch.bfloat16 or self.device.type != "cuda":
+                raise RuntimeError(
+                    "the gfx950 kernels need the model in bfloat16 on a GPU "
+                    f"(got {self.dtype} on {self.device}); there is no CPU path"
+                )
+            self._packed = self._pack()
+        return self._packed
+
+    def vision_tower_forward(self, pixel_values: torch.Tensor) -> torch.Tensor:
+        """pixel_values: bf16 [B,3,S,S] on the device -> [B, tokens, H] after post-layernorm."""
+        pk = self._ensure_packed()
+        vc = self.config.vision_config
+        H, nh = vc.hidden_size, vc.num_attention_heads
+        d = H // nh
+        B = pixel_values.shape[0]
+        tokens = (vc.image_size // vc.patch_size) ** 2
+        M = B * tokens
+        patches = ops.patchify_nchw(pixel_values.contiguous(), vc.patch_size, pk["kp"])
+        x = ops.gemm(patches, pk["pe_w"], pk["pe_b"], pos=pk["pos"])
+        plan = ops.attn_plan(np.arange(0, M + 1, tokens, dtype=np.int32), x.device)
+        n = torch.empty_like(x)
+        qkv = torch.empty((M, 3 * H), dtype=torch.bfloat16, device=x.device)
+        att = torch.empty((M, H), dtype=torch.bfloat16, device=x.device)
+        hmid = torch.empty((M, vc.intermediate_size), dtype=torch.bfloat16, device=x.device)
+        eps = vc.layer_norm_eps
+        act = getattr(vc, "hidden_act", "gelu_pytorch_tanh")
+        if act == "gelu_pytorch_tanh":
+            epi = ops.EPI_GELU_TANH
+        elif act == "gelu":
+            epi = ops.EPI_GELU_ERF
+        else:
+            raise NotImplementedError(f"Activation function {act!r} is not implemented.")
+        for lyr in pk["layers"]:
+            ops.layernorm(x, *lyr["ln1"], eps, out=n)
+            ops.gemm(n, lyr["qkv_w"], lyr["qkv_b"], out=qkv)
+            ops.attn_varlen(qkv[:, :H], qkv[:, H : 2 * H], qkv[:, 2 * H :], plan, nh, d, d**-0.5, out=att)
+            ops.gemm(att, *lyr["out"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+            ops.layernorm(x, *lyr["ln2"], eps, out=n)
+            ops.gemm(n, *lyr["fc1"], epilogue=epi, out=hmid)
+            ops.gemm(hmid, *lyr["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+        ops.layernorm(x, *pk["post"], eps, out=n)
+        return n.view(B, tokens, H)
+
+    @torch.inference_mode()
+    def forward(self, modality: Modality, adapter_name: str, batch: dict[str, list[torch.Tensor]]) -> list[torch.Tensor]:
+        """`pixel_values`: each [num_patches, 3, S, S]; `num_crops`: each [1] (reference: gemma3.py:90-136)."""
+        if modality != Modality.IMAGE:
+            raise ValueError(f"Unsupported modality: {modality}")
+        if adapter_name is None:
+            raise ValueError("Adapter name must be provided for Gemma 3 vision encoder.")
+        size = self.config.vision_config.image_size
+        assert len(batch["pixel_values"]) == len(batch["num_crops"])
+        for pixels in batch["pixel_values"]:
+            assert pixels.ndim == 4
+            assert pixels.shape[1] == 3
+            assert pixels.shape[2] == pixels.shape[3] == size
+        pixel_values = torch.cat(batch["pixel_values"]).to(device=self.device, dtype=self.dtype)
+        num_patches = torch.cat([c.reshape(-1) for c in batch["num_crops"]]).cpu() + 1
+        feats = self.vision_tower_forward(pixel_values)
+        embeds = self.multi_modal_projector(adapter_name, feats)
+        return [e.flatten(0, 1) for e in embeds.split(num_patches.tolist())]
+
+
+class ModalityProcessor(BaseModalityProcessor):
+    """Gemma 3 modality processor (reference: gemma3.py:139-156); needs the model files locally."""
+
+    def __init__(self, model_id: str) -> None:
+        super().__init__(model_id=model_id)
+        from transformers import AutoProcessor  # deferred
+
+        self.image_processor = AutoProcessor.from_pretrained(model_id).image_processor
+
+    def get_image_processor(self) -> Callable | None:
+        def processor(image) -> dict[str, torch.Tensor]:
+            return self.image_processor(images=[image], return_tensors="pt").data
+
+        return processor

@@ -1,0 +1,326 @@
+"""Qwen2.5-VL vision transformer on hand-written gfx950 kernels.
+
+Drop-in for `Qwen2_5_VisionTransformer` (reference: eric/models/qwen2_5_vl.py:262-485): same constructor
+argument (the HF config, of which only `vision_config` is read), same parameter names as the checkpoint
+after `visual.` is stripped, same `forward(modality, adapter_name, batch)` contract and output list.
+
+What differs is everything underneath.  The forward pass is a fixed sequence of C-ABI kernel launches
+on torch's current stream:
+
+    patch-embed GEMM (window permutation fused as a row gather of A)        :424,:438-440
+    per block:  RMSNorm -> QKV GEMM(+bias) -> varlen MFMA attention with rotary fused into the q/k load
+                -> proj GEMM(+bias,+residual) -> RMSNorm -> gate|up GEMM(+bias, SiLU*mul)
+                -> down GEMM(+bias,+residual)                                :168-178
+    merger:     RMSNorm -> GEMM(+bias, GELU) -> GEMM(+bias) with the inverse window permutation fused
+                as a row scatter of C                                        :225-233,:478-479
+
+Weights are repacked once after loading: gate and up rows are interleaved (so SiLU(gate)*up is a
+lane-local epilogue), the MLP intermediate size is zero-padded to a multiple of 64 so K loops have no
+tail, and optionally every linear weight is quantised to fp8-e4m3 with per-output-channel scales.
+"""
+
+from __future__ import annotations
+
+from collections.abc import Callable
+from typing import Any
+
+import numpy as np
+import torch
+import torch.nn as nn
+
+from cornserve_amd import ops
+from cornserve_amd.eric.api import Modality
+from cornserve_amd.eric.models.base import BaseModalityProcessor, EricModel
+
+
+class _Linear(nn.Module):
+    """Parameter holder with nn.Linear's names; arithmetic happens in the fused kernels."""
+
+    def __init__(self, in_features: int, out_features: int, bias: bool = True) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(out_features, in_features), requires_grad=False)
+        self.bias = nn.Parameter(torch.empty(out_features), requires_grad=False) if bias else None
+
+
+class _Scale(nn.Module):
+    def __init__(self, dim: int) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(dim), requires_grad=False)
+
+
+class _PatchProj(nn.Module):
+    def __init__(self, in_channels: int, hidden: int, t: int, p: int) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(hidden, in_channels, t, p, p), requires_grad=False)
+
+
+class _PatchEmbed(nn.Module):
+    def __init__(self, in_channels: int, hidden: int, t: int, p: int) -> None:
+        super().__init__()
+        self.proj = _PatchProj(in_channels, hidden, t, p)
+
+
+class _Attn(nn.Module):
+    def __init__(self, dim: int) -> None:
+        super().__init__()
+        self.qkv = _Linear(dim, 3 * dim)
+        self.proj = _Linear(dim, dim)
+
+
+class _MLP(nn.Module):
+    def __init__(self, dim: int, inter: int) -> None:
+        super().__init__()
+        self.gate_proj = _Linear(dim, inter)
+        self.up_proj = _Linear(dim, inter)
+        self.down_proj = _Linear(inter, dim)
+
+
+class _Block(nn.Module):
+    def __init__(self, dim: int, inter: int) -> None:
+        super().__init__()
+        self.norm1 = _Scale(dim)
+        self.norm2 = _Scale(dim)
+        self.attn = _Attn(dim)
+        self.mlp = _MLP(dim, inter)
+
+
+class _Merger(nn.Module):
+    def __init__(self, out_dim: int, context_dim: int, merge: int) -> None:
+        super().__init__()
+        hidden = context_dim * merge * merge
+        self.ln_q = _Scale(context_dim)
+        self.mlp = nn.ModuleList([_Linear(hidden, hidden), nn.Identity(), _Linear(hidden, out_dim)])
+
+
+def _no_mark(name: str) -> None:
+    return None
+
+
+def _round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
+
+
+def quantize_fp8_rows(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """Per-output-channel e4m3 quantisation: scale = amax/448 (fp32), q = rne(w/scale)."""
+    wf = w.float()
+    scale = wf.abs().amax(dim=1).clamp_min(1e-12) / 448.0
+    q = (wf / scale[:, None]).to(torch.float8_e4m3fn)
+    return q, scale.contiguous()
+
+
+class Qwen2_5_VisionTransformer(EricModel):
+    def __init__(self, config: Any, weight_format: str = "bf16") -> None:
+        super().__init__()
+        vc = config.vision_config if hasattr(config, "vision_config") else config
+        if weight_format not in ("bf16", "fp8_e4m3"):
+            raise ValueError(f"Unknown weight_format: {weight_format}")
+        self.weight_format = weight_format
+        self.hidden_size = vc.hidden_size
+        self.out_hidden_size = vc.out_hidden_size
+        self.num_heads = vc.num_heads
+        self.intermediate_size = vc.intermediate_size
+        self.window_size = vc.window_size
+        self.patch_size = vc.patch_size
+        self.temporal_patch_size = vc.temporal_patch_size
+        self.in_channels = getattr(vc, "in_channels", getattr(vc, "in_chans", 3))
+        self.spatial_merge_size = vc.spatial_merge_size
+        self.fullatt_block_indexes = list(vc.fullatt_block_indexes)
+        self.spatial_merge_unit = self.spatial_merge_size**2
+        self.norm_eps = getattr(config, "rms_norm_eps", 1e-6)
+        if getattr(vc, "hidden_act", "silu") != "silu":
+            raise NotImplementedError("only the SiLU-gated MLP of Qwen2.5-VL is implemented")
+        self.head_dim = self.hidden_size // self.num_heads
+
+        self.patch_embed = _PatchEmbed(self.in_channels, self.hidden_size, self.temporal_patch_size, self.patch_size)
+        self.blocks = nn.ModuleList([_Block(self.hidden_size, self.intermediate_size) for _ in range(vc.depth)])
+        self.merger = _Merger(self.out_hidden_size, self.hidden_size, self.spatial_merge_size)
+        self._packed: dict | None = None
+        self.register_load_state_dict_post_hook(lambda module, incompatible: module._invalidate())
+
+    # ------------------------------------------------------------------ EricModel properties
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.patch_embed.proj.weight.dtype
+
+    @property
+    def device(self) -> torch.device:
+        return self.patch_embed.proj.weight.device
+
+    @property
+    def chunk_shape(self) -> tuple[int, ...]:
+        return (1, self.out_hidden_size)
+
+    # ------------------------------------------------------------------ weight repacking
+    def _invalidate(self) -> None:
+        self._packed = None
+
+    def _apply(self, fn, recurse=True):  # .to()/.cuda()/.bfloat16() move the parameters: repack lazily
+        self._packed = None
+        return super()._apply(fn, recurse)
+
+    def _lin(self, w: torch.Tensor, b: torch.Tensor | None) -> dict:
+        """Device form of one linear layer: bf16 [N,K] or fp8 [N,K] + fp32 scale [N]."""
+        w = w.contiguous()
+        if self.weight_format == "fp8_e4m3":
+            q, s = quantize_fp8_rows(w)
+            return {"w": q.contiguous(), "s": s, "b": b}
+        return {"w": w, "s": None, "b": b}
+
+    @torch.no_grad()
+    def _pack(self) -> dict:
+        dev, H, I = self.device, self.hidden_size, self.intermediate_size
+        Ip = _round_up(I, 64)
+        pk: dict = {"Ip": Ip}
+        pk["pe_w"] = self.patch_embed.proj.weight.reshape(H, -1).contiguous()
+        blocks = []
+        for blk in self.blocks:
+            gu_w = torch.zeros((2 * Ip, H), dtype=self.dtype, device=dev)
+            gu_b = torch.zeros(2 * Ip, dtype=self.dtype, device=dev)
+            gu_w[0 : 2 * I : 2] = blk.mlp.gate_proj.weight
+            gu_w[1 : 2 * I : 2] = blk.mlp.up_proj.weight
+            gu_b[0 : 2 * I : 2] = blk.mlp.gate_proj.bias
+            gu_b[1 : 2 * I : 2] = blk.mlp.up_proj.bias
+            down_w = torch.zeros((H, Ip), dtype=self.dtype, device=dev)
+            down_w[:, :I] = blk.mlp.down_proj.weight
+            blocks.append(
+                {
+                    "n1": blk.norm1.weight,
+                    "n2": blk.norm2.weight,
+                    "qkv": self._lin(blk.attn.qkv.weight, blk.attn.qkv.bias),
+                    "proj": self._lin(blk.attn.proj.weight, blk.attn.proj.bias),
+                    "gu": self._lin(gu_w, gu_b),
+                    "down": self._lin(down_w, blk.mlp.down_proj.bias),
+                }
+            )
+        pk["blocks"] = blocks
+        pk["ln_q"] = self.merger.ln_q.weight
+        pk["fc1"] = self._lin(self.merger.mlp[0].weight, self.merger.mlp[0].bias)
+        pk["fc2"] = self._lin(self.merger.mlp[2].weight, self.merger.mlp[2].bias)
+        dim = self.head_dim // 2
+        inv_freq = 1.0 / (10000.0 ** (torch.arange(0, dim, 2, dtype=torch.float) / dim))
+        pk["inv_freq"] = inv_freq.to(dev)
+        return pk
+
+    def _ensure_packed(self) -> dict:
+        if self._packed is None:
+            if self.dtype != torch.bfloat16 or self.device.type != "cuda":
+                raise RuntimeError(
+                    "the gfx950 kernels need the model in bfloat16 on a GPU "
+                    f"(got {self.dtype} on {self.device}); there is no CPU path"
+                )
+            self._packed = self._pack()
+        return self._packed
+
+    # ------------------------------------------------------------------ forward
+    @staticmethod
+    def _g(a: torch.Tensor, lin: dict, **kw) -> torch.Tensor:
+        return ops.gemm(a, lin["w"], lin["b"], w_scale=lin["s"], **kw)
+
+    def get_window_index(self, grid_thw) -> tuple[torch.Tensor, list[int]]:
+        """Same results as the reference method (:357-386) followed by unique_consecutive (:436)."""
+        g = np.asarray(torch.as_tensor(grid_thw).cpu(), dtype=np.int64).reshape(-1, 3)
+        win = self.window_size // self.spatial_merge_size // self.patch_size
+        sl = ops.vit_seqlens_host(g, self.spatial_merge_size, win)
+        pk = self._ensure_packed()
+        meta = torch.from_numpy(sl.item_meta).to(self.device)
+        ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, self.spatial_merge_size, win, pk["inv_freq"])
+        return ix.window_index, sl.cu_window.tolist()
+
+    def forward_device(self, pixel_values: torch.Tensor, grid_thw: np.ndarray, mark=None) -> list[torch.Tensor]:
+        """pixel_values: bf16 [L, C*T*P*P] already on the device; grid_thw: host int64 [n,3].
+
+        `mark`, if given, is called as mark(name) right before the kernels of each named stage are
+        enqueued (profiling hook: the caller records a stream event there)."""
+        if mark is None:
+            mark = _no_mark
+        pk = self._ensure_packed()
+        H, nh, d = self.hidden_size, self.num_heads, self.head_dim
+        unit = self.spatial_merge_unit
+        merge = self.spatial_merge_size
+        win = self.window_size // merge // self.patch_size
+        dev = self.device
+
+        mark("index")
+        sl = ops.vit_seqlens_host(grid_thw, merge, win)
+        L = sl.total_patches
+        if pixel_values.shape[0] != L:
+            raise ValueError(f"pixel_values has {pixel_values.shape[0]} rows but grid_thw describes {L} patches")
+        meta = torch.from_numpy(sl.item_meta).to(dev, non_blocking=True)
+        ix = ops.vit_index(meta, L, sl.max_units_per_item, merge, win, pk["inv_freq"])
+        plan_win = ops.attn_plan(sl.cu_window, dev)
+        plan_full = ops.attn_plan(sl.cu_full, dev)
+
+        # patch embed; rows come out already in window order
+        mark("patch_embed")
+        x = ops.gemm(pixel_values, pk["pe_w"], None, a_rows=ix.src_rows)
+        n = torch.empty_like(x)
+        qkv = torch.empty((L, 3 * H), dtype=torch.bfloat16, device=dev)
+        att = torch.empty((L, H), dtype=torch.bfloat16, device=dev)
+        hmid = torch.empty((L, pk["Ip"]), dtype=torch.bfloat16, device=dev)
+        scale = d**-0.5
+        for i, b in enumerate(pk["blocks"]):
+            full = i in self.fullatt_block_indexes
+            plan = plan_full if full else plan_win
+            mark("norm")
+            ops.rmsnorm(x, b["n1"], self.norm_eps, out=n)
+            mark("gemm_qkv")
+            self._g(n, b["qkv"], out=qkv)
+            mark("attn_full" if full else "attn_window")
+            ops.attn_varlen(qkv[:, :H], qkv[:, H : 2 * H], qkv[:, 2 * H :], plan, nh, d, scale, cos_sin=ix.cos_sin, out=att)
+            mark("gemm_proj")
+            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+            mark("norm")
+            ops.rmsnorm(x, b["n2"], self.norm_eps, out=n)
+            mark("gemm_gate_up")
+            self._g(n, b["gu"], epilogue=ops.EPI_SWIGLU, out=hmid)
+            mark("gemm_down")
+            self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+
+        mark("norm")
+        ops.rmsnorm(x, pk["ln_q"], self.norm_eps, out=n)
+        mark("gemm_merger")
+        y = self._g(n.view(L // unit, H * unit), pk["fc1"], epilogue=ops.EPI_GELU_ERF)
+        out = torch.empty((L // unit, self.out_hidden_size), dtype=torch.bfloat16, device=dev)
+        # merged row m sits at window-order position m; it belongs at row window_index[m]
+        self._g(y, pk["fc2"], c_rows=ix.window_index32, out=out)
+        mark("end")
+        g = grid_thw.reshape(-1, 3)
+        seqlens = (g[:, 0] * g[:, 1] * g[:, 2]) // unit
+        return list(out.split([int(s) for s in seqlens], dim=0))
+
+    @torch.inference_mode()
+    def forward(self, modality: Modality, adapter_name: str, batch: dict[str, list[torch.Tensor]]) -> list[torch.Tensor]:
+        """See the reference docstring (:402-413): `pixel_values` + `image_grid_thw` for images,
+        `pixel_values_videos` + `video_grid_thw` for videos."""
+        if modality == Modality.IMAGE:
+            px_key, grid_key = "pixel_values", "image_grid_thw"
+        elif modality == Modality.VIDEO:
+            px_key, grid_key = "pixel_values_videos", "video_grid_thw"
+        else:
+            raise ValueError(f"Unsupported modality: {modality}")
+        pixel_values = torch.cat(batch[px_key], dim=0).to(device=self.device, dtype=self.dtype)
+        grid = torch.cat([g.reshape(-1, 3) for g in batch[grid_key]], dim=0).cpu().numpy().astype(np.int64)
+        return self.forward_device(pixel_values, grid)
+
+
+class ModalityProcessor(BaseModalityProcessor):
+    """Qwen2.5-VL modality processor (reference: :488-512). Wraps the HF image processor, which has to be
+    available locally; preprocessing is outside the accelerated path."""
+
+    def __init__(self, model_id: str) -> None:
+        super().__init__(model_id=model_id)
+        from transformers import AutoImageProcessor  # deferred: needs the model files
+
+        self.hf_processor = AutoImageProcessor.from_pretrained(model_id)
+
+    def get_image_processor(self) -> Callable | None:
+        def processor(image) -> dict[str, torch.Tensor]:
+            return self.hf_processor(images=[image], return_tensors="pt").data
+
+        return processor
+
+    def get_video_processor(self) -> Callable | None:
+        def processor(video) -> dict[str, torch.Tensor]:
+            return self.hf_processor(images=None, videos=[video], return_tensors="pt").data
+
+        return processor

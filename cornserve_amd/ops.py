@@ -1,0 +1,320 @@
+"""Thin tensor-level wrappers over the C ABI: torch supplies device memory and the stream, nothing else.
+
+Every function enqueues HIP kernels from libcornserve_amd.so on torch's current stream and returns
+torch tensors allocated by torch's caching allocator (so outputs stay IPC-exportable for the sidecar,
+reference: sidecar/api.py:198-242).  There is no eager-PyTorch fallback in this module.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import numpy as np
+import torch
+
+from . import lib as _l
+from .lib import (  # noqa: F401  (re-exported)
+    EPI_BIAS,
+    EPI_GELU_ERF,
+    EPI_GELU_TANH,
+    EPI_RESIDUAL,
+    EPI_SWIGLU,
+)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _req(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a device tensor")
+    if t.dtype != dtype:
+        raise ValueError(f"{name} must be {dtype}, got {t.dtype}")
+    if t.dim() >= 1 and t.stride(-1) != 1:
+        raise ValueError(f"{name} must be contiguous in its last dimension")
+
+
+# --------------------------------------------------------------------------------------------- GEMM
+def gemm(
+    a: torch.Tensor,
+    w: torch.Tensor,
+    bias: torch.Tensor | None = None,
+    *,
+    epilogue: int = EPI_BIAS,
+    residual: torch.Tensor | None = None,
+    w_scale: torch.Tensor | None = None,
+    pos: torch.Tensor | None = None,
+    a_rows: torch.Tensor | None = None,
+    c_rows: torch.Tensor | None = None,
+    out: torch.Tensor | None = None,
+    k: int | None = None,
+) -> torch.Tensor:
+    """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`."""
+    lib = _l.load()
+    _req(a, torch.bfloat16, "a")
+    if a.dim() != 2 or w.dim() != 2:
+        raise ValueError("gemm operands must be 2-D")
+    fp8 = w.dtype in (torch.float8_e4m3fn, torch.uint8)
+    if not fp8:
+        _req(w, torch.bfloat16, "w")
+    elif w_scale is None:
+        raise ValueError("fp8 weights need w_scale")
+    M = a.shape[0] if a_rows is None else a_rows.shape[0]
+    K = a.shape[1] if k is None else k
+    N = w.shape[0]
+    if w.shape[1] < K:
+        raise ValueError(f"w has {w.shape[1]} columns, need at least K={K}")
+    n_out = N // 2 if epilogue == EPI_SWIGLU else N
+    if out is None:
+        out = torch.empty((M, n_out), dtype=torch.bfloat16, device=a.device)
+    args = _l.CsGemmArgs()
+    args.A, args.lda = a.data_ptr(), a.stride(0)
+    args.W, args.ldw = w.data_ptr(), w.stride(0)
+    args.w_scale = _ptr(w_scale)
+    args.bias = _ptr(bias)
+    args.residual = _ptr(residual)
+    args.ldr = residual.stride(0) if residual is not None else 0
+    args.pos = _ptr(pos)
+    args.ldpos = pos.stride(0) if pos is not None else 0
+    args.pos_period = pos.shape[0] if pos is not None else 0
+    args.C, args.ldc = out.data_ptr(), out.stride(0)
+    args.a_rows = _ptr(a_rows)
+    args.c_rows = _ptr(c_rows)
+    args.M, args.N, args.K = M, N, K
+    args.epilogue = epilogue
+    args.w_fp8 = 1 if fp8 else 0
+    _l.check(lib.cs_gemm(ctypes.byref(args), _stream()), "cs_gemm")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- norms
+def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, *, gemma: bool = False,
+            out: torch.Tensor | None = None) -> torch.Tensor:
+    lib = _l.load()
+    _req(x, torch.bfloat16, "x")
+    _req(w, torch.bfloat16, "w")
+    x2 = x.reshape(-1, x.shape[-1])
+    if out is None:
+        out = torch.empty_like(x2)
+    _l.check(
+        lib.cs_rmsnorm(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
+                       x2.shape[0], x2.shape[1], eps, int(gemma), _stream()),
+        "cs_rmsnorm",
+    )
+    return out.view(x.shape)
+
+
+def layernorm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float,
+              out: torch.Tensor | None = None) -> torch.Tensor:
+    lib = _l.load()
+    _req(x, torch.bfloat16, "x")
+    _req(w, torch.bfloat16, "w")
+    _req(b, torch.bfloat16, "b")
+    x2 = x.reshape(-1, x.shape[-1])
+    if out is None:
+        out = torch.empty_like(x2)
+    _l.check(
+        lib.cs_layernorm(x2.data_ptr(), x2.stride(0), w.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
+                         x2.shape[0], x2.shape[1], eps, _stream()),
+        "cs_layernorm",
+    )
+    return out.view(x.shape)
+
+
+def avgpool_gemma_rmsnorm(x: torch.Tensor, w: torch.Tensor, side: int, k: int, eps: float) -> torch.Tensor:
+    """x [B, side*side, H] -> [B, (side/k)^2, H]: AvgPool2d(k) over the token grid, then GemmaRMSNorm."""
+    lib = _l.load()
+    _req(x, torch.bfloat16, "x")
+    _req(w, torch.bfloat16, "w")
+    if x.dim() != 3 or x.shape[1] != side * side or not x.is_contiguous():
+        raise ValueError("x must be contiguous [B, side*side, H]")
+    B, _, H = x.shape
+    out = torch.empty((B, (side // k) ** 2, H), dtype=torch.bfloat16, device=x.device)
+    _l.check(
+        lib.cs_avgpool_gemma_rmsnorm(x.data_ptr(), w.data_ptr(), out.data_ptr(), B, side, k, H, eps, _stream()),
+        "cs_avgpool_gemma_rmsnorm",
+    )
+    return out
+
+
+def cast_f32_bf16(x: torch.Tensor) -> torch.Tensor:
+    lib = _l.load()
+    _req(x, torch.float32, "x")
+    if not x.is_contiguous():
+        raise ValueError("x must be contiguous")
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    _l.check(lib.cs_cast_f32_bf16(x.data_ptr(), out.data_ptr(), x.numel(), _stream()), "cs_cast_f32_bf16")
+    return out
+
+
+# -------------------------------------------------------------------------- Qwen2.5-VL index routines
+@dataclass
+class VitSeqlens:
+    """Host-side result of cs_vit_seqlens_host (numpy arrays) for one batch of grids."""
+
+    cu_window: np.ndarray   # int32 [n_windows + 1]
+    cu_full: np.ndarray     # int32 [n_frames + 1]
+    item_meta: np.ndarray   # int32 [n_items, 8]
+    total_patches: int
+    max_units_per_item: int
+
+
+def vit_seqlens_host(grid_thw: np.ndarray, merge: int, win: int) -> VitSeqlens:
+    lib = _l.load()
+    g = np.ascontiguousarray(grid_thw, dtype=np.int64).reshape(-1, 3)
+    n = g.shape[0]
+    units = (g[:, 0] * (g[:, 1] // merge) * (g[:, 2] // merge)) if n else np.zeros(0, np.int64)
+    frames = int(g[:, 0].sum()) if n else 0
+    cap_w = int(units.sum()) + 2  # every window holds at least one merged unit
+    cap_f = frames + 2
+    cu_w = np.empty(cap_w, np.int32)
+    cu_f = np.empty(cap_f, np.int32)
+    meta = np.zeros((max(n, 1), 8), np.int32)
+    n_w, n_f, total = ctypes.c_int32(0), ctypes.c_int32(0), ctypes.c_int64(0)
+    _l.check(
+        lib.cs_vit_seqlens_host(g.ctypes.data, n, merge, win, cu_w.ctypes.data, cap_w, ctypes.byref(n_w),
+                                cu_f.ctypes.data, cap_f, ctypes.byref(n_f), meta.ctypes.data,
+                                ctypes.byref(total)),
+        "cs_vit_seqlens_host",
+    )
+    return VitSeqlens(cu_w[: n_w.value].copy(), cu_f[: n_f.value].copy(), meta[:n], int(total.value),
+                      int(units.max()) if n else 0)
+
+
+@dataclass
+class VitIndex:
+    window_index32: torch.Tensor  # int32 [U]
+    reverse_index: torch.Tensor  # int32 [U]
+    src_rows: torch.Tensor       # int32 [L]
+    pos_ids: torch.Tensor | None  # int32 [L, 2]
+    cos_sin: torch.Tensor        # fp32 [L, 2*rot_dim]
+
+    @property
+    def window_index(self) -> torch.Tensor:
+        """int64 view of the permutation, the dtype the reference returns."""
+        return self.window_index32.long()
+
+
+def vit_index(item_meta: torch.Tensor, total_patches: int, max_units_per_item: int, merge: int, win: int,
+              inv_freq: torch.Tensor, *, want_pos_ids: bool = False) -> VitIndex:
+    lib = _l.load()
+    _req(item_meta, torch.int32, "item_meta")
+    _req(inv_freq, torch.float32, "inv_freq")
+    dev = item_meta.device
+    L = total_patches
+    U = L // (merge * merge)
+    rot_dim = 2 * inv_freq.numel()
+    window_index = torch.empty(U, dtype=torch.int32, device=dev)
+    reverse_index = torch.empty(U, dtype=torch.int32, device=dev)
+    src_rows = torch.empty(L, dtype=torch.int32, device=dev)
+    pos_ids = torch.empty((L, 2), dtype=torch.int32, device=dev) if want_pos_ids else None
+    cos_sin = torch.empty((L, 2 * rot_dim), dtype=torch.float32, device=dev)
+    _l.check(
+        lib.cs_vit_index(item_meta.data_ptr(), item_meta.shape[0], max_units_per_item, merge, win,
+                         inv_freq.data_ptr(), rot_dim, window_index.data_ptr(), reverse_index.data_ptr(),
+                         src_rows.data_ptr(), _ptr(pos_ids), cos_sin.data_ptr(), _stream()),
+        "cs_vit_index",
+    )
+    return VitIndex(window_index, reverse_index, src_rows, pos_ids, cos_sin)
+
+
+def row_gather(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
+    """out[i] = x[rows[i]] for a 2-D tensor with contiguous rows."""
+    lib = _l.load()
+    _req(rows, torch.int32, "rows")
+    if not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
+        raise ValueError("x must be a 2-D device tensor with contiguous rows")
+    es = x.element_size()
+    out = torch.empty((rows.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    _l.check(
+        lib.cs_row_gather(x.data_ptr(), x.stride(0) * es, rows.data_ptr(), out.data_ptr(), out.stride(0) * es,
+                          rows.shape[0], x.shape[1] * es, _stream()),
+        "cs_row_gather",
+    )
+    return out
+
+
+def rope_qk_(qkv: torch.Tensor, cos_sin: torch.Tensor, heads: int, head_dim: int) -> torch.Tensor:
+    """In-place rotary on the q and k blocks of a packed [L, 3*heads*head_dim] buffer."""
+    lib = _l.load()
+    _req(qkv, torch.bfloat16, "qkv")
+    _req(cos_sin, torch.float32, "cos_sin")
+    if cos_sin.shape != (qkv.shape[0], head_dim) or not cos_sin.is_contiguous():
+        raise ValueError("cos_sin must be contiguous [L, head_dim]")
+    _l.check(
+        lib.cs_rope_qk(qkv.data_ptr(), qkv.stride(0), cos_sin.data_ptr(), qkv.shape[0], heads, head_dim, _stream()),
+        "cs_rope_qk",
+    )
+    return qkv
+
+
+# --------------------------------------------------------------------------------------- attention
+@dataclass
+class AttnPlan:
+    """Device work list for one cu_seqlens: query blocks of one segment each."""
+
+    work: torch.Tensor   # int32 [n_work, 4] on device
+    n_work: int
+    max_seqlen: int
+
+
+def attn_plan(cu_seqlens_host: np.ndarray, device: torch.device) -> AttnPlan:
+    lib = _l.load()
+    cu = np.ascontiguousarray(cu_seqlens_host, dtype=np.int32)
+    n_seg = cu.shape[0] - 1
+    if n_seg <= 0:
+        return AttnPlan(torch.zeros((0, 4), dtype=torch.int32, device=device), 0, 1)
+    lens = np.diff(cu)
+    max_seqlen = int(lens.max())
+    bq = lib.cs_attn_block_q(max_seqlen)
+    cap = int(((lens + bq - 1) // bq).sum()) + 1
+    work = np.empty((cap, 4), np.int32)
+    n_work = ctypes.c_int32(0)
+    _l.check(lib.cs_attn_work_host(cu.ctypes.data, n_seg, bq, work.ctypes.data, cap, ctypes.byref(n_work)),
+             "cs_attn_work_host")
+    w = torch.from_numpy(work[: n_work.value].copy()).to(device, non_blocking=True)
+    return AttnPlan(w, n_work.value, max_seqlen)
+
+
+def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan, heads: int, head_dim: int,
+                scale: float, cos_sin: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """q/k/v: [L, >= heads*head_dim] views sharing one row stride (e.g. thirds of a packed QKV buffer)."""
+    lib = _l.load()
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _req(t, torch.bfloat16, name)
+    if not (q.stride(0) == k.stride(0) == v.stride(0)):
+        raise ValueError("q, k, v must share a row stride")
+    L = q.shape[0]
+    if cos_sin is not None:
+        _req(cos_sin, torch.float32, "cos_sin")
+        if cos_sin.shape != (L, head_dim) or not cos_sin.is_contiguous():
+            raise ValueError("cos_sin must be contiguous [L, head_dim]")
+    if out is None:
+        out = torch.empty((L, heads * head_dim), dtype=torch.bfloat16, device=q.device)
+    _l.check(
+        lib.cs_attn_varlen(q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+                           plan.work.data_ptr(), plan.n_work, heads, head_dim, scale, _ptr(cos_sin),
+                           plan.max_seqlen, _stream()),
+        "cs_attn_varlen",
+    )
+    return out
+
+
+# ------------------------------------------------------------------------------------------ SigLIP
+def patchify_nchw(pixels: torch.Tensor, patch: int, ldo: int) -> torch.Tensor:
+    """[B,C,H,W] bf16 -> [B*(H/p)*(W/p), ldo] rows of (c,ky,kx)-ordered patch values, zero padded."""
+    lib = _l.load()
+    _req(pixels, torch.bfloat16, "pixels")
+    if pixels.dim() != 4 or not pixels.is_contiguous():
+        raise ValueError("pixels must be contiguous [B,C,H,W]")
+    B, C, H, W = pixels.shape
+    out = torch.empty((B * (H // patch) * (W // patch), ldo), dtype=torch.bfloat16, device=pixels.device)
+    _l.check(lib.cs_patchify_nchw(pixels.data_ptr(), B, C, H, W, patch, out.data_ptr(), ldo, _stream()),
+             "cs_patchify_nchw")
+    return out

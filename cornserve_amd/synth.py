@@ -1,0 +1,175 @@
+"""Seeded synthetic weights and inputs for the encoders (no files, no network).
+
+Values come from numpy's Philox generator keyed by (seed, crc32(parameter name)), so they are identical
+on every machine and numpy/torch version and do not depend on the order tensors are drawn in.  Matrices
+and biases are N(0, 0.02), norm scales 1 + N(0, 0.02) (GemmaRMSNorm's zero-centred scale: N(0, 0.02)),
+pixel values N(0, 1) for Qwen2.5-VL patches and U(-1, 1) for SigLIP images.
+"""
+
+from __future__ import annotations
+
+import zlib
+from types import SimpleNamespace
+
+import numpy as np
+import torch
+
+
+def _rng(seed: int, name: str) -> np.random.Generator:
+    return np.random.Generator(np.random.Philox(key=[seed & 0xFFFFFFFFFFFFFFFF, zlib.crc32(name.encode())]))
+
+
+def normal(seed: int, name: str, shape, std: float = 1.0, mean: float = 0.0) -> torch.Tensor:
+    a = _rng(seed, name).standard_normal(size=tuple(shape), dtype=np.float32)
+    if std != 1.0:
+        a *= np.float32(std)
+    if mean != 0.0:
+        a += np.float32(mean)
+    return torch.from_numpy(a)
+
+
+def uniform(seed: int, name: str, shape, lo: float, hi: float) -> torch.Tensor:
+    a = _rng(seed, name).random(size=tuple(shape), dtype=np.float32)
+    return torch.from_numpy(a * np.float32(hi - lo) + np.float32(lo))
+
+
+# ---------------------------------------------------------------------------------------- Qwen2.5-VL
+def qwen_vision_config(depth: int = 32, fullatt_block_indexes=(7, 15, 23, 31)) -> SimpleNamespace:
+    """The Qwen2.5-VL-7B vision tower's hyper-parameters as a plain object (only `vision_config` is read)."""
+    vc = SimpleNamespace(
+        depth=depth, hidden_size=1280, intermediate_size=3420, num_heads=16, in_channels=3, patch_size=14,
+        temporal_patch_size=2, spatial_merge_size=2, window_size=112, out_hidden_size=3584,
+        fullatt_block_indexes=list(fullatt_block_indexes), hidden_act="silu",
+    )
+    return SimpleNamespace(vision_config=vc, model_type="qwen2_5_vl")
+
+
+def qwen_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
+    """fp32 state dict with the checkpoint's names (after `visual.` is stripped)."""
+    vc = config.vision_config
+    H, I, O = vc.hidden_size, vc.intermediate_size, vc.out_hidden_size
+    M = H * vc.spatial_merge_size**2
+    sd: dict[str, torch.Tensor] = {}
+
+    def mat(name, *shape):
+        sd[name] = normal(seed, name, shape, 0.02)
+
+    def scale(name, n):
+        sd[name] = normal(seed, name, (n,), 0.02, 1.0)
+
+    mat("patch_embed.proj.weight", H, vc.in_channels, vc.temporal_patch_size, vc.patch_size, vc.patch_size)
+    for i in range(vc.depth):
+        p = f"blocks.{i}."
+        scale(p + "norm1.weight", H)
+        scale(p + "norm2.weight", H)
+        mat(p + "attn.qkv.weight", 3 * H, H)
+        mat(p + "attn.qkv.bias", 3 * H)
+        mat(p + "attn.proj.weight", H, H)
+        mat(p + "attn.proj.bias", H)
+        mat(p + "mlp.gate_proj.weight", I, H)
+        mat(p + "mlp.gate_proj.bias", I)
+        mat(p + "mlp.up_proj.weight", I, H)
+        mat(p + "mlp.up_proj.bias", I)
+        mat(p + "mlp.down_proj.weight", H, I)
+        mat(p + "mlp.down_proj.bias", H)
+    scale("merger.ln_q.weight", H)
+    mat("merger.mlp.0.weight", M, M)
+    mat("merger.mlp.0.bias", M)
+    mat("merger.mlp.2.weight", O, M)
+    mat("merger.mlp.2.bias", O)
+    return sd
+
+
+def qwen_linear_weight_keys(config) -> list[str]:
+    """Names of the 2-D linear weights (the set the fp8 path quantises)."""
+    keys = []
+    for i in range(config.vision_config.depth):
+        p = f"blocks.{i}."
+        keys += [p + "attn.qkv.weight", p + "attn.proj.weight", p + "mlp.gate_proj.weight",
+                 p + "mlp.up_proj.weight", p + "mlp.down_proj.weight"]
+    return keys + ["merger.mlp.0.weight", "merger.mlp.2.weight"]
+
+
+def qwen_inputs(grids, seed: int = 0) -> tuple[list[torch.Tensor], list[torch.Tensor]]:
+    """One [t*h*w, 1176] fp32 N(0,1) tensor and one [1,3] int64 grid per item."""
+    px, gr = [], []
+    for i, (t, h, w) in enumerate(grids):
+        px.append(normal(seed, f"pixel_values.{i}", (t * h * w, 1176)))
+        gr.append(torch.tensor([[t, h, w]], dtype=torch.int64))
+    return px, gr
+
+
+def ragged_grids(n: int = 16, seed: int = 0, lo: int = 224, hi: int = 1344) -> list[tuple[int, int, int]]:
+    """Image grids with H, W drawn independently and uniformly from the multiples of 28 in [lo, hi]."""
+    rng = _rng(seed, "ragged_grids")
+    sizes = rng.integers(lo // 28, hi // 28 + 1, size=(n, 2)) * 28
+    return [(1, int(h) // 14, int(w) // 14) for h, w in sizes]
+
+
+# --------------------------------------------------------------------------------------- Gemma-3 / SigLIP
+def gemma3_config(num_hidden_layers: int = 27, image_size: int = 896, text_hidden: int = 2560,
+                  mm_tokens_per_image: int = 256) -> SimpleNamespace:
+    vc = SimpleNamespace(
+        hidden_size=1152, intermediate_size=4304, num_hidden_layers=num_hidden_layers, num_attention_heads=16,
+        num_channels=3, image_size=image_size, patch_size=14, layer_norm_eps=1e-6,
+        hidden_act="gelu_pytorch_tanh", attention_dropout=0.0, vision_use_head=False,
+    )
+    return SimpleNamespace(vision_config=vc, text_config=SimpleNamespace(hidden_size=text_hidden),
+                           mm_tokens_per_image=mm_tokens_per_image, model_type="gemma3")
+
+
+def gemma3_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
+    """fp32 state dict with the checkpoint's names: `vision_tower.*` and `multi_modal_projector.*`."""
+    vc = config.vision_config
+    H, I = vc.hidden_size, vc.intermediate_size
+    VT = "vision_tower.vision_model."
+    sd: dict[str, torch.Tensor] = {}
+
+    def mat(name, *shape):
+        sd[name] = normal(seed, name, shape, 0.02)
+
+    def ln(prefix):
+        sd[prefix + ".weight"] = normal(seed, prefix + ".weight", (H,), 0.02, 1.0)
+        sd[prefix + ".bias"] = normal(seed, prefix + ".bias", (H,), 0.02)
+
+    mat(VT + "embeddings.patch_embedding.weight", H, vc.num_channels, vc.patch_size, vc.patch_size)
+    mat(VT + "embeddings.patch_embedding.bias", H)
+    mat(VT + "embeddings.position_embedding.weight", (vc.image_size // vc.patch_size) ** 2, H)
+    for i in range(vc.num_hidden_layers):
+        p = f"{VT}encoder.layers.{i}."
+        ln(p + "layer_norm1")
+        ln(p + "layer_norm2")
+        for proj in ("q_proj", "k_proj", "v_proj", "out_proj"):
+            mat(p + f"self_attn.{proj}.weight", H, H)
+            mat(p + f"self_attn.{proj}.bias", H)
+        mat(p + "mlp.fc1.weight", I, H)
+        mat(p + "mlp.fc1.bias", I)
+        mat(p + "mlp.fc2.weight", H, I)
+        mat(p + "mlp.fc2.bias", H)
+    ln(VT + "post_layernorm")
+    mat("multi_modal_projector.mm_input_projection_weight", H, config.text_config.hidden_size)
+    mat("multi_modal_projector.mm_soft_emb_norm.weight", H)
+    return sd
+
+
+def gemma3_inputs(n_images: int, image_size: int, seed: int = 0) -> tuple[list[torch.Tensor], list[torch.Tensor]]:
+    px = [uniform(seed, f"pixel_values.{i}", (1, 3, image_size, image_size), -1.0, 1.0) for i in range(n_images)]
+    crops = [torch.zeros(1, dtype=torch.int64) for _ in range(n_images)]
+    return px, crops
+
+
+def load_gemma3(model, sd: dict[str, torch.Tensor], adapter_name: str = "default") -> None:
+    """Load a full Gemma-3 checkpoint-style dict the way the reference loader does (eric/executor/loader.py:
+    121-174): tower weights into the model, `multi_modal_projector.*` (prefix stripped) into a new adapter."""
+    tower = {k: v for k, v in sd.items() if not k.startswith("multi_modal_projector.")}
+    inc = model.load_state_dict(tower, strict=False)
+    if inc.missing_keys:
+        raise ValueError(f"Missing weights in the model: {inc.missing_keys}")
+    if inc.unexpected_keys:
+        raise ValueError(f"Unexpected weights in the model: {inc.unexpected_keys}")
+    adapter = model.multi_modal_projector.make_adapter(adapter_name, model.config)
+    adapter.to(device=model.device, dtype=model.dtype)
+    ad = {k[len("multi_modal_projector."):]: v for k, v in sd.items() if k.startswith("multi_modal_projector.")}
+    inc = adapter.load_state_dict(ad, strict=False)
+    if inc.missing_keys or inc.unexpected_keys:
+        raise ValueError(f"Adapter weights mismatch: {inc}")

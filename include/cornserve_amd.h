@@ -1,0 +1,177 @@
+/*
+ * cornserve_amd.h -- C ABI of the MI355X (gfx950) kernels behind the Eric encoder forward pass.
+ *
+ * The reference (cornserve-ai/cornserve) is pure Python; its encoder forward
+ * (python/cornserve/task_executors/eric/models/{qwen2_5_vl,gemma3}.py, layers/{siglip,norm,linear,
+ * attention,activations}.py) reaches device code only through torch / flash-attn / xformers calls.
+ * Each entry point below replaces one of those call sites and cites it.  A reference-side binding is a
+ * ctypes (or torch.library) stub: load libcornserve_amd.so, pass tensor.data_ptr() values, sizes and
+ * torch.cuda.current_stream().cuda_stream.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the parameter name ends in _host;
+ *   - matrices are row-major with an explicit leading dimension in ELEMENTS;
+ *   - bf16 is the storage type of activations and weights (uint16 bit pattern of the upper half of an
+ *     IEEE fp32, round-to-nearest-even); fp8 weights are OCP e4m3 (e4m3fn) bytes;
+ *   - `stream` is a hipStream_t passed as void*; kernels are enqueued on it and the call returns
+ *     without synchronising;
+ *   - no entry point allocates or frees memory, and none takes ownership of a buffer;
+ *   - the return value is a status code (0 = ok); nothing aborts the process.  The host wrapper maps
+ *     CS_ERR_INVALID_ARG to ValueError and the rest to RuntimeError (reference error behaviour:
+ *     qwen2_5_vl.py:420-421, gemma3.py:112-123).
+ */
+#ifndef CORNSERVE_AMD_H
+#define CORNSERVE_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CS_OK 0
+#define CS_ERR_INVALID_ARG 1
+#define CS_ERR_UNSUPPORTED 2
+#define CS_ERR_LAUNCH 3
+#define CS_ERR_TOO_LARGE 4
+
+/* ABI version of this header; cs_abi_version() returns the value the library was built with. */
+#define CS_ABI_VERSION 1
+int cs_abi_version(void);
+
+/* ------------------------------------------------------------------------------------------------
+ * GEMM:  C[M,N] = epilogue(A[M,K] . W[N,K]^T)     (bf16 in, fp32 accumulate on MFMA, bf16 out)
+ * Replaces F.linear at linear.py:183 (ColumnParallelLinear) and linear.py:549 (RowParallelLinear),
+ * the Conv3d patch embed at qwen2_5_vl.py:195-201 (a GEMM on the flat [L,1176] input), the merger
+ * MLP at qwen2_5_vl.py:225-233, the SigLIP projections at siglip.py:121-125,142-143,155-163 and the
+ * Gemma-3 projection matmul at gemma3.py:48.
+ * ---------------------------------------------------------------------------------------------- */
+enum CsEpilogue {
+  CS_EPI_BIAS = 0,      /* y = acc (+ bias)                                                     */
+  CS_EPI_RESIDUAL = 1,  /* y = bf16(acc + bias) + residual[m,n]         qwen2_5_vl.py:175,177   */
+  CS_EPI_SWIGLU = 2,    /* W rows interleaved gate_j,up_j; y[m,j] = silu(g)*u; C is N/2 wide
+                           qwen2_5_vl.py:143-148                                               */
+  CS_EPI_GELU_ERF = 3,  /* y = gelu(acc + bias), erf form               qwen2_5_vl.py:220       */
+  CS_EPI_GELU_TANH = 4  /* y = gelu(acc + bias), tanh form              siglip.py:155-163       */
+};
+
+typedef struct CsGemmArgs {
+  const void* A;         /* bf16 [M,K], leading dimension lda                                    */
+  int64_t lda;
+  const void* W;         /* bf16 [N,K] (w_fp8 = 0) or e4m3 bytes [N,K] (w_fp8 = 1), ld = ldw      */
+  int64_t ldw;
+  const float* w_scale;  /* fp32 [N] per-output-channel scale; required when w_fp8, else NULL     */
+  const void* bias;      /* bf16 [N] or NULL                                                     */
+  const void* residual;  /* bf16 [M,N] (CS_EPI_RESIDUAL), leading dimension ldr                   */
+  int64_t ldr;
+  const void* pos;       /* optional bf16 [pos_period, N] addend indexed by (m % pos_period):     */
+  int64_t ldpos;         /*   SigLIP learned position embedding, siglip.py:100                    */
+  int32_t pos_period;
+  void* C;               /* bf16 [M,N] (or [M,N/2] for CS_EPI_SWIGLU), leading dimension ldc      */
+  int64_t ldc;
+  const int32_t* a_rows; /* optional [M]: A row used for output row m (gather, qwen2_5_vl.py:438-440) */
+  const int32_t* c_rows; /* optional [M]: C row written for output row m (scatter, :478-479)      */
+  int32_t M, N, K;
+  int32_t epilogue;      /* enum CsEpilogue                                                      */
+  int32_t w_fp8;
+  int32_t tiles_m, tiles_n; /* filled in by the library                                          */
+} CsGemmArgs;
+
+/* Constraints: K % 8 == 0 (16 with fp8), lda/ldw % 8 == 0, N % 4 == 0, A and W 16-byte aligned. */
+int cs_gemm(const CsGemmArgs* args, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Normalisation (HBM-bound, one wavefront per row).
+ * ---------------------------------------------------------------------------------------------- */
+/* RMSNorm, norm.py:35-70: y = bf16(x * rsqrt(mean(x^2) + eps)) * w   (cast BEFORE the weight).
+ * gemma = 1 selects GemmaRMSNorm, norm.py:90-113: y = bf16(x * rsqrt(..) * (1 + w)).              */
+int cs_rmsnorm(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int32_t rows, int32_t H,
+               float eps, int32_t gemma, void* stream);
+/* nn.LayerNorm with affine, siglip.py:173-175,333.                                                */
+int cs_layernorm(const void* x, int64_t ldx, const void* w, const void* b, void* y, int64_t ldy,
+                 int32_t rows, int32_t H, float eps, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Qwen2.5-VL index routines (integer, bit-exact).
+ * ---------------------------------------------------------------------------------------------- */
+/* Host routine.  From grid_thw_host[n_items][3] (t,h,w as int64) compute, exactly as
+ * get_window_index + unique_consecutive (qwen2_5_vl.py:357-386,431-436) and the cu_seqlens
+ * computation (:445-448):
+ *   cu_window_host  int32, n_cu_window entries written (capacity cap_window)
+ *   cu_full_host    int32, n_cu_full entries written   (capacity cap_full)
+ *   item_meta_host  int32 [n_items][8]: t, h/merge, w/merge, first merged unit, first window-order
+ *                   unit (== first merged unit), windows per row, windows per column, reserved
+ * merge = spatial merge size (2), win = window side in merged units (window_size/merge/patch = 4).
+ * Returns CS_ERR_TOO_LARGE if a capacity is too small.                                            */
+int cs_vit_seqlens_host(const int64_t* grid_thw_host, int32_t n_items, int32_t merge, int32_t win,
+                        int32_t* cu_window_host, int32_t cap_window, int32_t* n_cu_window,
+                        int32_t* cu_full_host, int32_t cap_full, int32_t* n_cu_full,
+                        int32_t* item_meta_host, int64_t* total_patches);
+
+/* Device routine.  From item_meta (device copy of the array above) fill, for L = total patches and
+ * U = L / merge^2 merged units:
+ *   window_index  int32 [U]   qwen2_5_vl.py:357-386 (value = original unit at window-order position;
+ *                             the reference holds the same values as int64)
+ *   reverse_index int32 [U]   argsort(window_index), :478
+ *   src_rows      int32 [L]   original patch row feeding window-order row m (units of merge^2 rows), :438-440
+ *   pos_ids       int32 [L,2] (h,w) of each patch in ORIGINAL order, rot_pos_emb :325-350
+ *   cos_sin       fp32  [L, 2*rot_dim] window-order rotary table: cos(angles) | sin(angles) with
+ *                 angles = [h*inv_freq | w*inv_freq], :251-259,352-354,441-443 and :26-29
+ * inv_freq: fp32 [rot_dim/2] on device.  Any output pointer may be NULL to skip it.               */
+int cs_vit_index(const int32_t* item_meta, int32_t n_items, int32_t max_units_per_item, int32_t merge,
+                 int32_t win, const float* inv_freq, int32_t rot_dim, int32_t* window_index,
+                 int32_t* reverse_index, int32_t* src_rows, int32_t* pos_ids, float* cos_sin, void* stream);
+
+/* out[i, :] = in[rows[i], :] for row_bytes-wide rows (row_bytes % 4 == 0): the advanced-indexing
+ * gathers at qwen2_5_vl.py:438-443 and :479.                                                     */
+int cs_row_gather(const void* in, int64_t in_stride_bytes, const int32_t* rows, void* out,
+                  int64_t out_stride_bytes, int32_t n_rows, int32_t row_bytes, void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Rotary embedding, qwen2_5_vl.py:26-33,100-103 (flash_attn apply_rotary_emb, non-interleaved,
+ * full head): for each row l, head h, j < d/2:
+ *   o[j] = x[j]*cos[l,j] - x[j+d/2]*sin[l,j];  o[j+d/2] = x[j]*sin[l,j] + x[j+d/2]*cos[l,j]
+ * fp32 math, one bf16 rounding.  In place on the q and k column blocks of a packed [L, 3*heads*d]
+ * QKV buffer.  cos_sin is the [L, d] table written by cs_vit_index (cos | sin, d/2 each).        */
+int cs_rope_qk(void* qkv, int64_t ld, const float* cos_sin, int32_t L, int32_t heads, int32_t head_dim,
+               void* stream);
+
+/* ------------------------------------------------------------------------------------------------
+ * Variable-length non-causal attention: replaces flash_attn_varlen_func (qwen2_5_vl.py:110-120)
+ * and xformers memory_efficient_attention_forward (attention.py:51).
+ * q, k, v: bf16, row l / head h at  base + l*ld + h*head_dim  (so a packed QKV buffer is passed as
+ * three pointers with ld = 3*heads*head_dim); out: bf16 [L, heads*head_dim] with leading dimension
+ * ldo.  cu_seqlens: int32 [n_seg+1] on device; work: int32 [n_work][4] = (segment start, segment
+ * end, first query row, number of query rows <= block_q) built by cs_attn_work_host.  If cos_sin is
+ * not NULL the rotary embedding above is applied to q and k as they are loaded (fused path).
+ * scale = head_dim^-0.5.  Supported head_dim: multiples of 8 up to 96.                            */
+int cs_attn_varlen(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
+                   const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
+                   const float* cos_sin, int32_t max_seqlen, void* stream);
+/* Host routine: expand cu_seqlens_host[n_seg+1] into query-block work items of at most block_q rows
+ * (block_q = cs_attn_block_q(max_seqlen)).  Writes n_work items of 4 int32 into work_host.      */
+int cs_attn_block_q(int32_t max_seqlen);
+int cs_attn_work_host(const int32_t* cu_seqlens_host, int32_t n_seg, int32_t block_q, int32_t* work_host,
+                      int32_t cap_items, int32_t* n_work);
+
+/* ------------------------------------------------------------------------------------------------
+ * SigLIP / Gemma-3 pieces.
+ * ---------------------------------------------------------------------------------------------- */
+/* Strided gather of non-overlapping patches (Conv2d k = s = patch, padding valid; siglip.py:30-36,
+ * 94-95) from NCHW pixels [B,C,H,W] (bf16) into the GEMM operand [B*(H/p)*(W/p), ldo] with columns
+ * ordered (c, ky, kx) and zero padding up to ldo.                                                 */
+int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_t H, int32_t W, int32_t patch,
+                     void* out, int64_t ldo, void* stream);
+/* Gemma3MultiModalProjector front half, gemma3.py:36-46: AvgPool2d(k) over the side x side token grid
+ * followed by GemmaRMSNorm.  x: bf16 [B, side*side, H] -> y: bf16 [B, (side/k)^2, H].             */
+int cs_avgpool_gemma_rmsnorm(const void* x, const void* w, void* y, int32_t B, int32_t side, int32_t k,
+                             int32_t H, float eps, void* stream);
+
+/* fp32 -> bf16 (round to nearest even) and the reverse, n elements: the `.to(dtype)` at
+ * qwen2_5_vl.py:415-419.                                                                         */
+int cs_cast_f32_bf16(const float* in, void* out, int64_t n, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CORNSERVE_AMD_H */

@@ -1,0 +1,151 @@
+"""Writes the golden fixtures in this directory.  Run once, in a container that has `transformers`:
+
+    python tests/golden/make_golden.py
+
+Source of truth: the third-party Hugging Face implementations of the same networks, which are what the
+reference's own tests compare Eric against (python/tests/task_executors/eric/models/test_qwen2_5_vl.py:
+63-105, test_gemma3.py:73-97).  The reference package itself is not imported (it needs Python >= 3.11,
+flash-attn and xformers).  Models are built from local config objects with the seeded synthetic weights
+of cornserve_amd.synth, fp32, CPU, eager/sdpa attention.  Outputs:
+
+    index_golden.json        window_index / cu_window_seqlens / cu_seqlens / position ids from
+                             transformers.vision_utils for the benchmark grids and a set of ragged grids
+                             (full arrays for small grids, sha256 + head for large ones)
+    qwen2_5_vl_cfg1.npz      config 1 (4 blocks, one 448x448 image): every 16th column of the [256,3584]
+                             output, per-row L2 norms, sum and abs-sum
+    gemma3_small.npz         2-layer SigLIP (224x224, 256 tokens) + projector to 16 tokens x 640: full output
+"""
+
+from __future__ import annotations
+
+import hashlib
+import json
+import sys
+from pathlib import Path
+
+import numpy as np
+import torch
+
+HERE = Path(__file__).resolve().parent
+sys.path.insert(0, str(HERE.parent.parent))
+
+from cornserve_amd import synth  # noqa: E402
+
+INDEX_GRIDS = {
+    "cfg1": [(1, 32, 32)],
+    "cfg2": [(1, 32, 32)] * 8,
+    "cfg5": [(8, 24, 42)] * 2,
+    "cfg4_ragged16": synth.ragged_grids(16, seed=4),
+    "tiny_mixed": [(1, 4, 4), (2, 6, 10), (1, 18, 14), (3, 2, 2), (1, 8, 16), (1, 10, 6)],
+    "edge_exact_multiple": [(1, 8, 8), (1, 16, 24), (2, 8, 40)],
+    "edge_single_unit": [(1, 2, 2), (1, 2, 34), (1, 34, 2)],
+}
+
+
+def sha(a: np.ndarray) -> str:
+    return hashlib.sha256(np.ascontiguousarray(a).tobytes()).hexdigest()
+
+
+def make_index() -> None:
+    from transformers import vision_utils as vu
+
+    out = {}
+    for name, grids in INDEX_GRIDS.items():
+        g = torch.tensor(grids, dtype=torch.int64)
+        wi, cu_w = vu.get_vision_window_index(g, spatial_merge_size=2, window_size=112, patch_size=14)
+        pos = vu.get_vision_position_ids(g, 2)
+        cu_f = vu.get_vision_cu_seqlens(g)
+        wi, cu_w, pos, cu_f = (np.asarray(t.cpu()) for t in (wi, cu_w, pos, cu_f))
+        rec = {
+            "grids": [list(x) for x in grids],
+            "window_index_len": int(wi.shape[0]),
+            "window_index_sha256_int64": sha(wi.astype(np.int64)),
+            "cu_window_seqlens": cu_w.astype(np.int64).tolist(),
+            "cu_seqlens": cu_f.astype(np.int64).tolist(),
+            "pos_ids_shape": list(pos.shape),
+            "pos_ids_sha256_int64": sha(pos.astype(np.int64)),
+        }
+        if wi.shape[0] <= 4096:
+            rec["window_index"] = wi.astype(np.int64).tolist()
+        else:
+            rec["window_index_head"] = wi[:64].astype(np.int64).tolist()
+        if pos.shape[0] <= 2048:
+            rec["pos_ids"] = pos.astype(np.int64).tolist()
+        out[name] = rec
+    (HERE / "index_golden.json").write_text(json.dumps(out))
+    print("index_golden.json", {k: v["window_index_len"] for k, v in out.items()})
+
+
+def make_qwen_cfg1() -> None:
+    from transformers.models.qwen2_5_vl.configuration_qwen2_5_vl import Qwen2_5_VLVisionConfig
+    from transformers.models.qwen2_5_vl.modeling_qwen2_5_vl import Qwen2_5_VisionTransformerPretrainedModel
+
+    cfg = synth.qwen_vision_config(depth=4, fullatt_block_indexes=(3,))
+    vc = cfg.vision_config
+    hf_cfg = Qwen2_5_VLVisionConfig(
+        depth=vc.depth, hidden_size=vc.hidden_size, intermediate_size=vc.intermediate_size, num_heads=vc.num_heads,
+        out_hidden_size=vc.out_hidden_size, fullatt_block_indexes=list(vc.fullatt_block_indexes),
+        window_size=vc.window_size, patch_size=vc.patch_size, spatial_merge_size=vc.spatial_merge_size,
+        temporal_patch_size=vc.temporal_patch_size, hidden_act="silu",
+    )
+    hf_cfg._attn_implementation = "sdpa"
+    model = Qwen2_5_VisionTransformerPretrainedModel(hf_cfg).float().eval()
+    sd = synth.qwen_state_dict(cfg, seed=1)
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys, inc
+    px, grid = synth.qwen_inputs([(1, 32, 32)], seed=1)
+    with torch.no_grad():
+        out = model(px[0], grid_thw=grid[0]).pooler_output.float().numpy()
+    assert out.shape == (256, 3584)
+    np.savez_compressed(
+        HERE / "qwen2_5_vl_cfg1.npz",
+        sample=out[:, ::16].astype(np.float32),
+        row_l2=np.linalg.norm(out.astype(np.float64), axis=1).astype(np.float32),
+        total=np.float64(out.astype(np.float64).sum()),
+        abs_total=np.float64(np.abs(out.astype(np.float64)).sum()),
+        seed=np.int64(1),
+    )
+    print("qwen2_5_vl_cfg1.npz", out.shape, float(np.abs(out).mean()))
+
+
+def make_gemma3_small() -> None:
+    from transformers.models.gemma3.configuration_gemma3 import Gemma3Config, Gemma3TextConfig
+    from transformers.models.gemma3.modeling_gemma3 import Gemma3MultiModalProjector
+    from transformers.models.siglip.configuration_siglip import SiglipVisionConfig
+    from transformers.models.siglip.modeling_siglip import SiglipVisionModel
+
+    cfg = synth.gemma3_config(num_hidden_layers=2, image_size=224, text_hidden=640, mm_tokens_per_image=16)
+    vc = cfg.vision_config
+    hf_vc = SiglipVisionConfig(
+        hidden_size=vc.hidden_size, intermediate_size=vc.intermediate_size, num_hidden_layers=vc.num_hidden_layers,
+        num_attention_heads=vc.num_attention_heads, image_size=vc.image_size, patch_size=vc.patch_size,
+        hidden_act=vc.hidden_act, layer_norm_eps=vc.layer_norm_eps, vision_use_head=False,
+    )
+    hf_vc._attn_implementation = "sdpa"
+    tower = SiglipVisionModel(hf_vc).float().eval()
+    g3 = Gemma3Config(vision_config=hf_vc, text_config=Gemma3TextConfig(hidden_size=640), mm_tokens_per_image=16)
+    proj = Gemma3MultiModalProjector(g3).float().eval()
+    sd = synth.gemma3_state_dict(cfg, seed=2)
+    # HF's SiglipVisionModel in this version is flat (no `vision_model.` level).
+    tower_keys = set(tower.state_dict().keys())
+    prefix = "vision_tower.vision_model." if not any(k.startswith("vision_model.") for k in tower_keys) else "vision_tower."
+    tsd = {k[len(prefix):]: v for k, v in sd.items() if k.startswith("vision_tower.")}
+    inc = tower.load_state_dict(tsd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys, inc
+    psd = {k[len("multi_modal_projector."):]: v for k, v in sd.items() if k.startswith("multi_modal_projector.")}
+    inc = proj.load_state_dict(psd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys, inc
+    px, _ = synth.gemma3_inputs(2, 224, seed=2)
+    with torch.no_grad():
+        feats = tower(pixel_values=torch.cat(px)).last_hidden_state
+        out = proj(feats).float().numpy()
+    assert out.shape == (2, 16, 640), out.shape
+    np.savez_compressed(HERE / "gemma3_small.npz", out=out.astype(np.float32),
+                        feats_sample=feats.float().numpy()[:, ::8, ::8].astype(np.float32), seed=np.int64(2))
+    print("gemma3_small.npz", out.shape, float(np.abs(out).mean()))
+
+
+if __name__ == "__main__":
+    make_index()
+    make_qwen_cfg1()
+    make_gemma3_small()

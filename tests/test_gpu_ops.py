@@ -1,0 +1,303 @@
+"""Per-kernel parity on a real MI355X, through the C ABI, against the oracle's pieces.
+
+Bars: integer/byte/index work bit-exact; floating point within the tolerances written at each check
+(bf16 outputs: one or two bf16 roundings of slack, i.e. max |err| <= 2^-7 relative to the row scale).
+"""
+
+import json
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import gemma3 as og
+from oracle import qwen2_5_vl as oq
+from oracle import vit_index as vi
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch.device("cuda:0")
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from cornserve_amd import ops as _ops
+
+    return _ops
+
+
+def close(got: torch.Tensor, ref: torch.Tensor, rel: float, what: str = ""):
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert not torch.isnan(got).any(), what
+    err = (got - ref).abs().max().item()
+    scale = ref.abs().max().item() + 1e-12
+    assert err <= rel * scale, f"{what}: max err {err:.4g} vs scale {scale:.4g} (rel {err / scale:.4g} > {rel})"
+
+
+def rnd(shape, std=1.0, seed=0, dev="cpu"):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * std).bfloat16().to(dev)
+
+
+# ------------------------------------------------------------------------------------------- index
+def test_vit_index_bit_exact(ops, dev, golden_dir):
+    golden = json.loads((golden_dir / "index_golden.json").read_text())
+    inv_freq = (1.0 / (10000.0 ** (torch.arange(0, 40, 2, dtype=torch.float) / 40))).to(dev)
+    cases = {k: v["grids"] for k, v in golden.items()}
+    rng = np.random.default_rng(3)
+    cases["random"] = [(int(rng.integers(1, 4)), int(rng.integers(1, 40)) * 2, int(rng.integers(1, 40)) * 2) for _ in range(7)]
+    for name, grids in cases.items():
+        g = np.array(grids, np.int64)
+        sl = ops.vit_seqlens_host(g, 2, 4)
+        ix = ops.vit_index(torch.from_numpy(sl.item_meta).to(dev), sl.total_patches, sl.max_units_per_item, 2, 4,
+                           inv_freq, want_pos_ids=True)
+        wi, cu = vi.get_window_index(grids)
+        assert ix.window_index.dtype == torch.int64
+        assert np.array_equal(ix.window_index.cpu().numpy(), wi), name
+        assert np.array_equal(ix.reverse_index.cpu().numpy(), np.argsort(wi)), name
+        assert np.array_equal(ix.pos_ids.cpu().numpy(), vi.rot_pos_ids(grids)), name
+        src = (wi[:, None] * 4 + np.arange(4)[None, :]).reshape(-1)
+        assert np.array_equal(ix.src_rows.cpu().numpy(), src), name
+        # rotary table: window-ordered angles [h*f | w*f] -> cos | sin, fp32
+        ocfg = oq.QwenVisionConfig()
+        ang = oq.rot_pos_emb(ocfg, g).reshape(-1, 4, 40)[torch.from_numpy(wi)].reshape(-1, 40)
+        ref = torch.cat([ang.cos(), ang.sin()], dim=-1)
+        assert (ix.cos_sin.cpu() - ref).abs().max().item() <= 2e-6, name  # fp32 cos/sin, angles < 100 rad
+
+
+def test_row_gather_bit_exact(ops, dev):
+    x = rnd((1000, 1280), dev=dev)
+    rows = torch.randperm(1000, generator=torch.Generator().manual_seed(0)).int().to(dev)
+    assert torch.equal(ops.row_gather(x, rows), x[rows.long()])
+    xf = torch.randn(333, 40, device=dev)  # fp32 rows of 160 bytes (the rotary table)
+    rows = torch.randint(0, 333, (500,), device=dev).int()
+    assert torch.equal(ops.row_gather(xf, rows), xf[rows.long()])
+    assert ops.row_gather(x, rows[:0]).shape == (0, 1280)
+
+
+def test_cast_bit_exact(ops, dev):
+    for n in (0, 1, 7, 8, 1176 * 333, 100003):
+        x = torch.randn(n, device=dev) * 3
+        assert torch.equal(ops.cast_f32_bf16(x), x.bfloat16())
+
+
+def test_patchify_bit_exact(ops, dev):
+    px = rnd((2, 3, 56, 84), dev=dev)
+    got = ops.patchify_nchw(px, 14, 592)
+    ref = px.view(2, 3, 4, 14, 6, 14).permute(0, 2, 4, 1, 3, 5).reshape(48, 588)
+    assert torch.equal(got[:, :588], ref) and (got[:, 588:] == 0).all()
+
+
+# ------------------------------------------------------------------------------------------- norms
+@pytest.mark.parametrize("rows,H", [(1, 1280), (1023, 1280), (64, 1152), (5, 64), (7, 5120)])
+def test_rmsnorm(ops, dev, rows, H):
+    x = rnd((rows, H), 2.0, 1, dev)
+    w = (1 + 0.02 * torch.randn(H)).bfloat16().to(dev)
+    ref = oq.rms_norm(x.cpu(), w.cpu(), 1e-6)
+    close(ops.rmsnorm(x, w, 1e-6), ref, 2**-7, "rmsnorm")
+    refg = og.gemma_rms_norm(x.cpu(), w.cpu(), 1e-6)
+    close(ops.rmsnorm(x, w, 1e-6, gemma=True), refg, 2**-7, "gemma rmsnorm")
+
+
+def test_rmsnorm_special_cases(ops, dev):
+    x = torch.full((3, 1280), 3.0, dtype=torch.bfloat16, device=dev)
+    w = torch.arange(1280, dtype=torch.float).bfloat16().to(dev)
+    assert torch.equal(ops.rmsnorm(x, w, 0.0), w.expand(3, 1280))  # constant row -> exactly w
+
+
+@pytest.mark.parametrize("rows,H", [(1, 1152), (777, 1152), (9, 1280)])
+def test_layernorm(ops, dev, rows, H):
+    x = rnd((rows, H), 2.0, 2, dev)
+    w = (1 + 0.02 * torch.randn(H)).bfloat16().to(dev)
+    b = (0.02 * torch.randn(H)).bfloat16().to(dev)
+    ref = F.layer_norm(x.float().cpu(), (H,), w.float().cpu(), b.float().cpu(), 1e-6)
+    close(ops.layernorm(x, w, b, 1e-6), ref, 2**-7, "layernorm")
+
+
+def test_avgpool_gemma_rmsnorm(ops, dev):
+    cfg = og.SiglipConfig(image_size=224, mm_tokens_per_image=16)
+    x = rnd((2, 256, 1152), 1.0, 3, dev)
+    w = (0.1 * torch.randn(1152)).bfloat16().to(dev)
+    got = ops.avgpool_gemma_rmsnorm(x, w, 16, 4, 1e-6)
+    xc = x.cpu()
+    pooled = F.avg_pool2d(xc.transpose(1, 2).reshape(2, 1152, 16, 16), 4).flatten(2).transpose(1, 2)
+    ref = og.gemma_rms_norm(pooled, w.cpu(), cfg.layer_norm_eps)
+    close(got, ref, 2**-7, "avgpool+gemma rmsnorm")
+
+
+# -------------------------------------------------------------------------------------------- GEMM
+def lin_ref(a, w, bias):
+    return a.float().cpu() @ w.float().cpu().t() + (bias.float().cpu() if bias is not None else 0.0)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 1280, 1280), (255, 256, 64), (257, 260, 72), (1000, 1280, 1176),
+                                   (300, 1152, 4304), (2048, 3840, 1280), (64, 3584, 5120), (130, 2560, 1152)])
+def test_gemm_bias(ops, dev, M, N, K):
+    a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.02, 2, dev), rnd((N,), 0.02, 3, dev)
+    close(ops.gemm(a, w, b), lin_ref(a, w, b), 2**-7, f"gemm {M}x{N}x{K}")
+    close(ops.gemm(a, w, None), lin_ref(a, w, None), 2**-7, f"gemm nobias {M}x{N}x{K}")
+
+
+def test_gemm_exact_small_integers(ops, dev):
+    # products and sums of small integers are exact in bf16/fp32: any indexing mistake shows up bit-exactly
+    g = torch.Generator().manual_seed(0)
+    a = torch.randint(-3, 4, (300, 136), generator=g).bfloat16().to(dev)
+    w = torch.randint(-3, 4, (200, 136), generator=g).bfloat16().to(dev)
+    ref = (a.float() @ w.float().t())
+    assert ref.abs().max() < 256  # representable in bf16
+    assert torch.equal(ops.gemm(a, w, None).float(), ref)
+
+
+def test_gemm_epilogues(ops, dev):
+    M, N, K = 515, 1280, 1280
+    a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
+    res = rnd((M, N), 1.0, 4, dev)
+    base = lin_ref(a, w, b).bfloat16().float()
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res), base + res.float().cpu(), 2**-7, "residual")
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_ERF), F.gelu(base), 2**-7, "gelu erf")
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_TANH), F.gelu(base, approximate="tanh"), 2**-7, "gelu tanh")
+    gate, up = base[:, 0::2], base[:, 1::2]
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_SWIGLU), F.silu(gate).bfloat16().float() * up, 2**-7, "swiglu")
+    # in-place residual (out aliases residual), as the model uses it
+    x = res.clone()
+    ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+    close(x, base + res.float().cpu(), 2**-7, "residual in place")
+    pos = rnd((103, N), 1.0, 5, dev)
+    idx = torch.arange(M) % 103
+    close(ops.gemm(a, w, b, pos=pos), base + pos.float().cpu()[idx], 2**-7, "pos")
+
+
+def test_gemm_row_maps(ops, dev):
+    M, N, K = 400, 512, 256
+    a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
+    plain = ops.gemm(a, w, b)
+    perm = torch.randperm(M, generator=torch.Generator().manual_seed(1)).int().to(dev)
+    assert torch.equal(ops.gemm(a, w, b, a_rows=perm), plain[perm.long()])   # gather is bit-exact data movement
+    scat = ops.gemm(a, w, b, c_rows=perm)
+    ref = torch.empty_like(plain)
+    ref[perm.long()] = plain
+    assert torch.equal(scat, ref)
+
+
+def test_gemm_linearity_at_full_size(ops, dev):
+    # size-independent property at the benchmark's shape: f(a1 + a2) == f(a1) + f(a2) up to bf16 rounding
+    M, N, K = 8192, 3840, 1280
+    a1, a2, w = rnd((M, K), 1.0, 1, dev), rnd((M, K), 1.0, 2, dev), rnd((N, K), 0.02, 3, dev)
+    s = (a1.float() + a2.float()).bfloat16()
+    y = ops.gemm(s, w, None).float()
+    y12 = ops.gemm(a1, w, None).float() + ops.gemm(a2, w, None).float()
+    assert (y - y12).abs().max().item() <= 2**-5 * y.abs().max().item()
+    # and a sampled check against the oracle's F.linear
+    rows = torch.arange(0, M, 257, device=dev)
+    close(y[rows], lin_ref(s[rows], w, None), 2**-7, "sampled rows")
+
+
+def test_gemm_fp8_weights(ops, dev):
+    M, N, K = 300, 1280, 1280
+    a, b = rnd((M, K), 1.0, 1, dev), rnd((N,), 0.02, 3, dev)
+    w = torch.randn(N, K, generator=torch.Generator().manual_seed(2)) * 0.02
+    scale = w.abs().amax(dim=1) / 448.0
+    q = (w / scale[:, None]).to(torch.float8_e4m3fn)
+    ref = a.float().cpu() @ (q.float() * scale[:, None]).t() + b.float().cpu()
+    got = ops.gemm(a, q.to(dev), b, w_scale=scale.to(dev))
+    close(got, ref, 2**-7, "fp8 weights")
+    # every finite e4m3 byte decodes exactly: one-hot activations read the weight matrix back
+    bytes_ = torch.tensor([v for v in range(256) if (v & 0x7F) != 0x7F], dtype=torch.uint8)
+    K2 = 256
+    wq = torch.zeros((16, K2), dtype=torch.uint8)
+    wq[:, : bytes_.numel()] = bytes_
+    eye = torch.eye(K2).bfloat16().to(dev)
+    dec = ops.gemm(eye, wq.view(torch.float8_e4m3fn).to(dev), None, w_scale=torch.ones(16, device=dev))
+    assert torch.equal(dec.float().cpu(), wq.view(torch.float8_e4m3fn).float().t())
+
+
+def test_gemm_rejects_bad_shapes(ops, dev):
+    a, w = rnd((8, 60), dev=dev), rnd((8, 60), dev=dev)
+    with pytest.raises(ValueError):
+        ops.gemm(a, w, None)   # K not a multiple of 8
+    with pytest.raises(ValueError):
+        ops.gemm(a.float(), w, None)
+
+
+# --------------------------------------------------------------------------------------- attention
+def attn_ref(qkv, cu, nh, d, cos_sin=None):
+    L = qkv.shape[0]
+    q, k, v = (t.reshape(L, nh, d) for t in qkv.cpu().chunk(3, dim=-1))
+    if cos_sin is not None:
+        ang = cos_sin
+        q, k = oq.apply_rotary(q, ang), oq.apply_rotary(k, ang)
+    return oq.varlen_attention(q, k, v, cu, d**-0.5).reshape(L, nh * d)
+
+
+@pytest.mark.parametrize("d,cu", [
+    (80, [0, 64, 128, 176, 192, 256]),      # windows, ragged edges (48 and 16 rows)
+    (80, [0, 1024, 1324]),                  # full segments, partial last tile
+    (80, [0, 1, 3, 70, 200]),               # tiny segments
+    (72, [0, 500, 1000]),                   # SigLIP head dim (zero padded in LDS)
+    (72, [0, 64]),
+    (64, [0, 130]),
+])
+def test_attention(ops, dev, d, cu):
+    nh, L = 16, cu[-1]
+    qkv = rnd((L, 3 * nh * d), 1.0, 7, dev)
+    plan = ops.attn_plan(np.array(cu, np.int32), dev)
+    H = nh * d
+    got = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], plan, nh, d, d**-0.5)
+    close(got, attn_ref(qkv, cu, nh, d), 2**-6, f"attention d={d} cu={cu}")
+
+
+def test_attention_fused_rotary_and_standalone_rotary(ops, dev):
+    nh, d, cu = 16, 80, [0, 64, 128, 1024 + 128, 1024 + 128 + 37]
+    L = cu[-1]
+    qkv = rnd((L, 3 * nh * d), 1.0, 8, dev)
+    ang = torch.rand(L, 40, generator=torch.Generator().manual_seed(1)) * 60
+    cs = torch.cat([ang.cos(), ang.sin()], -1).contiguous().to(dev)
+    plan = ops.attn_plan(np.array(cu, np.int32), dev)
+    H = nh * d
+    ref = attn_ref(qkv, cu, nh, d, ang)
+    got = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], plan, nh, d, d**-0.5, cos_sin=cs)
+    close(got, ref, 2**-6, "fused rotary attention")
+    # standalone rotary kernel: same rounding as the oracle (fp32 math, one bf16 rounding) -> near bit-exact
+    q2 = qkv.clone()
+    ops.rope_qk_(q2, cs, nh, d)
+    qr = oq.apply_rotary(qkv[:, :H].cpu().reshape(L, nh, d), ang).reshape(L, H)
+    kr = oq.apply_rotary(qkv[:, H:2 * H].cpu().reshape(L, nh, d), ang).reshape(L, H)
+    close(q2[:, :H], qr, 2**-8, "rope q")
+    close(q2[:, H:2 * H], kr, 2**-8, "rope k")
+    assert torch.equal(q2[:, 2 * H:], qkv[:, 2 * H:])
+    got2 = ops.attn_varlen(q2[:, :H], q2[:, H:2 * H], q2[:, 2 * H:], plan, nh, d, d**-0.5)
+    close(got2, ref, 2**-6, "rotary then attention")
+
+
+def test_attention_invariants_at_full_size(ops, dev):
+    nh, d, L = 16, 80, 8192
+    H = nh * d
+    qkv = rnd((L, 3 * H), 1.0, 9, dev)
+    for seg in (64, 1024):
+        cu = np.arange(0, L + 1, seg, dtype=np.int32)
+        plan = ops.attn_plan(cu, dev)
+        base = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], plan, nh, d, d**-0.5)
+        # segments are independent: perturbing segment 0 leaves every other segment bit-identical
+        q2 = qkv.clone()
+        q2[:seg] += 1.0
+        pert = ops.attn_varlen(q2[:, :H], q2[:, H:2 * H], q2[:, 2 * H:], plan, nh, d, d**-0.5)
+        assert torch.equal(pert[seg:], base[seg:]) and not torch.equal(pert[:seg], base[:seg])
+        # uniform V -> output equals V
+        q3 = qkv.clone()
+        q3[:, 2 * H:] = 0.75
+        out = ops.attn_varlen(q3[:, :H], q3[:, H:2 * H], q3[:, 2 * H:], plan, nh, d, d**-0.5)
+        assert (out.float() - 0.75).abs().max().item() <= 2**-8
+        # sampled segments against the oracle
+        s0 = (L // seg - 1) * seg
+        ref = attn_ref(qkv[s0:], [0, seg], nh, d)
+        close(base[s0:], ref, 2**-6, f"last segment of {seg}")
+    # one-token segments return V exactly
+    cu = np.arange(0, 257, dtype=np.int32)
+    plan = ops.attn_plan(cu, dev)
+    out = ops.attn_varlen(qkv[:256, :H], qkv[:256, H:2 * H], qkv[:256, 2 * H:], plan, nh, d, d**-0.5)
+    assert torch.equal(out, qkv[:256, 2 * H:])

@@ -1,0 +1,84 @@
+"""Host-side mirror of the Eric model interface (CPU only): names, registry, error behaviour."""
+
+import importlib
+
+import pytest
+import torch
+
+from cornserve_amd import synth
+from cornserve_amd.eric.api import Modality
+from cornserve_amd.eric.models import base, registry
+from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
+from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
+
+
+def test_registry_resolves_like_the_reference_loader():
+    for model_type in ("qwen2_5_vl", "gemma3"):
+        entry = registry.MODEL_REGISTRY[model_type]
+        module = importlib.import_module(f"cornserve_amd.eric.models.{entry.module}")
+        cls = getattr(module, entry.class_name)
+        assert issubclass(cls, base.EricModel)
+        assert issubclass(module.ModalityProcessor, base.BaseModalityProcessor)
+    with pytest.raises(ValueError):
+        registry.RegistryEntry("m", "C", "adapter", registry.ViTResolutionType.FIXED,
+                               registry.WeightInfo(required_prefixes=["x."]), {})
+
+
+def test_qwen_state_dict_names_and_properties():
+    cfg = synth.qwen_vision_config(depth=2, fullatt_block_indexes=(1,))
+    with torch.device("meta"):
+        model = Qwen2_5_VisionTransformer(cfg)
+    names = set(model.state_dict().keys())
+    assert names == set(synth.qwen_state_dict(cfg).keys())
+    expect = {"patch_embed.proj.weight", "blocks.0.norm1.weight", "blocks.1.attn.qkv.bias", "blocks.0.mlp.down_proj.weight",
+              "merger.ln_q.weight", "merger.mlp.0.weight", "merger.mlp.2.bias"}
+    assert expect <= names
+    assert model.state_dict()["patch_embed.proj.weight"].shape == (1280, 3, 2, 14, 14)
+    assert model.chunk_shape == (1, 3584)
+    assert model.device.type == "meta"
+
+
+def test_qwen_loads_checkpoint_names_strictly():
+    cfg = synth.qwen_vision_config(depth=1, fullatt_block_indexes=(0,))
+    model = Qwen2_5_VisionTransformer(cfg)
+    sd = synth.qwen_state_dict(cfg, seed=0)
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys
+    assert torch.equal(model.blocks[0].attn.qkv.weight, sd["blocks.0.attn.qkv.weight"])
+
+
+def test_qwen_errors():
+    cfg = synth.qwen_vision_config(depth=1, fullatt_block_indexes=(0,))
+    model = Qwen2_5_VisionTransformer(cfg)
+    with pytest.raises(ValueError, match="Unsupported modality"):
+        model(Modality.AUDIO, "", {})
+    px, grid = synth.qwen_inputs([(1, 4, 4)])
+    # fp32 on the CPU: the kernels have no CPU path and must say so instead of silently falling back
+    with pytest.raises(RuntimeError, match="no CPU path"):
+        model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    with pytest.raises(ValueError):
+        Qwen2_5_VisionTransformer(cfg, weight_format="int4")
+
+
+def test_gemma3_names_adapters_and_errors():
+    cfg = synth.gemma3_config(num_hidden_layers=1, image_size=56, text_hidden=64, mm_tokens_per_image=4)
+    model = Gemma3VisionEncoder(cfg)
+    sd = synth.gemma3_state_dict(cfg, seed=0)
+    synth.load_gemma3(model, sd, adapter_name="google/gemma-3-4b-it")
+    assert model.chunk_shape == (1, 4, 256)
+    assert set(model.state_dict().keys()) == {k for k in sd if k.startswith("vision_tower.")}
+    adapter = model.multi_modal_projector.adapters["google/gemma-3-4b-it"]
+    assert set(adapter.state_dict().keys()) == {"mm_input_projection_weight", "mm_soft_emb_norm.weight"}
+    px, crops = synth.gemma3_inputs(1, 56)
+    with pytest.raises(ValueError, match="Unsupported modality"):
+        model(Modality.VIDEO, "google/gemma-3-4b-it", {"pixel_values": px, "num_crops": crops})
+    with pytest.raises(ValueError, match="Adapter name"):
+        model(Modality.IMAGE, None, {"pixel_values": px, "num_crops": crops})
+    with pytest.raises(AssertionError):
+        model(Modality.IMAGE, "google/gemma-3-4b-it", {"pixel_values": [torch.zeros(1, 3, 28, 28)], "num_crops": crops})
+    with pytest.raises(ValueError, match="not found"):
+        model.multi_modal_projector("nope", torch.zeros(1))
+
+
+def test_modality_is_a_str_enum():
+    assert Modality.IMAGE == "image" and str(Modality.VIDEO) == "video" and Modality("audio") is Modality.AUDIO

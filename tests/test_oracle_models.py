@@ -1,0 +1,108 @@
+"""Pins oracle/qwen2_5_vl.py and oracle/gemma3.py (CPU only).
+
+  * committed golden samples written from the Hugging Face implementations (the reference's own test oracle)
+    on the same seeded weights and inputs -- an fp32-vs-fp32 comparison, so the tolerance is tight;
+  * closed forms / special cases of the pieces: rotary at angle 0 is the identity and preserves the norm of
+    each (j, j+d/2) pair; a one-token segment returns V; uniform V returns V; segments are independent;
+    RMSNorm of a constant row; conv-as-linear identity for the patch embed.
+"""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from cornserve_amd import synth
+from oracle import gemma3 as og
+from oracle import qwen2_5_vl as oq
+
+
+def test_qwen_cfg1_against_golden(golden_dir):
+    gold = np.load(golden_dir / "qwen2_5_vl_cfg1.npz")
+    cfg = synth.qwen_vision_config(depth=4, fullatt_block_indexes=(3,))
+    ocfg = oq.QwenVisionConfig(depth=4, fullatt_block_indexes=[3])
+    sd = synth.qwen_state_dict(cfg, seed=int(gold["seed"]))
+    px, grid = synth.qwen_inputs([(1, 32, 32)], seed=int(gold["seed"]))
+    out = oq.forward(sd, ocfg, px, grid, dtype=torch.float32)
+    assert len(out) == 1 and out[0].shape == (256, 3584)
+    o = out[0].numpy()
+    scale = np.abs(gold["sample"]).max()
+    assert np.abs(o[:, ::16] - gold["sample"]).max() <= 2e-4 * scale
+    assert np.allclose(np.linalg.norm(o.astype(np.float64), axis=1), gold["row_l2"], rtol=1e-4)
+    assert abs(np.abs(o.astype(np.float64)).sum() - float(gold["abs_total"])) <= 1e-4 * float(gold["abs_total"])
+
+
+def test_gemma3_small_against_golden(golden_dir):
+    gold = np.load(golden_dir / "gemma3_small.npz")
+    cfg = synth.gemma3_config(num_hidden_layers=2, image_size=224, text_hidden=640, mm_tokens_per_image=16)
+    ocfg = og.SiglipConfig(num_hidden_layers=2, image_size=224, mm_tokens_per_image=16, text_hidden_size=640)
+    sd = synth.gemma3_state_dict(cfg, seed=int(gold["seed"]))
+    px, crops = synth.gemma3_inputs(2, 224, seed=int(gold["seed"]))
+    feats = og.vision_tower(sd, ocfg, torch.cat(px))
+    fs = gold["feats_sample"]
+    assert np.abs(feats.numpy()[:, ::8, ::8] - fs).max() <= 2e-4 * np.abs(fs).max()
+    out = og.forward(sd, ocfg, px, crops)
+    assert len(out) == 2 and out[0].shape == (16, 640)
+    got = torch.stack(out).numpy()
+    assert np.abs(got - gold["out"]).max() <= 2e-4 * np.abs(gold["out"]).max()
+
+
+def test_rotary_special_cases():
+    torch.manual_seed(0)
+    t = torch.randn(7, 3, 80)
+    assert torch.equal(oq.apply_rotary(t, torch.zeros(7, 40)), t)
+    fr = torch.rand(7, 40) * 6
+    r = oq.apply_rotary(t, fr)
+    n0 = t[..., :40] ** 2 + t[..., 40:] ** 2
+    n1 = r[..., :40] ** 2 + r[..., 40:] ** 2
+    assert torch.allclose(n0, n1, atol=1e-5)
+    # quarter turn: (x1, x2) -> (-x2, x1)
+    q = oq.apply_rotary(t, torch.full((7, 40), np.pi / 2))
+    assert torch.allclose(q[..., :40], -t[..., 40:], atol=1e-6) and torch.allclose(q[..., 40:], t[..., :40], atol=1e-6)
+
+
+def test_attention_special_cases():
+    torch.manual_seed(0)
+    q, k, v = torch.randn(3, 10, 4, 16).unbind(0)
+    one = oq.varlen_attention(q, k, v, list(range(11)), 0.25)
+    assert torch.allclose(one, v, atol=1e-6)  # one-token segments return V
+    vu = torch.ones(10, 4, 16) * 3.0
+    assert torch.allclose(oq.varlen_attention(q, k, vu, [0, 4, 10], 0.25), vu, atol=1e-6)
+    base = oq.varlen_attention(q, k, v, [0, 4, 10], 0.25)
+    k2, v2 = k.clone(), v.clone()
+    k2[4:] += 1.0
+    v2[4:] -= 2.0
+    pert = oq.varlen_attention(q, k2, v2, [0, 4, 10], 0.25)
+    assert torch.equal(pert[:4], base[:4]) and not torch.allclose(pert[4:], base[4:])
+    # against the library routine
+    ref = F.scaled_dot_product_attention(q[:4].transpose(0, 1), k[:4].transpose(0, 1), v[:4].transpose(0, 1), scale=0.25)
+    assert torch.allclose(base[:4], ref.transpose(0, 1), atol=1e-6)
+
+
+def test_norms():
+    x = torch.full((2, 8), 3.0)
+    w = torch.arange(8, dtype=torch.float)
+    assert torch.allclose(oq.rms_norm(x, w, 0.0), w.expand(2, 8))
+    assert torch.allclose(og.gemma_rms_norm(x, w, 0.0), (1 + w).expand(2, 8))
+    y = torch.randn(5, 32)
+    assert torch.allclose(oq.rms_norm(y, torch.ones(32), 1e-6), F.rms_norm(y, (32,), eps=1e-6), atol=1e-6)
+
+
+def test_patch_embed_is_a_linear_map():
+    cfg = synth.qwen_vision_config(depth=0)
+    w = synth.normal(3, "w", (1280, 3, 2, 14, 14), 0.02)
+    x = synth.normal(3, "x", (16, 1176))
+    conv = F.conv3d(x.view(16, 3, 2, 14, 14), w, stride=(2, 14, 14)).view(16, 1280)
+    assert torch.allclose(conv, x @ w.view(1280, -1).t(), atol=1e-5)
+    assert cfg.vision_config.hidden_size == 1280
+
+
+def test_bf16_stepwise_close_to_fp32():
+    cfg = synth.qwen_vision_config(depth=2, fullatt_block_indexes=(1,))
+    ocfg = oq.QwenVisionConfig(depth=2, fullatt_block_indexes=[1])
+    sd = synth.qwen_state_dict(cfg, seed=5)
+    px, grid = synth.qwen_inputs([(1, 8, 12)], seed=5)
+    a = oq.forward(sd, ocfg, px, grid, dtype=torch.float32)[0]
+    b = oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)[0].float()
+    cos = F.cosine_similarity(a.flatten(), b.flatten(), dim=0).item()
+    assert cos > 0.999
