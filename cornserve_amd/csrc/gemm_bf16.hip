@@ -23,24 +23,16 @@
 // optional gather of A rows (a_rows) and scatter of C rows (c_rows) used to fuse the window permutation
 // (qwen2_5_vl.py:438-440) and its inverse (:478-479) into the neighbouring GEMMs, and an optional second
 // residual-like addend indexed by (row % pos_period) for the SigLIP position embedding (siglip.py:100).
-#include "common.h"
+#include "gemm_common.h"
+
+int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled);
 
 namespace {
 
-constexpr int BK = 64;           // K step (bf16 elements): 128 bytes per tile row = 8 chunks of 16 B
+using namespace csgemm;
 constexpr int NTHREADS = 512;    // 8 waves
 constexpr int WAVES_M = 2;
 constexpr int WAVES_N = 4;
-
-CS_DEVICE int swz(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
-
-CS_DEVICE float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
-CS_DEVICE float gelu_tanh(float x) {
-  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-  float inner = k0 * (x + k1 * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(inner));
-}
-CS_DEVICE float silu(float x) { return x / (1.0f + __expf(-x)); }
 
 // 16 fp8-e4m3 (OCP) values -> 16 bf16.  Conversion is exact: every e4m3 value is representable in bf16.
 CS_DEVICE void fp8x16_to_bf16(const i32x4_t& in, bf16x8_t& lo, bf16x8_t& hi) {
@@ -65,10 +57,6 @@ template <int BM, int BN, int EPI, bool W_FP8>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const bf16_t* const pA = (const bf16_t*)p.A;
-  const bf16_t* const pBias = (const bf16_t*)p.bias;
-  const bf16_t* const pRes = (const bf16_t*)p.residual;
-  const bf16_t* const pPos = (const bf16_t*)p.pos;
-  bf16_t* const pC = (bf16_t*)p.C;
   constexpr int A_BYTES = BM * BK * 2;
   constexpr int W_BYTES = BN * BK * 2;
   constexpr int STAGE = A_BYTES + W_BYTES;
@@ -205,64 +193,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const CsGemmArgs p) {
     __syncthreads();
   }
 
-  // ---- epilogue.  acc[i][j][4g+q] = C[m][n], m = m0+wm*WTM+i*32+lane%32,
-  //      n = n0+wn*WTN+j*32+8g+4*(lane/32)+q.
-#pragma unroll
-  for (int i = 0; i < MT; ++i) {
-    const int m = m0 + wm * WTM + i * 32 + frag_row;
-    if (m >= p.M) continue;
-    const int64_t crow = p.c_rows ? (int64_t)p.c_rows[m] : (int64_t)m;
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int n = n0 + wn * WTN + j * 32 + 8 * g + 4 * frag_half;
-        if (n >= p.N) continue;
-        float v[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] = acc[i][j][4 * g + q];
-        if (p.w_scale) {
-          const f32x4_t s = *(const f32x4_t*)(p.w_scale + n);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] *= s[q];
-        }
-        if (p.bias) {
-          const bf16x4_t b = *(const bf16x4_t*)(pBias + n);
-#pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] += bf2f(b[q]);
-        }
-        if (EPI == CS_EPI_SWIGLU) {
-          const float gate0 = rbf(silu(rbf(v[0]))), up0 = rbf(v[1]);
-          const float gate1 = rbf(silu(rbf(v[2]))), up1 = rbf(v[3]);
-          bf16x2_t o;
-          o[0] = f2bf(gate0 * up0);
-          o[1] = f2bf(gate1 * up1);
-          *(bf16x2_t*)(pC + crow * p.ldc + (n >> 1)) = o;
-        } else {
-          if (EPI == CS_EPI_GELU_ERF) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = gelu_erf(rbf(v[q]));
-          } else if (EPI == CS_EPI_GELU_TANH) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = gelu_tanh(rbf(v[q]));
-          } else if (EPI == CS_EPI_RESIDUAL) {
-            const bf16x4_t r = *(const bf16x4_t*)(pRes + (int64_t)m * p.ldr + n);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = rbf(v[q]) + bf2f(r[q]);
-          }
-          if (p.pos) {
-            const bf16x4_t r = *(const bf16x4_t*)(pPos + (int64_t)(m % p.pos_period) * p.ldpos + n);
-#pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = rbf(v[q]) + bf2f(r[q]);
-          }
-          bf16x4_t o;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) o[q] = f2bf(v[q]);
-          *(bf16x4_t*)(pC + crow * p.ldc + n) = o;
-        }
-      }
-    }
-  }
+  csgemm::epilogue<EPI, MT, NT>(p, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
 template <int BM, int BN, int EPI, bool W_FP8>
@@ -313,6 +244,12 @@ extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
   if (((uintptr_t)a.C | (uintptr_t)a.bias | (uintptr_t)a.residual | (uintptr_t)a.pos) & 7) return CS_ERR_INVALID_ARG;
   if ((uintptr_t)a.w_scale & 15) return CS_ERR_INVALID_ARG;
 
+  // Fast path (direct-to-LDS pipeline) when the shape allows it; otherwise the general kernel below.
+  {
+    bool handled = false;
+    const int st = cs_gemm_fast(a, stream, &handled);
+    if (handled) return st;
+  }
   // Tile choice: 256x256 when that fills the chip's 256 CUs reasonably, else smaller tiles for more workgroups.
   const int64_t t256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
   const bool small = t256 < 192;
