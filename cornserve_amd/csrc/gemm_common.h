@@ -20,7 +20,8 @@ CS_DEVICE float gelu_tanh(float x) {
   float inner = k0 * (x + k1 * x * x * x);
   return 0.5f * x * (1.0f + tanhf(inner));
 }
-CS_DEVICE float silu(float x) { return x / (1.0f + __expf(-x)); }
+// x * sigmoid(x) with the hardware reciprocal (1 ulp) instead of an IEEE division sequence.
+CS_DEVICE float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
 
 // Fused epilogue for one wave's accumulators.  acc[i][j][4g+q] = C[m][n] with
