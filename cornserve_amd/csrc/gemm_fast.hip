@@ -153,8 +153,15 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
     const char* base = smem + stage * STAGE;
 #pragma unroll
     for (int j = 0; j < NT; ++j) wf[b][j] = *(const bf16x8_t*)(base + w_off[ks] + j * 4 * 128);
+#ifdef CS_EXP_SKIP_X  // experiment: issue only half of the activation-fragment reads (results are wrong)
+#pragma unroll
+    for (int i = 0; i < MT / 2; ++i) xf[b][i] = *(const bf16x8_t*)(base + x_off[ks] + i * 16 * 128);
+#pragma unroll
+    for (int i = MT / 2; i < MT; ++i) xf[b][i] = xf[b][i - MT / 2];
+#else
 #pragma unroll
     for (int i = 0; i < MT; ++i) xf[b][i] = *(const bf16x8_t*)(base + x_off[ks] + i * 16 * 128);
+#endif
   };
   auto mfmas = [&](int b) {
 #pragma unroll
