@@ -15,10 +15,11 @@ CS_DEVICE int swz_key(int row) { return (row ^ (row >> 3)) & 7; }
 CS_DEVICE int swz(int row, int chunk) { return row * 128 + ((chunk ^ swz_key(row)) << 4); }
 
 CS_DEVICE float gelu_erf(float x) { return 0.5f * x * (1.0f + erff(x * 0.70710678118654752440f)); }
+// 0.5 x (1 + tanh(u)) == x * sigmoid(2u): one exponential and one hardware reciprocal instead of tanhf.
 CS_DEVICE float gelu_tanh(float x) {
   const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-  float inner = k0 * (x + k1 * x * x * x);
-  return 0.5f * x * (1.0f + tanhf(inner));
+  const float u = k0 * (x + k1 * x * x * x);
+  return x * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
 }
 // x * sigmoid(x) with the hardware reciprocal (1 ulp) instead of an IEEE division sequence.
 CS_DEVICE float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }

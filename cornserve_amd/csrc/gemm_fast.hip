@@ -420,5 +420,36 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   const double c160 = rounds_cost(a.M, a.N, 256, 160) * 1.15;  // narrower tiles: more LDS and L2 traffic per FLOP
   static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160" or "256"
   if (force ? force[0] == '1' : c160 < c256) return dispatch_epi<256, 160, 4, 2>(a, stream);
+  // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
+  // that fill whole rounds go to one launch and the remaining columns to a second launch with 256x128
+  // tiles (twice as many workgroups, half as long).  The two launches write disjoint column ranges of C.
+  if (!force) {
+    const int tm = (a.M + 255) / 256, tn = (a.N + 255) / 256;
+    double best = c256;
+    int best_cols = 0;
+    for (int c = tn - 1; c >= 1 && c >= tn - 12; --c) {
+      const int rest = a.N - c * 256;
+      const double cost = rounds_cost(a.M, c * 256, 256, 256) + rounds_cost(a.M, rest, 256, 128) * 1.10;
+      if (cost < best - 0.05) {
+        best = cost;
+        best_cols = c;
+      }
+    }
+    (void)tm;
+    if (best_cols > 0) {
+      const int n1 = best_cols * 256;
+      CsGemmArgs lo = a, hi = a;
+      lo.N = n1;
+      hi.N = a.N - n1;
+      hi.W = (const char*)a.W + (int64_t)n1 * a.ldw * 2;
+      if (a.bias) hi.bias = (const char*)a.bias + (int64_t)n1 * 2;
+      if (a.residual) hi.residual = (const char*)a.residual + (int64_t)n1 * 2;
+      if (a.pos) hi.pos = (const char*)a.pos + (int64_t)n1 * 2;
+      hi.C = (char*)a.C + (int64_t)(a.epilogue == CS_EPI_SWIGLU ? n1 / 2 : n1) * 2;
+      const int st = dispatch_epi<256, 256, 2, 4>(lo, stream);
+      if (st != CS_OK) return st;
+      return dispatch_epi<256, 128, 4, 2>(hi, stream);
+    }
+  }
   return dispatch_epi<256, 256, 2, 4>(a, stream);
 }
