@@ -231,6 +231,276 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
   }
 }
 
+// Full-attention variant (segments longer than 64 rows): 4 waves x 32 query rows, K/V tiles double-buffered.
+// The global loads of tile t+1 are issued before the matrix-core work on tile t and land in registers;
+// rotary (K) and the transpose (V) are applied when those registers are written to the other LDS buffer
+// after the compute, so one barrier per tile is enough and memory latency hides behind the MFMAs.  The Q
+// tile shares its LDS region with the second K/V buffer: Q is only needed until its fragments are in
+// registers.
+template <int D, bool ROPE>
+__global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
+  constexpr int NT = 256, BQ = 128;
+  constexpr int KS = (D + 15) / 16, DT = (D + 31) / 32, DC = D / 8, DKC = KS * 2;
+  constexpr int RS = (DKC | 1) * 16;
+  constexpr int HC = DC / 2;
+  static_assert(D % 8 == 0 && D <= 96, "head dim");
+  static_assert(!ROPE || D % 16 == 0, "rotary needs an even number of chunks per half");
+  constexpr int K_BYTES = BKV * RS, V_BYTES = DT * 32 * VT_STRIDE * 2, Q_BYTES = BQ * RS;
+  constexpr int REGION_B = (K_BYTES + V_BYTES) > Q_BYTES ? (K_BYTES + V_BYTES) : Q_BYTES;
+  __shared__ __attribute__((aligned(16))) char lds[K_BYTES + V_BYTES + REGION_B];
+  auto k_buf = [&](int b) -> char* { return lds + b * (K_BYTES + V_BYTES); };
+  auto v_buf = [&](int b) -> bf16_t* { return (bf16_t*)(lds + b * (K_BYTES + V_BYTES) + K_BYTES); };
+  char* const q_lds = lds + K_BYTES + V_BYTES;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int fr = lane & 31, hf = lane >> 5;
+  const int head = blockIdx.y;
+  const int seg_start = a.work[blockIdx.x * 4 + 0];
+  const int seg_end = a.work[blockIdx.x * 4 + 1];
+  const int q0 = a.work[blockIdx.x * 4 + 2];
+  const int nq = a.work[blockIdx.x * 4 + 3];
+  const int64_t hoff = (int64_t)head * D;
+  const int seg_len = seg_end - seg_start;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const f32x4_t zero4 = {0, 0, 0, 0};
+
+  // ---- register staging of one K/V tile
+  constexpr int K_ITEMS = ROPE ? BKV * HC : BKV * DC;
+  constexpr int K_PER = (K_ITEMS + NT - 1) / NT;
+  constexpr int V_ITEMS = (BKV / 2) * DC;
+  constexpr int V_PER = (V_ITEMS + NT - 1) / NT;
+  bf16x8_t kx1[K_PER], kx2[ROPE ? K_PER : 1];
+  f32x4_t kc0[ROPE ? K_PER : 1], kc1[ROPE ? K_PER : 1], ks0[ROPE ? K_PER : 1], ks1[ROPE ? K_PER : 1];
+  bf16x8_t vx0[V_PER], vx1[V_PER];
+
+  auto gload_tile = [&](int kv0, int nvalid) {
+#pragma unroll
+    for (int u = 0; u < K_PER; ++u) {
+      const int i = tid + u * NT;
+      constexpr int PER_ROW = ROPE ? HC : DC;
+      const int r = i / PER_ROW, jc = i - r * PER_ROW;
+      const bool ok = i < K_ITEMS && r < nvalid;
+      const int64_t g = seg_start + kv0 + (ok ? r : 0);
+      const bf16_t* p = a.k + g * a.ld + hoff + jc * 8;
+      kx1[u] = ok ? *(const bf16x8_t*)p : zero8;
+      if (ROPE) {
+        kx2[u] = ok ? *(const bf16x8_t*)(p + D / 2) : zero8;
+        const float* cs = a.cos_sin + g * D + jc * 8;
+        kc0[u] = ok ? *(const f32x4_t*)cs : zero4;
+        kc1[u] = ok ? *(const f32x4_t*)(cs + 4) : zero4;
+        ks0[u] = ok ? *(const f32x4_t*)(cs + D / 2) : zero4;
+        ks1[u] = ok ? *(const f32x4_t*)(cs + D / 2 + 4) : zero4;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < V_PER; ++u) {
+      const int i = tid + u * NT;
+      const int kp = i / DC, c = i - kp * DC;   // consecutive lanes: consecutive chunks of one key pair
+      const int r0 = 2 * kp;
+      const bool ok0 = i < V_ITEMS && r0 < nvalid, ok1 = i < V_ITEMS && r0 + 1 < nvalid;
+      const bf16_t* p = a.v + (int64_t)(seg_start + kv0 + (ok0 ? r0 : 0)) * a.ld + hoff + c * 8;
+      vx0[u] = ok0 ? *(const bf16x8_t*)p : zero8;
+      vx1[u] = ok1 ? *(const bf16x8_t*)(p + a.ld) : zero8;
+    }
+  };
+  auto lstore_tile = [&](int b) {
+    char* kd = k_buf(b);
+    bf16_t* vd = v_buf(b);
+#pragma unroll
+    for (int u = 0; u < K_PER; ++u) {
+      const int i = tid + u * NT;
+      if (i < K_ITEMS) {
+        constexpr int PER_ROW = ROPE ? HC : DC;
+        const int r = i / PER_ROW, jc = i - r * PER_ROW;
+        if (ROPE) {
+          bf16x8_t o1, o2;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float co = e < 4 ? kc0[u][e] : kc1[u][e - 4];
+            const float si = e < 4 ? ks0[u][e] : ks1[u][e - 4];
+            const float xa = bf2f(kx1[u][e]), xb = bf2f(kx2[u][e]);
+            o1[e] = f2bf(xa * co - xb * si);
+            o2[e] = f2bf(xa * si + xb * co);
+          }
+          *(bf16x8_t*)(kd + r * RS + jc * 16) = o1;
+          *(bf16x8_t*)(kd + r * RS + (jc + HC) * 16) = o2;
+        } else {
+          *(bf16x8_t*)(kd + r * RS + jc * 16) = kx1[u];
+        }
+      }
+    }
+    if (!ROPE && DKC > DC) {  // zero the pad chunks of the K rows (head dims that are not multiples of 16)
+      for (int i = tid; i < BKV * (DKC - DC); i += NT) {
+        const int r = i / (DKC - DC), c = DC + i % (DKC - DC);
+        *(bf16x8_t*)(kd + r * RS + c * 16) = zero8;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < V_PER; ++u) {
+      const int i = tid + u * NT;
+      if (i < V_ITEMS) {
+        const int kp = i / DC, c = i - kp * DC;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          bf16x2_t pr;
+          pr[0] = vx0[u][e];
+          pr[1] = vx1[u][e];
+          *(bf16x2_t*)(vd + (c * 8 + e) * VT_STRIDE + 2 * kp) = pr;
+        }
+      }
+    }
+  };
+
+  // ---- prologue: Q -> LDS (rotated), tile 0 -> LDS buffer 0
+  gload_tile(0, min(BKV, seg_len));
+  {
+    if (ROPE) {
+      for (int i = tid; i < BQ * HC; i += NT) {
+        const int r = i / HC, jc = i - r * HC;
+        bf16x8_t o1 = zero8, o2 = zero8;
+        if (r < nq) {
+          const int64_t g = q0 + r;
+          const bf16_t* p = a.q + g * a.ld + hoff + jc * 8;
+          const bf16x8_t x1 = *(const bf16x8_t*)p;
+          const bf16x8_t x2 = *(const bf16x8_t*)(p + D / 2);
+          const float* cs = a.cos_sin + g * D + jc * 8;
+          const f32x4_t c0 = *(const f32x4_t*)cs, c1 = *(const f32x4_t*)(cs + 4);
+          const f32x4_t s0 = *(const f32x4_t*)(cs + D / 2), s1 = *(const f32x4_t*)(cs + D / 2 + 4);
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float co = e < 4 ? c0[e] : c1[e - 4];
+            const float si = e < 4 ? s0[e] : s1[e - 4];
+            const float xa = bf2f(x1[e]), xb = bf2f(x2[e]);
+            o1[e] = f2bf(xa * co - xb * si);
+            o2[e] = f2bf(xa * si + xb * co);
+          }
+        }
+        *(bf16x8_t*)(q_lds + r * RS + jc * 16) = o1;
+        *(bf16x8_t*)(q_lds + r * RS + (jc + HC) * 16) = o2;
+      }
+    } else {
+      for (int i = tid; i < BQ * DKC; i += NT) {
+        const int r = i / DKC, c = i - r * DKC;
+        bf16x8_t x = zero8;
+        if (r < nq && c < DC) x = *(const bf16x8_t*)(a.q + (int64_t)(q0 + r) * a.ld + hoff + c * 8);
+        *(bf16x8_t*)(q_lds + r * RS + c * 16) = x;
+      }
+    }
+  }
+  lstore_tile(0);
+  __syncthreads();
+  bf16x8_t qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8_t*)(q_lds + (wave * 32 + fr) * RS + (2 * ks + hf) * 16);
+  __syncthreads();  // every wave holds its Q fragments: the Q region may now become K/V buffer 1
+
+  f32x16_t oacc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const bool wave_active = wave * 32 < nq;
+  const float sl2 = a.scale_log2e;
+
+  int buf = 0;
+  for (int kv0 = 0; kv0 < seg_len; kv0 += BKV, buf ^= 1) {
+    const int nvalid = min(BKV, seg_len - kv0);
+    const bool more = kv0 + BKV < seg_len;
+    if (more) gload_tile(kv0 + BKV, min(BKV, seg_len - kv0 - BKV));
+    if (wave_active) {
+      const char* kd = k_buf(buf);
+      const bf16_t* vd = v_buf(buf);
+      f32x16_t sacc[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[kt][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t kf = *(const bf16x8_t*)(kd + (kt * 32 + fr) * RS + (2 * ks + hf) * 16);
+          sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kt], 0, 0, 0);
+        }
+      }
+      if (nvalid < BKV) {  // only the last tile of a segment can be partial
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+            if (key >= nvalid) sacc[kt][r] = -INFINITY;
+          }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run, mx);
+      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
+      const float mb = m_new * sl2;
+      float psum = 0.f;
+      bf16x8_t pf[2][2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * sl2 - mb);
+          psum += pv;
+          pf[kt][r >> 3][r & 7] = f2bf(pv);
+        }
+      psum += __shfl_xor(psum, 32, 64);
+      l_run = l_run * alpha + psum;
+      if (__any(m_new != m_run)) {  // the running maximum moved for some query of this wave: rescale O
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+      }
+      m_run = m_new;
+#pragma unroll
+      for (int t = 0; t < DT; ++t) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int kk = 0; kk < 2; ++kk) {
+            const bf16_t* vp = vd + (t * 32 + fr) * VT_STRIDE + kt * 32 + 16 * kk + 4 * hf;
+            const bf16x4_t v0 = *(const bf16x4_t*)vp;
+            const bf16x4_t v1 = *(const bf16x4_t*)(vp + 8);
+            bf16x8_t vf;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              vf[e] = v0[e];
+              vf[4 + e] = v1[e];
+            }
+            oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][kk], oacc[t], 0, 0, 0);
+          }
+      }
+    }
+    if (more) lstore_tile(buf ^ 1);
+    __syncthreads();
+  }
+
+  const int qi = wave * 32 + fr;
+  if (qi < nq) {
+    const float inv = 1.0f / l_run;
+    bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d0 = t * 32 + 8 * g + 4 * hf;
+        if (d0 < D) {
+          bf16x4_t o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
+          *(bf16x4_t*)(orow + d0) = o;
+        }
+      }
+  }
+}
+
 template <int D>
 int launch_attn(const AttnArgs& a, int n_work, int heads, int block_q, bool rope, hipStream_t stream) {
   const dim3 grid(n_work, heads);
@@ -243,10 +513,10 @@ int launch_attn(const AttnArgs& a, int n_work, int heads, int block_q, bool rope
     }
   } else {
     if (rope) {
-      if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_kernel<D, 4, true>), grid, dim3(256), 0, stream, a);
+      if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_full_kernel<D, true>), grid, dim3(256), 0, stream, a);
       else return CS_ERR_UNSUPPORTED;
     } else {
-      hipLaunchKernelGGL((attn_kernel<D, 4, false>), grid, dim3(256), 0, stream, a);
+      hipLaunchKernelGGL((attn_full_kernel<D, false>), grid, dim3(256), 0, stream, a);
     }
   }
   return cs_launch_status();
