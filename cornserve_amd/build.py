@@ -7,6 +7,7 @@ written next to the sources so that it travels with the tree; nothing is JIT-com
 from __future__ import annotations
 
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -42,11 +43,52 @@ def _hipcc() -> str:
 
 def _run(cmd: list[str]) -> None:
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(line for line in proc.stdout.splitlines() if "packed-fp32-ops" not in line)
+    out = "\n".join(line for line in proc.stdout.splitlines() if "packed-fp32-ops" not in line and "--hip-link" not in line)
     if proc.returncode != 0:
         raise RuntimeError(f"command failed ({proc.returncode}): {' '.join(cmd)}\n{out}")
     if out.strip():
         print(out, file=sys.stderr)
+
+
+# Sources with this marker keep their accumulators in accumulation registers that only inline assembly
+# touches; the compiler does not know they are occupied, so its output is checked after every build.
+HAND_MANAGED_ACC_MARKER = "CS_ALL_ACC_REGS"
+_ACC_REG = re.compile(r"\ba(\d+|\[)")
+
+
+def check_hand_managed_acc_registers(asm_text: str) -> list[str]:
+    """Return the kernels that use inline-assembly accumulation registers AND in which compiler-generated
+    code touches an accumulation register too (a register spill or a staging copy would corrupt the
+    accumulators).  An empty list means the convention holds."""
+    offenders = []
+    for m in re.finditer(r"^(_Z\S+):.*?s_endpgm", asm_text, re.S | re.M):
+        in_asm, uses_inline, outside = False, False, 0
+        for line in m.group(0).splitlines():
+            if "#ASMSTART" in line:
+                in_asm = True
+                continue
+            if "#ASMEND" in line:
+                in_asm = False
+                continue
+            code = line.split(";")[0]
+            if _ACC_REG.search(code):
+                if in_asm:
+                    uses_inline = True
+                else:
+                    outside += 1
+        if uses_inline and outside:
+            offenders.append(f"{m.group(1)}: {outside} compiler-generated accumulation-register references")
+    return offenders
+
+
+def _check_source(hipcc: str, src: Path) -> None:
+    asm = OBJ_DIR / (src.stem + ".gfx950.s")
+    _run([hipcc, *HIPCC_FLAGS, "-S", "--cuda-device-only", str(src), "-o", str(asm)])
+    offenders = check_hand_managed_acc_registers(asm.read_text())
+    asm.unlink()
+    if offenders:
+        raise RuntimeError(f"{src.name}: the compiler used accumulation registers that inline assembly owns:\n  "
+                           + "\n  ".join(offenders))
 
 
 def build_library(force: bool = True, jobs: int = 6) -> Path:
@@ -63,9 +105,11 @@ def build_library(force: bool = True, jobs: int = 6) -> Path:
         objs.append(obj)
         stale = force or not obj.exists() or obj.stat().st_mtime < max(src.stat().st_mtime, newest_hdr)
         if stale:
-            todo.append([hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)])
+            todo.append(lambda cmd=[hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]: _run(cmd))
+            if HAND_MANAGED_ACC_MARKER in src.read_text():
+                todo.append(lambda src=src: _check_source(hipcc, src))
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo) or 1))) as pool:
-        list(pool.map(_run, todo))
+        list(pool.map(lambda job: job(), todo))
     _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)])
     return LIB_PATH
 

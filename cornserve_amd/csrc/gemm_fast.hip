@@ -1,30 +1,38 @@
 // Fast-path bf16 MFMA GEMM for gfx950:  C[M,N] = epilogue(A[M,K] . W[N,K]^T),  K % 64 == 0, bf16 weights.
 //
-// Pipeline.  One 512-thread workgroup (8 waves, 2 per SIMD) owns a BM x BN tile of C and walks K in steps
-// of 64.  Tiles go global -> LDS directly (global_load_lds_dwordx4: each lane fetches 16 bytes and the
-// hardware stores the wave's 64 chunks contiguously at M0 + lane*16), two LDS stages.  The loop is skewed:
-// the single barrier of an iteration sits BEFORE its last k-step, so the first fragments of the next tile
-// are read while the matrix cores work on that last step, and the refill of the stage that was just
-// drained (tile kt+2) is issued right after the barrier and has a full iteration to land.
+// Pipeline.  One workgroup owns a BM x BN tile of C and walks K in steps of 64.  Tiles go global -> LDS
+// directly (buffer_load_dwordx4 ... lds: each lane fetches 16 bytes and the hardware stores the wave's 64
+// chunks contiguously at M0 + lane*16), two LDS stages.  The loop is skewed: the single barrier of an
+// iteration sits BEFORE its last k-step, so the first fragments of the next tile are read while the matrix
+// cores work on that last step, and the refill of the stage that was just drained (tile kt+2) is issued
+// right after the barrier and has a full iteration to land.
+//
+// Two forms share the code.  The 256x256 tile runs with FOUR waves, one per SIMD, 128x128 outputs and all
+// 512 registers per lane: 256 accumulation registers hold the accumulators and are driven by inline
+// assembly in a fixed instruction order (LDS traffic per FLOP is a third lower than with eight waves, and
+// the compiler cannot shuffle or spill the accumulators).  The narrower tiles (256x160, 256x128) run with
+// EIGHT waves, two per SIMD, compiler-scheduled builtins.
 //
 // Matrix cores.  v_mfma_f32_16x16x32_bf16 (k = 32 per instruction: each accumulator register is touched
 // half as often as with the 32x32x16 form).  W rows are the MFMA "A" operand and activation rows the "B"
-// operand, so a lane owns output row m = lane%16 of a 16x16 block.  The W rows that feed fragment j of a
-// wave are PERMUTED: fragment row 4q+r holds W row q*(4*NT) + 4j + r of the wave's WTN = 16*NT rows, which
-// makes the 4*NT accumulator values a lane holds for one output row CONSECUTIVE in n.  The epilogue can
-// therefore read bias/residual and write C in 8/16-byte pieces that tile whole 128-byte lines, with no
-// trip through LDS.
+// operand, so a lane owns output row m = lane%16 of a 16x16 block.  The W rows that feed the fragments of a
+// wave are PERMUTED in groups of G fragments (G = 2 when the wave has an even number of them): fragment j,
+// fragment row 4q+r holds W row (j/G)*16G + q*4G + (j%G)*4 + r of the wave's rows.  The 4G accumulator
+// values a lane holds for one output row and group are then CONSECUTIVE in n, and the four lanes of that
+// output row hold 16G consecutive columns: with G = 2 every store instruction writes 16 bytes per lane and
+// 64 contiguous bytes per output row, with no trip through LDS.
 //
 // LDS layout.  A tile row is 128 bytes = 8 chunks of 16 bytes; logical chunk c of row r lives in slot
 // c ^ key(r).  The LDS has 64 four-byte banks, so a 16-byte-per-lane read is served 16 lanes at a time and
 // is conflict-free when those lanes hit 16 distinct 16-byte groups of a 256-byte span; with 128-byte rows
 // the row parity picks the half and the key must differ across the 8 rows of equal parity.  Activation
-// fragments read 16 consecutive rows (key = (r>>1)&7); W fragments read rows q*(4*NT)+4j+r
+// fragments read 16 consecutive rows (key = (r>>1)&7); W fragments read rows q*4G + r plus a multiple of 4
 // (key = q*2 + ((r>>1)&1)).  Since a direct-to-LDS load fixes the LDS side (lane -> consecutive chunk),
 // the swizzle is applied on the GLOBAL side: the lane that lands in slot s of row r fetches chunk s ^ key(r).
 #include <stdlib.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "gemm_common.h"
 
@@ -32,18 +40,14 @@ namespace {
 
 using namespace csgemm;
 
-constexpr int NTHREADS = 512;  // 8 waves, 2 per SIMD
 constexpr int CS_EPI_BIAS_POS = 100;  // internal: CS_EPI_BIAS plus the (row % pos_period) position addend
 
 // s_waitcnt with only vmcnt set (lgkmcnt/expcnt left at "don't wait"), gfx9 encoding.
 #define CS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 0xF) | (((n) >> 4) << 14)) | 0x0F70)
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void_t;
-typedef const __attribute__((address_space(1))) void global_void_t;
 
-CS_DEVICE void load_chunk_to_lds(const char* gptr, char* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((global_void_t*)gptr, (lds_void_t*)lds_wave_base, 16, 0, 0);
-}
 // Workgroup barrier without the full memory fence of __syncthreads(): the callers order LDS traffic with
 // explicit waits, and the asm statements keep the compiler from moving memory operations across it.
 CS_DEVICE void wg_barrier() {
@@ -59,21 +63,59 @@ __device__ long long* cs_ts_buf;  // [tiles][8]: 4 wall-clock stamps + 4 shader-
 #define CS_TS(slot) do { } while (0)
 #endif
 
+// every accumulation register, as an inline-asm clobber list
+#define CS_ALL_ACC_REGS \
+  "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", \
+  "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", \
+  "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", \
+  "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63", \
+  "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", \
+  "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", \
+  "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", \
+  "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127", \
+  "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", \
+  "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", \
+  "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", \
+  "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", \
+  "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", \
+  "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", \
+  "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", \
+  "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
+
+template <int V>
+using ic = std::integral_constant<int, V>;
+template <class F, int... Is>
+CS_DEVICE void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(ic<Is>{}), ...);
+}
+// f(ic<0>{}), f(ic<1>{}), ... f(ic<N-1>{}): a loop whose index is a constant expression in the body
+template <int N, class F>
+CS_DEVICE void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
-__global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p, const int stagger) {
+__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const CsGemmArgs p, const int stagger) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  static_assert(WAVES_M * WAVES_N == 8, "8 waves");
+  constexpr int NW = WAVES_M * WAVES_N;
+  static_assert(NW == 8 || NW == 4, "8 waves (2 per SIMD, 256 registers each) or 4 waves (1 per SIMD, 512 registers)");
+  static_assert(NW == 8 || (BM / WAVES_M) * (BN / WAVES_N) <= 128 * 128, "the 4-wave form has 256 accumulation registers");
   constexpr int A_BYTES = BM * BK * 2;
   constexpr int W_BYTES = BN * BK * 2;
   constexpr int STAGE = A_BYTES + W_BYTES;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   static_assert(WTM % 16 == 0 && WTN % 16 == 0 && BM % 8 == 0 && BN % 8 == 0, "tile shape");
   constexpr int MT = WTM / 16, NT = WTN / 16;
+  // W fragments come in groups of G: fragment j, fragment row 4q+r holds W row (j/G)*16G + q*4G + (j%G)*4 + r of
+  // the wave's rows, so a lane owns 4G consecutive output columns per group and the four lanes q = 0..3 of
+  // one output row own 16G consecutive columns.
+  constexpr int G = (NT % 2 == 0) ? 2 : NT;
+  auto piece_col = [](int j) { return (j / G) * 16 * G + (j % G) * 4; };  // first column of fragment j's piece
   // Pinning a fine MFMA/LDS interleave costs registers; only tiles whose accumulators and two fragment
   // sets leave room for it use it (the 256x256 tile would spill).
-  constexpr bool ILV = (MT * NT * 4 + (MT + NT) * 8) <= 176;
+  constexpr bool ILV = NW == 4 || (MT * NT * 4 + (MT + NT) * 8) <= 176;
   constexpr int A_BLK = BM / 8, W_BLK = BN / 8;            // 8-row blocks = direct loads per stage
-  constexpr int A_LD = (A_BLK + 7) / 8, W_LD = (W_BLK + 7) / 8;  // per wave
+  constexpr int A_LD = (A_BLK + NW - 1) / NW, W_LD = (W_BLK + NW - 1) / NW;  // per wave
 
   // ---- tile coordinates of virtual block vb in [0, tiles): XCD-aware remap (workgroup i runs on XCD i%8,
   //      and the persistent stride gridDim.x is a multiple of 8, so a workgroup's tiles stay on its XCD),
@@ -92,6 +134,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
     n0 = (within / rows_in_band) * BN;
   };
 
+  if constexpr (NW == 4) asm volatile("" ::: CS_ALL_ACC_REGS);  // accounts a[0:255] to this kernel
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -107,31 +150,41 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
   auto setup_sources = [&](int m0, int n0) {
 #pragma unroll
     for (int j = 0; j < A_LD; ++j) {
-      const int row = (j * 8 + wave) * 8 + l_row;  // tile-local
+      const int row = (j * NW + wave) * 8 + l_row;  // tile-local
       const int key = (row >> 1) & 7;
       const int r = min(m0 + row, p.M - 1);
       a_src[j] = (uint32_t)(((int64_t)r * p.lda + ((l_slot ^ key) << 3)) * 2);
     }
 #pragma unroll
     for (int j = 0; j < W_LD; ++j) {
-      const int row = (j * 8 + wave) * 8 + l_row;
-      const int key = ((((row % WTN) / (4 * NT)) & 3) << 1) | ((row >> 1) & 1);
+      const int row = (j * NW + wave) * 8 + l_row;
+      const int key = ((((row % (16 * G)) / (4 * G)) & 3) << 1) | ((row >> 1) & 1);
       const int r = min(n0 + row, p.N - 1);
       w_src[j] = (uint32_t)(((int64_t)r * p.ldw + ((l_slot ^ key) << 3)) * 2);
     }
   };
-  auto issue_loads = [&](int kt, int stage) {
-    char* As = smem + stage * STAGE;
-    char* Ws = As + A_BYTES;
-    const char* Ak = (const char*)p.A + (int64_t)kt * (BK * 2);
-    const char* Wk = (const char*)p.W + (int64_t)kt * (BK * 2);
-#pragma unroll
-    for (int j = 0; j < A_LD; ++j)
-      if ((A_BLK % 8 == 0) || j * 8 + wave < A_BLK) load_chunk_to_lds(Ak + a_src[j], As + (j * 8 + wave) * 1024);
-#pragma unroll
-    for (int j = 0; j < W_LD; ++j)
-      if ((W_BLK % 8 == 0) || j * 8 + wave < W_BLK) load_chunk_to_lds(Wk + w_src[j], Ws + (j * 8 + wave) * 1024);
+  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void*)p.W, 0, -1, 0x00020000);
+  // Direct loads are buffer loads: a 32-bit per-lane byte offset plus a scalar K offset on a scalar descriptor,
+  // so an address costs one register and no vector arithmetic.
+  auto load_a = [&](int kt, char* lds_dst, uint32_t off) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t*)lds_dst, 16, off, kt * (BK * 2), 0, 0);
   };
+  auto load_w = [&](int kt, char* lds_dst, uint32_t off) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void_t*)lds_dst, 16, off, kt * (BK * 2), 0, 0);
+  };
+  // one direct load of K tile kt into `stage`: IDX < A_LD activation row blocks, then the W row blocks
+  auto issue_one_load = [&](int kt, int stage, auto idx_c) {
+    constexpr int IDX = decltype(idx_c)::value;
+    char* As = smem + stage * STAGE;
+    if constexpr (IDX < A_LD) {
+      if ((A_BLK % NW == 0) || IDX * NW + wave < A_BLK) load_a(kt, As + (IDX * NW + wave) * 1024, a_src[IDX]);
+    } else {
+      constexpr int J = IDX - A_LD;
+      if ((W_BLK % NW == 0) || J * NW + wave < W_BLK) load_w(kt, As + A_BYTES + (J * NW + wave) * 1024, w_src[J]);
+    }
+  };
+  auto issue_loads = [&](int kt, int stage) { static_for<A_LD + W_LD>([&](auto n) { issue_one_load(kt, stage, n); }); };
 
   // ---- fragment addressing.  Lane (a = lane%16, kq = lane/16) reads chunk ks*4 + kq of its fragment row.
   //      Both keys depend only on the lane, so the per-lane part of the address is loop-invariant.
@@ -144,7 +197,7 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
     x_off[ks] = (wm * WTM + fa) * 128 + (((ks * 4 + kq) ^ x_key) << 4);
-    w_off[ks] = A_BYTES + (wn * WTN + fq * (4 * NT) + fr) * 128 + (((ks * 4 + kq) ^ w_key) << 4);
+    w_off[ks] = A_BYTES + (wn * WTN + fq * (4 * G) + fr) * 128 + (((ks * 4 + kq) ^ w_key) << 4);
   }
 
   f32x4_t acc[MT][NT];
@@ -152,16 +205,9 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
   auto read_frags = [&](int stage, int ks, int b) {
     const char* base = smem + stage * STAGE;
 #pragma unroll
-    for (int j = 0; j < NT; ++j) wf[b][j] = *(const bf16x8_t*)(base + w_off[ks] + j * 4 * 128);
-#ifdef CS_EXP_SKIP_X  // experiment: issue only half of the activation-fragment reads (results are wrong)
-#pragma unroll
-    for (int i = 0; i < MT / 2; ++i) xf[b][i] = *(const bf16x8_t*)(base + x_off[ks] + i * 16 * 128);
-#pragma unroll
-    for (int i = MT / 2; i < MT; ++i) xf[b][i] = xf[b][i - MT / 2];
-#else
+    for (int j = 0; j < NT; ++j) wf[b][j] = *(const bf16x8_t*)(base + w_off[ks] + piece_col(j) * 128);
 #pragma unroll
     for (int i = 0; i < MT; ++i) xf[b][i] = *(const bf16x8_t*)(base + x_off[ks] + i * 16 * 128);
-#endif
   };
   auto mfmas = [&](int b) {
 #pragma unroll
@@ -169,6 +215,35 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
 #pragma unroll
       for (int j = 0; j < NT; ++j)
         acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[b][j], xf[b][i], acc[i][j], 0, 0, 0);
+  };
+
+  // ---- one-wave-per-SIMD form (NW == 4, 8x8 fragments per wave, 512 registers per lane).  The 64
+  //      accumulators live in the accumulation registers a[0:255], accumulator (i, j) in a[4(8i+j) .. +3],
+  //      and are touched ONLY by the inline-asm statements below (MFMAs here, v_accvgpr_read in the
+  //      epilogue): the compiler sees no accumulator values at all, so it cannot copy, rotate or spill them.
+  //      It is told once that the 256 registers are in use (the clobber list at the top of the kernel) so
+  //      that the kernel's register allocation covers them, and it has no reason to use them itself as long
+  //      as the rest of the kernel fits the 256 architectural registers (the build checks the generated
+  //      code for that).  asm volatile statements keep their program order, so the hook called after each
+  //      MFMA places LDS reads and direct loads at fixed points of the instruction stream.  The first k-step
+  //      of an output tile takes a zero addend, which saves clearing the accumulators.
+  auto read_one = [&](int stage, int ks, int b, auto idx_c) {
+    constexpr int IDX = decltype(idx_c)::value;
+    const char* base = smem + stage * STAGE;
+    if constexpr (IDX < NT) wf[b][IDX] = *(const bf16x8_t*)(base + w_off[ks] + piece_col(IDX) * 128);
+    else xf[b][IDX - NT] = *(const bf16x8_t*)(base + x_off[ks] + (IDX - NT) * 16 * 128);
+  };
+  auto mfmas_pinned = [&](auto b_c, auto zero_c, auto&& hook) {
+    constexpr int B = decltype(b_c)::value;
+    constexpr bool ZERO = decltype(zero_c)::value;
+    static_for<MT * NT>([&](auto n) {
+      constexpr int N = decltype(n)::value, I = N / NT, J = N % NT, R = N * 4;
+      if constexpr (ZERO)
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(wf[B][J]), "v"(xf[B][I]), "n"(R), "n"(R + 3));
+      else
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(wf[B][J]), "v"(xf[B][I]), "n"(R), "n"(R + 3));
+      hook(n);
+    });
   };
 
   const int nk = p.K / BK;
@@ -189,12 +264,14 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
   // NEXT output tile are requested inside the last K iteration of the current one, so they travel while
   // the epilogue runs.
   for (;;) {
+  if constexpr (NW == 8) {
 #pragma unroll
-  for (int i = 0; i < MT; ++i)
+    for (int i = 0; i < MT; ++i)
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
+      for (int j = 0; j < NT; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+  }
   const int vb_next = vb + gridDim.x;
   const bool has_next = vb_next < ntiles;
   int m0_next = 0, n0_next = 0;
@@ -206,10 +283,38 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
   read_frags(0, 0, 0);
 
   // One K iteration.  LOADS: tile kt+2 exists and is fetched; NEXT: tile kt+1 exists; LAST: final iteration.
-  auto body = [&](int kt, auto loads_c, auto next_c) {
-    constexpr bool LOADS = decltype(loads_c)::value, NEXT = decltype(next_c)::value;
+  auto body = [&](int kt, auto first_c, auto loads_c, auto next_c) {
+    constexpr bool FIRST = decltype(first_c)::value, LOADS = decltype(loads_c)::value, NEXT = decltype(next_c)::value;
     const int cur = kt & 1;
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (NW == 4) {
+      constexpr int NLD = A_LD + W_LD, NFR = MT + NT;
+      static_assert(2 * NLD <= MT * NT && 2 * NFR <= MT * NT, "one slot after an MFMA per LDS read / direct load");
+      // first k-step; meanwhile the fragments of the second k-step
+      mfmas_pinned(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
+        constexpr int N = decltype(n)::value;
+        if constexpr (N < NFR) read_one(cur, 1, 1, n);
+      });
+      // K tile kt+1 (requested one iteration ago) has landed in this wave's part of the other stage, and
+      // this wave has received its last fragments of the current stage
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+      wg_barrier();
+      if (!NEXT && has_next) {
+        tile_origin(vb_next, m0_next, n0_next);
+        setup_sources(m0_next, n0_next);
+      }
+      // second k-step; meanwhile the first fragments of K tile kt+1 and the request for K tile kt+2 into
+      // the stage that was just drained (or, at the end, for the next output tile's first two K tiles)
+      mfmas_pinned(ic<1>{}, std::false_type{}, [&](auto n) {
+        constexpr int N = decltype(n)::value;
+        if constexpr (NEXT && N < 2 * NFR && N % 2 == 0) read_one(cur ^ 1, 0, 0, ic<N / 2>{});
+        if constexpr (LOADS && N < 2 * NLD && N % 2 == 1) issue_one_load(kt + 2, cur, ic<N / 2>{});
+        if constexpr (!NEXT && N < 2 * NLD) {
+          if (has_next && (nk > 1 || N < NLD)) issue_one_load(N / NLD, N / NLD, ic<N % NLD>{});
+        }
+      });
+      return;
+    }
     read_frags(cur, 1, 1);
     mfmas(0);
     // Issue order: one fragment read after each of the first MFMAs, so the matrix cores never wait for
@@ -253,17 +358,29 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  int kt = 0;
-  for (; kt + 2 < nk; ++kt) body(kt, std::true_type{}, std::true_type{});
-  if (kt + 1 < nk) {
-    body(kt, std::false_type{}, std::true_type{});
-    ++kt;
+  {
+    constexpr std::true_type T{};
+    constexpr std::false_type F{};
+    if (nk >= 3) {
+      body(0, T, T, T);
+      int kt = 1;
+      for (; kt + 2 < nk; ++kt) body(kt, F, T, T);
+      body(kt, F, F, T);
+      body(kt + 1, F, F, F);
+    } else if (nk == 2) {
+      body(0, T, F, T);
+      body(1, F, F, F);
+    } else {
+      body(0, T, F, F);
+    }
   }
-  body(kt, std::false_type{}, std::false_type{});
+  // inline-asm MFMAs are opaque to the compiler's hazard tracking: let the last results land before the
+  // epilogue reads the accumulation registers
+  if constexpr (NW == 4) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   CS_TS(2);
 
   // ---- epilogue.  acc[i][j][r] = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
-  //      n = n0 + wn*WTN + (lane/16)*(4*NT) + 4j + r : 4*NT consecutive columns per lane and row.
+  //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
   //      Every load the epilogue needs (row map, bias, residual / position rows) is issued up front, from
   //      clamped addresses so that no branch guards a load: a load inside the store loop would make the
   //      compiler wait for ALL outstanding memory operations (vmcnt counts stores too), i.e. for every
@@ -271,46 +388,61 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
   {
     const bf16_t* const pBias = (const bf16_t*)p.bias;
     bf16_t* const pC = (bf16_t*)p.C;
-    const int n_lane = n0 + wn * WTN + kq * (4 * NT);
+    const int n_lane = n0 + wn * WTN + kq * (4 * G);
     int mrow[MT];
-    int64_t crow[MT];
+    int crow[MT];  // 32-bit row numbers; the 64-bit address is formed at the store
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
       mrow[i] = m0 + wm * WTM + i * 16 + fa;
       const int mc = min(mrow[i], p.M - 1);
-      crow[i] = p.c_rows ? (int64_t)p.c_rows[mc] : (int64_t)mc;
+      crow[i] = p.c_rows ? p.c_rows[mc] : mc;
     }
-    float bias_v[NT][4];
+    bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
 #pragma unroll
     for (int j = 0; j < NT; ++j) {
-      const int nc = min(n_lane + 4 * j, p.N - 4);
-      bf16x4_t bb = {0, 0, 0, 0};
-      if (pBias) bb = *(const bf16x4_t*)(pBias + nc);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) bias_v[j][r] = bf2f(bb[r]);
+      const int nc = min(n_lane + piece_col(j), p.N - 4);
+      bias_v[j] = bf16x4_t{0, 0, 0, 0};
+      if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + nc);
     }
     constexpr bool ADDEND = (EPI == CS_EPI_RESIDUAL) || (EPI == CS_EPI_BIAS_POS);
     bf16x4_t addend[ADDEND ? MT : 1][ADDEND ? NT : 1];
-    if (ADDEND) {
+    auto load_addend = [&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      const int mc = min(mrow[i], p.M - 1);
+      const bf16_t* row = (EPI == CS_EPI_RESIDUAL)
+                              ? (const bf16_t*)p.residual + (int64_t)mc * p.ldr
+                              : (const bf16_t*)p.pos + (int64_t)(mc % p.pos_period) * p.ldpos;
 #pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        const int mc = min(mrow[i], p.M - 1);
-        const bf16_t* row = (EPI == CS_EPI_RESIDUAL)
-                                ? (const bf16_t*)p.residual + (int64_t)mc * p.ldr
-                                : (const bf16_t*)p.pos + (int64_t)(mc % p.pos_period) * p.ldpos;
-#pragma unroll
-        for (int j = 0; j < NT; ++j) addend[i][j] = *(const bf16x4_t*)(row + min(n_lane + 4 * j, p.N - 4));
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
+      for (int j = 0; j < NT; ++j)
+        addend[ADDEND ? i : 0][ADDEND ? j : 0] = *(const bf16x4_t*)(row + min(n_lane + piece_col(j), p.N - 4));
+    };
+    // The one-wave-per-SIMD form must stay inside the architectural registers (its accumulation registers
+    // are not the compiler's to use), so it fetches the addend rows in two batches.
+    constexpr int ADD_BATCH = (NW == 4) ? MT / 2 : MT;
+    if constexpr (ADDEND) static_for<ADD_BATCH>(load_addend);
+    static_for<MT>([&](auto i_c) {
+      constexpr int i = decltype(i_c)::value;
+      if constexpr (ADDEND && i == ADD_BATCH && ADD_BATCH < MT)
+        static_for<MT - ADD_BATCH>([&](auto k_c) { load_addend(ic<ADD_BATCH + decltype(k_c)::value>{}); });
       const bool mok = mrow[i] < p.M;
+      f32x4_t racc[NT];
+      if constexpr (NW == 4) {
+        static_for<NT * 4>([&](auto e_c) {
+          constexpr int E = decltype(e_c)::value;
+          float t;
+          asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(i * NT * 4 + E));
+          racc[E / 4][E % 4] = t;
+        });
+      } else {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) racc[j] = acc[i][j];
+      }
       bf16x4_t out[NT];
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
         float v[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = acc[i][j][r] + bias_v[j][r];
+        for (int r = 0; r < 4; ++r) v[r] = racc[j][r] + bf2f(bias_v[j][r]);
         if (EPI == CS_EPI_SWIGLU) {
           // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the
           // product stay in fp32 until the single output rounding
@@ -333,24 +465,46 @@ __global__ __launch_bounds__(NTHREADS) void gemm_fast_kernel(const CsGemmArgs p,
           for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
         }
       }
+      // With G == 2 the pieces of fragments 2g and 2g+1 are adjacent: one 16-byte store per lane, and the
+      // four lanes of an output row write 64 consecutive bytes (32 with the halved SwiGLU output).
       if (EPI == CS_EPI_SWIGLU) {
-        bf16_t* dst = pC + crow[i] * p.ldc + (n_lane >> 1);
+        bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + (n_lane >> 1);
+        if constexpr (G == 2) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          if (mok && n_lane + 4 * j < p.N) {
-            bf16x2_t o;
-            o[0] = out[j][0];
-            o[1] = out[j][1];
-            *(bf16x2_t*)(dst + 2 * j) = o;
+          for (int j = 0; j < NT; j += 2) {
+            if (mok && n_lane + piece_col(j) < p.N) {
+              bf16x4_t o = {out[j][0], out[j][1], out[j + 1][0], out[j + 1][1]};
+              *(bf16x4_t*)(dst + (piece_col(j) >> 1)) = o;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            if (mok && n_lane + piece_col(j) < p.N) {
+              bf16x2_t o;
+              o[0] = out[j][0];
+              o[1] = out[j][1];
+              *(bf16x2_t*)(dst + (piece_col(j) >> 1)) = o;
+            }
           }
         }
       } else {
-        bf16_t* dst = pC + crow[i] * p.ldc + n_lane;
+        bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + n_lane;
+        if constexpr (G == 2) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
-          if (mok && n_lane + 4 * j < p.N) *(bf16x4_t*)(dst + 4 * j) = out[j];
+          for (int j = 0; j < NT; j += 2) {
+            if (mok && n_lane + piece_col(j) < p.N) {
+              bf16x8_t o = {out[j][0], out[j][1], out[j][2], out[j][3], out[j + 1][0], out[j + 1][1], out[j + 1][2], out[j + 1][3]};
+              *(bf16x8_t*)(dst + piece_col(j)) = o;
+            }
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+            if (mok && n_lane + piece_col(j) < p.N) *(bf16x4_t*)(dst + piece_col(j)) = out[j];
+        }
       }
-    }
+    });
   }
   CS_TS(3);
   if (!has_next) break;
@@ -378,7 +532,7 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   const int grid = tiles <= 256 ? tiles : 256;
   static const char* st_env = getenv("CS_GEMM_STAGGER");  // experiment knob: ticks of 10 ns per slot
   const int stagger = tiles > 256 ? (st_env ? atoi(st_env) : 0) : 0;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(NTHREADS), lds, stream, p, stagger);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES_M * WAVES_N), lds, stream, p, stagger);
   return cs_launch_status();
 }
 
@@ -408,7 +562,9 @@ double rounds_cost(int M, int N, int bm, int bn) {
 // Called by cs_gemm after argument validation.  Sets *handled when this path took the problem.
 int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   *handled = false;
-  if (a.w_fp8 || a.K % BK || a.M < 1 || a.w_scale || a.N < 4) return CS_OK;
+  if (a.w_fp8 || a.K % BK || a.M < 1 || a.w_scale || a.N < 8) return CS_OK;
+  // 16-byte output stores
+  if (a.N % 8 || a.ldc % 8 || ((uintptr_t)a.C & 15)) return CS_OK;
   if (a.pos && a.epilogue != CS_EPI_BIAS) return CS_OK;
   // per-lane source offsets are 32-bit byte offsets from the matrix bases
   if (a.a_rows) return CS_OK;  // gathered A rows can lie anywhere: the general kernel keeps 64-bit pointers
@@ -418,8 +574,9 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   // 256x160 tile exists for N = 1280 (8 column tiles: 8192 rows give exactly 256 workgroups).
   const double c256 = rounds_cost(a.M, a.N, 256, 256);
   const double c160 = rounds_cost(a.M, a.N, 256, 160) * 1.15;  // narrower tiles: more LDS and L2 traffic per FLOP
-  static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160" or "256"
-  if (force ? force[0] == '1' : c160 < c256) return dispatch_epi<256, 160, 4, 2>(a, stream);
+  static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160", "256" or "8" (8-wave 256x256)
+  if (force && force[0] == '8') return dispatch_epi<256, 256, 2, 4>(a, stream);
+  if (force ? force[0] == '1' : c160 < c256) return dispatch_epi<256, 160, 4, 1>(a, stream);
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with 256x128
   // tiles (twice as many workgroups, half as long).  The two launches write disjoint column ranges of C.
@@ -446,10 +603,10 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
       if (a.residual) hi.residual = (const char*)a.residual + (int64_t)n1 * 2;
       if (a.pos) hi.pos = (const char*)a.pos + (int64_t)n1 * 2;
       hi.C = (char*)a.C + (int64_t)(a.epilogue == CS_EPI_SWIGLU ? n1 / 2 : n1) * 2;
-      const int st = dispatch_epi<256, 256, 2, 4>(lo, stream);
+      const int st = dispatch_epi<256, 256, 2, 2>(lo, stream);
       if (st != CS_OK) return st;
-      return dispatch_epi<256, 128, 4, 2>(hi, stream);
+      return dispatch_epi<256, 128, 2, 2>(hi, stream);
     }
   }
-  return dispatch_epi<256, 256, 2, 4>(a, stream);
+  return dispatch_epi<256, 256, 2, 2>(a, stream);
 }
