@@ -308,9 +308,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
       mfmas_pinned(ic<1>{}, std::false_type{}, [&](auto n) {
         constexpr int N = decltype(n)::value;
         if constexpr (NEXT && N < 2 * NFR && N % 2 == 0) read_one(cur ^ 1, 0, 0, ic<N / 2>{});
-        if constexpr (LOADS && N < 2 * NLD && N % 2 == 1) issue_one_load(kt + 2, cur, ic<N / 2>{});
-        if constexpr (!NEXT && N < 2 * NLD) {
-          if (has_next && (nk > 1 || N < NLD)) issue_one_load(N / NLD, N / NLD, ic<N % NLD>{});
+        // four waves share the CU's one memory pipeline: space the direct loads as widely as the half allows
+        constexpr int LD_EVERY = (MT * NT) / NLD >= 4 ? 4 : ((MT * NT) / NLD >= 3 ? 3 : 2);
+        if constexpr (LOADS && N < LD_EVERY * NLD && N % LD_EVERY == LD_EVERY - 1)
+          issue_one_load(kt + 2, cur, ic<N / LD_EVERY>{});
+        constexpr int PF_EVERY = (MT * NT) / (2 * NLD);
+        if constexpr (!NEXT && N < PF_EVERY * 2 * NLD && N % PF_EVERY == PF_EVERY - 1) {
+          constexpr int L = N / PF_EVERY;
+          if (has_next && (nk > 1 || L < NLD)) issue_one_load(L / NLD, L / NLD, ic<L % NLD>{});
         }
       });
       return;
