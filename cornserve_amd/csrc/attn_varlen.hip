@@ -19,6 +19,8 @@
 // order, which is legal because a dot product does not care about the order of its terms.
 // V is transposed once per tile on its way into LDS (pairs of keys packed into 32-bit writes).
 // Head dims that are not multiples of 16 (SigLIP's 72) are zero-padded in LDS only.
+#include <type_traits>
+
 #include "common.h"
 
 namespace {
@@ -38,7 +40,7 @@ struct AttnArgs {
   float scale_log2e;
 };
 
-template <int D, int NWAVES, bool ROPE>
+template <int D, int NWAVES, bool ROPE, int HPW>
 __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
   constexpr int NT = NWAVES * 64;
   constexpr int BQ = NWAVES * 32;
@@ -56,12 +58,12 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 31, hf = lane >> 5;
-  const int head = blockIdx.y;
+  const int head0 = blockIdx.y * HPW;  // this workgroup's HPW consecutive heads
   const int seg_start = a.work[blockIdx.x * 4 + 0];
   const int seg_end = a.work[blockIdx.x * 4 + 1];
   const int q0 = a.work[blockIdx.x * 4 + 2];
   const int nq = a.work[blockIdx.x * 4 + 3];
-  const int64_t hoff = (int64_t)head * D;
+  int64_t hoff = (int64_t)head0 * D;  // column offset of the head being processed
 
   // Stage `nrows` rows starting at global row g0 (valid rows: < g0 + nvalid) of a [*, ld] tensor into an
   // LDS tile with row stride RS, zero-filling invalid rows and pad chunks, optionally rotating.
@@ -127,29 +129,46 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
     }
   };
 
-  stage_rows(a.q, q_lds, q0, BQ, nq);
-  __syncthreads();
-  bf16x8_t qf[KS];
-#pragma unroll
-  for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8_t*)(q_lds + (wave * 32 + fr) * RS + (2 * ks + hf) * 16);
-
   f32x16_t oacc[DT];
+  float m_run, l_run;
+  auto reset_state = [&]() {
 #pragma unroll
-  for (int t = 0; t < DT; ++t)
+    for (int t = 0; t < DT; ++t)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
-  float m_run = -INFINITY, l_run = 0.f;
+      for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
+    m_run = -INFINITY;
+    l_run = 0.f;
+  };
   const bool wave_active = wave * 32 < nq;
+  // O^T[d][q] / l -> out[q][head*D + d]; lane owns query wave*32 + fr and 4 consecutive d per group.
+  auto write_out = [&]() {
+    const int qi = wave * 32 + fr;
+    if (qi < nq) {
+      const float inv = 1.0f / l_run;
+      bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
+#pragma unroll
+      for (int t = 0; t < DT; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int d0 = t * 32 + 8 * g + 4 * hf;
+          if (d0 < D) {
+            bf16x4_t o;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
+            *(bf16x4_t*)(orow + d0) = o;
+          }
+        }
+    }
+  };
+  bf16x8_t qf[KS];
+  auto load_q_frags = [&]() {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8_t*)(q_lds + (wave * 32 + fr) * RS + (2 * ks + hf) * 16);
+  };
 
-  const int seg_len = seg_end - seg_start;
-  for (int kv0 = 0; kv0 < seg_len; kv0 += BKV) {
-    const int nvalid = min(BKV, seg_len - kv0);
-    __syncthreads();  // previous tile fully consumed
-    stage_rows(a.k, k_lds, seg_start + kv0, BKV, nvalid);
-    stage_v(seg_start + kv0, nvalid);
-    __syncthreads();
-    if (!wave_active) continue;
-
+  // One K/V tile in LDS (nvalid keys): S^T = K Q^T, online softmax, O^T += V^T P^T.
+  auto compute_tile = [&](int nvalid, auto first_c) {
+    constexpr bool FIRST_TILE = decltype(first_c)::value;  // nothing accumulated yet: no rescale of O
     f32x16_t sacc[2];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
@@ -163,18 +182,22 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
     }
     // mask keys past the segment end, running max
     float mx = -INFINITY;
+    if (nvalid < BKV) {  // uniform: only a segment's last tile can be partial
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+          if (key >= nvalid) sacc[kt][r] = -INFINITY;
+        }
+    }
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-        const float s = key < nvalid ? sacc[kt][r] : -INFINITY;
-        sacc[kt][r] = s;
-        mx = fmaxf(mx, s);
-      }
+      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
     const float m_new = fmaxf(m_run, mx);
-    const float alpha = exp2f((m_run - m_new) * a.scale_log2e);
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
     const float mb = m_new * a.scale_log2e;
     float psum = 0.f;
     bf16x8_t pf[2][2];
@@ -182,7 +205,7 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        const float pv = exp2f(sacc[kt][r] * a.scale_log2e - mb);
+        const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * a.scale_log2e - mb);
         psum += pv;
         pf[kt][r >> 3][r & 7] = f2bf(pv);
       }
@@ -191,8 +214,10 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
     m_run = m_new;
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
+      if (!FIRST_TILE) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+        for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+      }
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -209,25 +234,123 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
           oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][kk], oacc[t], 0, 0, 0);
         }
     }
-  }
+  };
 
-  // O^T[d][q] / l -> out[q][head*D + d]; lane owns query wave*32 + fr and 4 consecutive d per group.
-  const int qi = wave * 32 + fr;
-  if (qi < nq) {
-    const float inv = 1.0f / l_run;
-    bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
+  const int seg_len = seg_end - seg_start;
+  if (ROPE && BQ == BKV && seg_len <= BKV && q0 == seg_start) {
+    // A whole segment in one tile (window attention): the query rows ARE the key rows.  Every global load
+    // of a head -- q, k, v -- is issued in one batch into registers, the rotary table is fetched once
+    // for all HPW heads, and the batch of head h+1 is requested before the matrix-core work on head h,
+    // so after the first head the memory latency hides behind compute.
+    constexpr int HC = DC / 2;
+    constexpr int NI = (BKV * HC + NT - 1) / NT, NV = ((BKV / 2) * DC + NT - 1) / NT;
+    const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    bf16x8_t q1[NI], q2[NI], k1[NI], k2[NI], v0[NV], v1[NV];
+    f32x4_t c0[NI], c1[NI], s0[NI], s1[NI];
+    // Unconditional loads from clamped rows (no branch between them, so they are all in flight together).
+    // Rows past the segment end therefore hold copies of the last row: as keys they are masked (P = 0, and
+    // 0 times a finite V row is 0), as queries their outputs are never written.
 #pragma unroll
-    for (int t = 0; t < DT; ++t)
+    for (int it = 0; it < NI; ++it) {
+      const int i = min(tid + it * NT, BKV * HC - 1), r = i / HC, jc = i - r * HC;
+      const float* cs = a.cos_sin + (int64_t)(seg_start + min(r, seg_len - 1)) * D + jc * 8;
+      c0[it] = *(const f32x4_t*)cs;
+      c1[it] = *(const f32x4_t*)(cs + 4);
+      s0[it] = *(const f32x4_t*)(cs + D / 2);
+      s1[it] = *(const f32x4_t*)(cs + D / 2 + 4);
+    }
+    auto issue_qkv = [&](int64_t ho) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int d0 = t * 32 + 8 * g + 4 * hf;
-        if (d0 < D) {
-          bf16x4_t o;
+      for (int it = 0; it < NI; ++it) {
+        const int i = min(tid + it * NT, BKV * HC - 1), r = i / HC, jc = i - r * HC;
+        const int64_t off = (int64_t)(seg_start + min(r, seg_len - 1)) * a.ld + ho + jc * 8;
+        q1[it] = *(const bf16x8_t*)(a.q + off);
+        q2[it] = *(const bf16x8_t*)(a.q + off + D / 2);
+        k1[it] = *(const bf16x8_t*)(a.k + off);
+        k2[it] = *(const bf16x8_t*)(a.k + off + D / 2);
+      }
 #pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
-          *(bf16x4_t*)(orow + d0) = o;
+      for (int it = 0; it < NV; ++it) {
+        const int i = min(tid + it * NT, (BKV / 2) * DC - 1), kp = i % (BKV / 2), c = i / (BKV / 2), r0 = 2 * kp;
+        v0[it] = *(const bf16x8_t*)(a.v + (int64_t)(seg_start + min(r0, seg_len - 1)) * a.ld + ho + c * 8);
+        v1[it] = *(const bf16x8_t*)(a.v + (int64_t)(seg_start + min(r0 + 1, seg_len - 1)) * a.ld + ho + c * 8);
+      }
+    };
+    issue_qkv(hoff);
+    if (DKC > DC) {  // pad chunks of the q and k tiles: written once, never overwritten
+      for (int i = tid; i < BKV * (DKC - DC); i += NT) {
+        const int r = i / (DKC - DC), c = DC + i % (DKC - DC);
+        *(bf16x8_t*)(q_lds + r * RS + c * 16) = zero;
+        *(bf16x8_t*)(k_lds + r * RS + c * 16) = zero;
+      }
+    }
+#pragma unroll
+    for (int hh = 0; hh < HPW; ++hh) {
+      if (hh > 0) __syncthreads();  // every wave is done reading the previous head's tiles
+#pragma unroll
+      for (int it = 0; it < NI; ++it) {
+        const int i = tid + it * NT, r = i / HC, jc = i - r * HC;
+        if (i < BKV * HC) {
+          bf16x8_t qa, qb, ka, kb;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const float co = e < 4 ? c0[it][e] : c1[it][e - 4];
+            const float si = e < 4 ? s0[it][e] : s1[it][e - 4];
+            const float xa = bf2f(q1[it][e]), xb = bf2f(q2[it][e]);
+            qa[e] = f2bf(xa * co - xb * si);
+            qb[e] = f2bf(xa * si + xb * co);
+            const float ya = bf2f(k1[it][e]), yb = bf2f(k2[it][e]);
+            ka[e] = f2bf(ya * co - yb * si);
+            kb[e] = f2bf(ya * si + yb * co);
+          }
+          *(bf16x8_t*)(q_lds + r * RS + jc * 16) = qa;
+          *(bf16x8_t*)(q_lds + r * RS + (jc + HC) * 16) = qb;
+          *(bf16x8_t*)(k_lds + r * RS + jc * 16) = ka;
+          *(bf16x8_t*)(k_lds + r * RS + (jc + HC) * 16) = kb;
         }
       }
+#pragma unroll
+      for (int it = 0; it < NV; ++it) {
+        const int i = tid + it * NT, kp = i % (BKV / 2), c = i / (BKV / 2), r0 = 2 * kp;
+        if (i < (BKV / 2) * DC) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            bf16x2_t pr;
+            pr[0] = v0[it][e];
+            pr[1] = v1[it][e];
+            *(bf16x2_t*)(vt_lds + (c * 8 + e) * VT_STRIDE + r0) = pr;
+          }
+        }
+      }
+      __syncthreads();
+      if (hh + 1 < HPW) issue_qkv(hoff + D);  // the staging registers are free again
+      reset_state();
+      if (wave_active) {
+        load_q_frags();
+        compute_tile(seg_len, std::true_type{});
+      }
+      write_out();
+      hoff += D;
+    }
+  } else {
+    for (int hh = 0; hh < HPW; ++hh) {
+      if (hh > 0) __syncthreads();
+      reset_state();
+      stage_rows(a.q, q_lds, q0, BQ, nq);
+      __syncthreads();
+      load_q_frags();
+      for (int kv0 = 0; kv0 < seg_len; kv0 += BKV) {
+        const int nvalid = min(BKV, seg_len - kv0);
+        __syncthreads();  // previous tile fully consumed
+        stage_rows(a.k, k_lds, seg_start + kv0, BKV, nvalid);
+        stage_v(seg_start + kv0, nvalid);
+        __syncthreads();
+        if (!wave_active) continue;
+        compute_tile(nvalid, std::false_type{});
+      }
+      write_out();
+      hoff += D;
+    }
   }
 }
 
@@ -506,10 +629,16 @@ int launch_attn(const AttnArgs& a, int n_work, int heads, int block_q, bool rope
   const dim3 grid(n_work, heads);
   if (block_q == 64) {
     if (rope) {
-      if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_kernel<D, 2, true>), grid, dim3(128), 0, stream, a);
-      else return CS_ERR_UNSUPPORTED;
+      // two heads per workgroup when that still leaves several workgroups per CU
+      const bool pair = heads % 2 == 0 && (int64_t)n_work * heads >= 2048;
+      if constexpr (D % 16 == 0) {
+        if (pair) hipLaunchKernelGGL((attn_kernel<D, 2, true, 2>), dim3(n_work, heads / 2), dim3(128), 0, stream, a);
+        else hipLaunchKernelGGL((attn_kernel<D, 2, true, 1>), grid, dim3(128), 0, stream, a);
+      } else {
+        return CS_ERR_UNSUPPORTED;
+      }
     } else {
-      hipLaunchKernelGGL((attn_kernel<D, 2, false>), grid, dim3(128), 0, stream, a);
+      hipLaunchKernelGGL((attn_kernel<D, 2, false, 1>), grid, dim3(128), 0, stream, a);
     }
   } else {
     if (rope) {
