@@ -116,6 +116,10 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   constexpr bool ILV = NW == 4 || (MT * NT * 4 + (MT + NT) * 8) <= 176;
   constexpr int A_BLK = BM / 8, W_BLK = BN / 8;            // 8-row blocks = direct loads per stage
   constexpr int A_LD = (A_BLK + NW - 1) / NW, W_LD = (W_BLK + NW - 1) / NW;  // per wave
+  // Tiles whose stage is small enough get a ring of THREE stages (one-wave-per-SIMD form only): the direct
+  // loads of a K tile are then spread over two half-iterations and have a whole iteration more to land.
+  constexpr bool RING = NW == 4 && 3 * STAGE <= 160 * 1024;
+  constexpr int NLD = A_LD + W_LD, H1 = NLD / 2, H2 = NLD - H1;  // direct loads per wave and K tile; its two halves
 
   // ---- tile coordinates of virtual block vb in [0, tiles): XCD-aware remap (workgroup i runs on XCD i%8,
   //      and the persistent stride gridDim.x is a multiple of 8, so a workgroup's tiles stay on its XCD),
@@ -259,6 +263,8 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   setup_sources(m0, n0);
   issue_loads(0, 0);
   if (nk > 1) issue_loads(1, 1);
+  if constexpr (RING) static_for<H1>([&](auto n) { issue_one_load(2, 2, n); });  // nk >= 3 (checked on the host)
+  int st = 0;  // ring form: LDS stage of the current K tile; keeps rotating across output tiles
 
   // Persistent loop over this workgroup's tiles (vb, vb + gridDim.x, ...).  The first two K tiles of the
   // NEXT output tile are requested inside the last K iteration of the current one, so they travel while
@@ -277,10 +283,68 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   int m0_next = 0, n0_next = 0;
 
   CS_TS(0);
-  CS_WAIT_VMCNT(0);  // K tiles 0 and 1 of this output tile (and the previous tile's stores)
-  wg_barrier();
-  CS_TS(1);
-  read_frags(0, 0, 0);
+  if constexpr (RING) {
+    // K tile 0 has landed once at most the loads issued after it are outstanding: K tile 1 and the first
+    // half of K tile 2.  (Loads complete in order; stores of the previous epilogue that are still in
+    // flight only make this wait longer, never shorter.)
+    CS_WAIT_VMCNT(NLD + H1);
+    wg_barrier();
+    CS_TS(1);
+    read_frags(st, 0, 0);
+  } else {
+    CS_WAIT_VMCNT(0);  // K tiles 0 and 1 of this output tile (and the previous tile's stores)
+    wg_barrier();
+    CS_TS(1);
+    read_frags(0, 0, 0);
+  }
+
+  // Ring form of one K iteration.  MODE 0: steady state; 3, 2, 1: that many iterations before the end of
+  // the output tile, where the loads switch over to the next output tile's first K tiles.  In iteration kt
+  // the first half requests the SECOND half of K tile kt+2 (stage freed one barrier ago) and the second
+  // half requests the FIRST half of K tile kt+3 (the stage this iteration's barrier has just freed).
+  auto body_ring = [&](int kt, auto first_c, auto mode_c) {
+    constexpr bool FIRST = decltype(first_c)::value;
+    constexpr int MODE = decltype(mode_c)::value;
+    constexpr int NFR = MT + NT;
+    constexpr int EA = (MT * NT) / H2, EB = (MT * NT) / H1;  // MFMAs per direct load in each half
+    static_assert(2 * NFR <= MT * NT && EA >= 1 && EB >= 1, "one slot after an MFMA per LDS read / direct load");
+    const int s_cur = st, s_nxt = st == 2 ? 0 : st + 1, s_prv = st == 0 ? 2 : st - 1;
+    const int k_a = (MODE == 0 || MODE == 3) ? kt + 2 : 2 - MODE;  // MODE 2 -> next tile's 0, MODE 1 -> 1
+    const int k_b = MODE == 0 ? kt + 3 : 3 - MODE;                 // MODE 3 -> next tile's 0, 2 -> 1, 1 -> 2
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas_pinned(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
+      constexpr int N = decltype(n)::value;
+      if constexpr (N < NFR) read_one(s_cur, 1, 1, n);
+      if constexpr (N < EA * H2 && N % EA == EA - 1) {
+        if constexpr (MODE == 0 || MODE == 3) issue_one_load(k_a, s_prv, ic<H1 + N / EA>{});
+        else if (has_next) issue_one_load(k_a, s_prv, ic<H1 + N / EA>{});
+      }
+    });
+    // K tile kt+1 has landed once at most the NLD loads issued after it (K tile kt+2) are outstanding
+    if constexpr (MODE == 1) {
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): nothing more is read from LDS for this output tile
+    } else if (MODE == 2 && !has_next) {
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    } else {
+      __builtin_amdgcn_s_waitcnt(((NLD & 0xF) | ((NLD >> 4) << 14)) | 0x0070);  // vmcnt(NLD) lgkmcnt(0)
+    }
+    wg_barrier();
+    if constexpr (MODE == 3) {
+      if (has_next) {
+        tile_origin(vb_next, m0_next, n0_next);
+        setup_sources(m0_next, n0_next);
+      }
+    }
+    mfmas_pinned(ic<1>{}, std::false_type{}, [&](auto n) {
+      constexpr int N = decltype(n)::value;
+      if constexpr (MODE != 1 && N < 2 * NFR && N % 2 == 0) read_one(s_nxt, 0, 0, ic<N / 2>{});
+      if constexpr (N < EB * H1 && N % EB == EB - 1) {
+        if constexpr (MODE == 0) issue_one_load(k_b, s_cur, ic<N / EB>{});
+        else if (has_next) issue_one_load(k_b, s_cur, ic<N / EB>{});
+      }
+    });
+    st = s_nxt;
+  };
 
   // One K iteration.  LOADS: tile kt+2 exists and is fetched; NEXT: tile kt+1 exists; LAST: final iteration.
   auto body = [&](int kt, auto first_c, auto loads_c, auto next_c) {
@@ -363,7 +427,20 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  {
+  if constexpr (RING) {
+    constexpr std::true_type T{};
+    constexpr std::false_type F{};
+    if (nk == 3) {
+      body_ring(0, T, ic<3>{});
+    } else {
+      body_ring(0, T, ic<0>{});
+      int kt = 1;
+      for (; kt < nk - 3; ++kt) body_ring(kt, F, ic<0>{});
+      body_ring(nk - 3, F, ic<3>{});
+    }
+    body_ring(nk - 2, F, ic<2>{});
+    body_ring(nk - 1, F, ic<1>{});
+  } else {
     constexpr std::true_type T{};
     constexpr std::false_type F{};
     if (nk >= 3) {
@@ -524,7 +601,8 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   CsGemmArgs p = a;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  constexpr int lds = 2 * (BM + BN) * BK * 2;
+  constexpr int stage_bytes = (BM + BN) * BK * 2;
+  constexpr int lds = ((WAVES_M * WAVES_N == 4 && 3 * stage_bytes <= 160 * 1024) ? 3 : 2) * stage_bytes;
   static bool attr_set = false;
   auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
   if (!attr_set) {
@@ -567,7 +645,7 @@ double rounds_cost(int M, int N, int bm, int bn) {
 // Called by cs_gemm after argument validation.  Sets *handled when this path took the problem.
 int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   *handled = false;
-  if (a.w_fp8 || a.K % BK || a.M < 1 || a.w_scale || a.N < 8) return CS_OK;
+  if (a.w_fp8 || a.K % BK || a.K < 3 * BK || a.M < 1 || a.w_scale || a.N < 8) return CS_OK;
   // 16-byte output stores
   if (a.N % 8 || a.ldc % 8 || ((uintptr_t)a.C & 15)) return CS_OK;
   if (a.pos && a.epilogue != CS_EPI_BIAS) return CS_OK;
@@ -583,21 +661,30 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   if (force && force[0] == '8') return dispatch_epi<256, 256, 2, 4>(a, stream);
   if (force ? force[0] == '1' : c160 < c256) return dispatch_epi<256, 160, 4, 1>(a, stream);
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
-  // that fill whole rounds go to one launch and the remaining columns to a second launch with 256x128
-  // tiles (twice as many workgroups, half as long).  The two launches write disjoint column ranges of C.
+  // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller
+  // tiles (256x128 or 128x192: more workgroups, each shorter).  The two launches write disjoint column
+  // ranges of C.
   if (!force) {
-    const int tm = (a.M + 255) / 256, tn = (a.N + 255) / 256;
+    const int tn = (a.N + 255) / 256;
     double best = c256;
     int best_cols = 0;
+    bool best_192 = false;
     for (int c = tn - 1; c >= 1 && c >= tn - 12; --c) {
       const int rest = a.N - c * 256;
-      const double cost = rounds_cost(a.M, c * 256, 256, 256) + rounds_cost(a.M, rest, 256, 128) * 1.10;
-      if (cost < best - 0.05) {
-        best = cost;
+      const double lead = rounds_cost(a.M, c * 256, 256, 256);
+      const double c128 = lead + rounds_cost(a.M, rest, 256, 128) * 1.10 + 0.15;  // + per-tile fixed cost of a round
+      const double c192 = lead + rounds_cost(a.M, rest, 128, 192) * 1.20 + 0.15;
+      if (c128 < best - 0.05) {
+        best = c128;
         best_cols = c;
+        best_192 = false;
+      }
+      if (c192 < best - 0.02) {
+        best = c192;
+        best_cols = c;
+        best_192 = true;
       }
     }
-    (void)tm;
     if (best_cols > 0) {
       const int n1 = best_cols * 256;
       CsGemmArgs lo = a, hi = a;
@@ -610,6 +697,7 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
       hi.C = (char*)a.C + (int64_t)(a.epilogue == CS_EPI_SWIGLU ? n1 / 2 : n1) * 2;
       const int st = dispatch_epi<256, 256, 2, 2>(lo, stream);
       if (st != CS_OK) return st;
+      if (best_192) return dispatch_epi<128, 192, 2, 2>(hi, stream);
       return dispatch_epi<256, 128, 2, 2>(hi, stream);
     }
   }
