@@ -120,6 +120,11 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   // loads of a K tile are then spread over two half-iterations and have a whole iteration more to land.
   constexpr bool RING = NW == 4 && 3 * STAGE <= 160 * 1024;
   constexpr int NLD = A_LD + W_LD, H1 = NLD / 2, H2 = NLD - H1;  // direct loads per wave and K tile; its two halves
+  // The 256x256 tile (two 32 KB operand tiles per K tile) uses the whole 160 KB as a ring of FIVE 32 KB units
+  // holding A(kt), W(kt), A(kt+1), W(kt+1) and one unit in flight: A(kt+2) is requested in the first half
+  // of iteration kt, W(kt+2) in the second half into the unit the barrier has just freed.
+  constexpr bool RING5 = NW == 4 && !RING && A_BYTES == W_BYTES && 5 * A_BYTES <= 160 * 1024;
+  constexpr int UNIT = A_BYTES;
 
   // ---- tile coordinates of virtual block vb in [0, tiles): XCD-aware remap (workgroup i runs on XCD i%8,
   //      and the persistent stride gridDim.x is a multiple of 8, so a workgroup's tiles stay on its XCD),
@@ -188,6 +193,13 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
       if ((W_BLK % NW == 0) || J * NW + wave < W_BLK) load_w(kt, As + A_BYTES + (J * NW + wave) * 1024, w_src[J]);
     }
   };
+  // five-unit ring: one direct load of operand tile (A or W) of K tile kt into ring unit `slot`
+  auto issue_unit_load = [&](int kt, auto is_w_c, int slot, auto idx_c) {
+    constexpr int IDX = decltype(idx_c)::value;
+    char* dst = smem + slot * UNIT + (IDX * NW + wave) * 1024;
+    if constexpr (decltype(is_w_c)::value) load_w(kt, dst, w_src[IDX]);
+    else load_a(kt, dst, a_src[IDX]);
+  };
   auto issue_loads = [&](int kt, int stage) { static_for<A_LD + W_LD>([&](auto n) { issue_one_load(kt, stage, n); }); };
 
   // ---- fragment addressing.  Lane (a = lane%16, kq = lane/16) reads chunk ks*4 + kq of its fragment row.
@@ -237,6 +249,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
     if constexpr (IDX < NT) wf[b][IDX] = *(const bf16x8_t*)(base + w_off[ks] + piece_col(IDX) * 128);
     else xf[b][IDX - NT] = *(const bf16x8_t*)(base + x_off[ks] + (IDX - NT) * 16 * 128);
   };
+  // five-unit ring: fragment IDX of k-step ks from the units holding the A and W tiles
+  auto read_one5 = [&](int slot_a, int slot_w, int ks, int b, auto idx_c) {
+    constexpr int IDX = decltype(idx_c)::value;
+    if constexpr (IDX < NT)
+      wf[b][IDX] = *(const bf16x8_t*)(smem + slot_w * UNIT + (w_off[ks] - A_BYTES) + piece_col(IDX) * 128);
+    else
+      xf[b][IDX - NT] = *(const bf16x8_t*)(smem + slot_a * UNIT + x_off[ks] + (IDX - NT) * 16 * 128);
+  };
   auto mfmas_pinned = [&](auto b_c, auto zero_c, auto&& hook) {
     constexpr int B = decltype(b_c)::value;
     constexpr bool ZERO = decltype(zero_c)::value;
@@ -261,8 +281,16 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   int m0, n0;
   tile_origin(vb, m0, n0);
   setup_sources(m0, n0);
-  issue_loads(0, 0);
-  if (nk > 1) issue_loads(1, 1);
+  if constexpr (RING5) {  // units 0..3 = A(0), W(0), A(1), W(1); nk >= 3 (checked on the host)
+    static_for<A_LD>([&](auto n) { issue_unit_load(0, std::false_type{}, 0, n); });
+    static_for<W_LD>([&](auto n) { issue_unit_load(0, std::true_type{}, 1, n); });
+    static_for<A_LD>([&](auto n) { issue_unit_load(1, std::false_type{}, 2, n); });
+    static_for<W_LD>([&](auto n) { issue_unit_load(1, std::true_type{}, 3, n); });
+  } else {
+    issue_loads(0, 0);
+    if (nk > 1) issue_loads(1, 1);
+  }
+  int ua = 0;  // five-unit ring: unit of A(kt); W(kt), A(kt+1), W(kt+1), A(kt+2) follow cyclically
   if constexpr (RING) static_for<H1>([&](auto n) { issue_one_load(2, 2, n); });  // nk >= 3 (checked on the host)
   int st = 0;  // ring form: LDS stage of the current K tile; keeps rotating across output tiles
 
@@ -283,7 +311,12 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   int m0_next = 0, n0_next = 0;
 
   CS_TS(0);
-  if constexpr (RING) {
+  if constexpr (RING5) {
+    CS_WAIT_VMCNT(NLD);  // K tile 0 has landed once at most K tile 1's loads are outstanding
+    wg_barrier();
+    CS_TS(1);
+    static_for<MT + NT>([&](auto n) { read_one5(ua, (ua + 1) % 5, 0, 0, n); });
+  } else if constexpr (RING) {
     // K tile 0 has landed once at most the loads issued after it are outstanding: K tile 1 and the first
     // half of K tile 2.  (Loads complete in order; stores of the previous epilogue that are still in
     // flight only make this wait longer, never shorter.)
@@ -344,6 +377,51 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
       }
     });
     st = s_nxt;
+  };
+
+  // Five-unit-ring form of one K iteration.  MODE 0: steady state; 2, 1: that many iterations before the
+  // end of the output tile, where the loads belong to the next output tile.
+  auto body_ring5 = [&](int kt, auto first_c, auto mode_c) {
+    constexpr bool FIRST = decltype(first_c)::value;
+    constexpr int MODE = decltype(mode_c)::value;
+    constexpr int NFR = MT + NT;
+    constexpr int EA = (MT * NT) / A_LD, EB = (MT * NT) / W_LD;
+    static_assert(2 * NFR <= MT * NT, "one slot after an MFMA per LDS read");
+    const int u_a0 = ua, u_w0 = (ua + 1) % 5, u_a1 = (ua + 2) % 5, u_w1 = (ua + 3) % 5, u_a2 = (ua + 4) % 5;
+    const int k_ld = MODE == 0 ? kt + 2 : 2 - MODE;  // MODE 2 -> next tile's K tile 0, MODE 1 -> 1
+    if constexpr (MODE == 2) {
+      if (has_next) {  // every load of this output tile has been issued
+        tile_origin(vb_next, m0_next, n0_next);
+        setup_sources(m0_next, n0_next);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mfmas_pinned(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
+      constexpr int N = decltype(n)::value;
+      if constexpr (N < NFR) read_one5(u_a0, u_w0, 1, 1, n);
+      if constexpr (N < EA * A_LD && N % EA == EA - 1) {
+        if constexpr (MODE == 0) issue_unit_load(k_ld, std::false_type{}, u_a2, ic<N / EA>{});
+        else if (has_next) issue_unit_load(k_ld, std::false_type{}, u_a2, ic<N / EA>{});
+      }
+    });
+    // K tile kt+1 has landed once at most the A_LD loads issued after it (A of K tile kt+2) are outstanding
+    if constexpr (MODE == 1) {
+      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): nothing more is read from LDS for this output tile
+    } else if (MODE == 2 && !has_next) {
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    } else {
+      __builtin_amdgcn_s_waitcnt(((A_LD & 0xF) | ((A_LD >> 4) << 14)) | 0x0070);  // vmcnt(A_LD) lgkmcnt(0)
+    }
+    wg_barrier();
+    mfmas_pinned(ic<1>{}, std::false_type{}, [&](auto n) {
+      constexpr int N = decltype(n)::value;
+      if constexpr (MODE != 1 && N < 2 * NFR && N % 2 == 0) read_one5(u_a1, u_w1, 0, 0, ic<N / 2>{});
+      if constexpr (N < EB * W_LD && N % EB == EB - 1) {
+        if constexpr (MODE == 0) issue_unit_load(k_ld, std::true_type{}, u_a0, ic<N / EB>{});
+        else if (has_next) issue_unit_load(k_ld, std::true_type{}, u_a0, ic<N / EB>{});
+      }
+    });
+    ua = u_a1;
   };
 
   // One K iteration.  LOADS: tile kt+2 exists and is fetched; NEXT: tile kt+1 exists; LAST: final iteration.
@@ -427,7 +505,14 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
     }
     __builtin_amdgcn_sched_barrier(0);
   };
-  if constexpr (RING) {
+  if constexpr (RING5) {
+    constexpr std::true_type T{};
+    constexpr std::false_type F{};
+    body_ring5(0, T, ic<0>{});
+    for (int kt = 1; kt < nk - 2; ++kt) body_ring5(kt, F, ic<0>{});
+    body_ring5(nk - 2, F, ic<2>{});
+    body_ring5(nk - 1, F, ic<1>{});
+  } else if constexpr (RING) {
     constexpr std::true_type T{};
     constexpr std::false_type F{};
     if (nk == 3) {
@@ -602,7 +687,9 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   constexpr int stage_bytes = (BM + BN) * BK * 2;
-  constexpr int lds = ((WAVES_M * WAVES_N == 4 && 3 * stage_bytes <= 160 * 1024) ? 3 : 2) * stage_bytes;
+  constexpr bool ring3 = WAVES_M * WAVES_N == 4 && 3 * stage_bytes <= 160 * 1024;
+  constexpr bool ring5 = WAVES_M * WAVES_N == 4 && !ring3 && BM == BN && 5 * BM * BK * 2 <= 160 * 1024;
+  constexpr int lds = ring5 ? 5 * BM * BK * 2 : (ring3 ? 3 : 2) * stage_bytes;
   static bool attr_set = false;
   auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
   if (!attr_set) {
