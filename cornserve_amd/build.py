@@ -91,6 +91,19 @@ def _check_source(hipcc: str, src: Path) -> None:
                            + "\n  ".join(offenders))
 
 
+def _check_no_missing_kernels(lib: Path) -> None:
+    """A shared library links with undefined symbols; a kernel whose host-side launch stub the compiler
+    dropped would only show up as a load error on the GPU box.  Every undefined symbol must be external
+    (HIP runtime, libc/libstdc++): none may come from this library's own (anonymous) namespaces."""
+    nm = shutil.which("nm")
+    if nm is None:
+        return
+    out = subprocess.run([nm, "-D", "--undefined-only", str(lib)], stdout=subprocess.PIPE, text=True).stdout
+    own = [line.split()[-1] for line in out.splitlines() if "GLOBAL__N" in line or " cs_" in line]
+    if own:
+        raise RuntimeError(f"{lib.name} has undefined symbols of its own (dropped kernels?):\n  " + "\n  ".join(own))
+
+
 def build_library(force: bool = True, jobs: int = 6) -> Path:
     """Compile every .hip source under csrc/ and link the shared library. Returns its path."""
     hipcc = _hipcc()
@@ -111,6 +124,7 @@ def build_library(force: bool = True, jobs: int = 6) -> Path:
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(todo) or 1))) as pool:
         list(pool.map(lambda job: job(), todo))
     _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(LIB_PATH), *map(str, objs)])
+    _check_no_missing_kernels(LIB_PATH)
     return LIB_PATH
 
 

@@ -1,17 +1,28 @@
 // Fast-path bf16 MFMA GEMM for gfx950:  C[M,N] = epilogue(A[M,K] . W[N,K]^T),  K % 64 == 0, bf16 weights.
 //
-// Pipeline.  One workgroup owns a BM x BN tile of C and walks K in steps of 64.  Tiles go global -> LDS
-// directly (buffer_load_dwordx4 ... lds: each lane fetches 16 bytes and the hardware stores the wave's 64
-// chunks contiguously at M0 + lane*16), two LDS stages.  The loop is skewed: the single barrier of an
-// iteration sits BEFORE its last k-step, so the first fragments of the next tile are read while the matrix
-// cores work on that last step, and the refill of the stage that was just drained (tile kt+2) is issued
-// right after the barrier and has a full iteration to land.
+// Shape of a workgroup.  FOUR waves, one per SIMD, each with all 512 registers of a lane: the 256
+// accumulation registers hold the wave's accumulators (up to 128x128 outputs), the architectural registers
+// hold two sets of operand fragments and the addresses.  The accumulators are driven by inline assembly in a
+// fixed instruction order: the compiler never sees them, so it cannot copy, rotate or spill them, and the LDS
+// reads and direct loads sit at chosen places between the MFMAs.  One workgroup per CU (LDS-bound), the
+// kernel is persistent over output tiles.
 //
-// Two forms share the code.  The 256x256 tile runs with FOUR waves, one per SIMD, 128x128 outputs and all
-// 512 registers per lane: 256 accumulation registers hold the accumulators and are driven by inline
-// assembly in a fixed instruction order (LDS traffic per FLOP is a third lower than with eight waves, and
-// the compiler cannot shuffle or spill the accumulators).  The narrower tiles (256x160, 256x128) run with
-// EIGHT waves, two per SIMD, compiler-scheduled builtins.
+// Pipeline.  K is walked in steps of 64.  Tiles go global -> LDS directly (buffer_load_dwordx4 ... lds: each
+// lane fetches 16 bytes and the hardware stores the wave's 64 chunks contiguously at M0 + lane*16).  The loop
+// is skewed: the single barrier of an iteration sits BEFORE its last k-step, so the first fragments of the
+// next K tile are read while the matrix cores work on that last step.  The four waves share the CU's one
+// memory pipeline, and a K tile costs it about half an iteration, so the direct loads must not come in
+// bursts: LDS is organised as a RING with more than two K tiles of room, which lets the loads of a K tile be
+// issued in two different half-iterations, evenly spaced between the MFMAs, and gives them a whole
+// iteration more to land (the weights of an encoder block come from HBM, not from a cache):
+//   * 256x256 tile: five 32 KB units = A(kt), W(kt), A(kt+1), W(kt+1) and one in flight.  A(kt+2) is
+//     requested in the first half of iteration kt, W(kt+2) in the second half, into the unit that the
+//     barrier has just freed.
+//   * narrower tiles (256x160, 256x128, 128x192): three whole stages.  The second half of K tile kt+2 is
+//     requested in the first half of iteration kt, the first half of K tile kt+3 in the second half.
+// The sequence of K tiles runs on across output tiles: the next output tile's first K tiles are requested
+// in the last iterations of the current one and travel while the epilogue runs.  Waits use the in-order
+// completion of loads: "K tile j has landed" == "at most the loads issued after it are outstanding".
 //
 // Matrix cores.  v_mfma_f32_16x16x32_bf16 (k = 32 per instruction: each accumulator register is touched
 // half as often as with the 32x32x16 form).  W rows are the MFMA "A" operand and activation rows the "B"
@@ -41,11 +52,14 @@ namespace {
 using namespace csgemm;
 
 constexpr int CS_EPI_BIAS_POS = 100;  // internal: CS_EPI_BIAS plus the (row % pos_period) position addend
+constexpr int NW = 4;                 // waves per workgroup, one per SIMD
+constexpr int LDS_BYTES = 160 * 1024;
 
-// s_waitcnt with only vmcnt set (lgkmcnt/expcnt left at "don't wait"), gfx9 encoding.
-#define CS_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt((((n) & 0xF) | (((n) >> 4) << 14)) | 0x0F70)
+// s_waitcnt encodings (gfx9): vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8.
+constexpr int waitcnt_vm(int n) { return ((n & 0xF) | ((n >> 4) << 14)) | 0x0F70; }       // vmcnt(n) only
+constexpr int waitcnt_vm_lgkm0(int n) { return ((n & 0xF) | ((n >> 4) << 14)) | 0x0070; }  // vmcnt(n) lgkmcnt(0)
+constexpr int WAITCNT_LGKM0 = 0xC07F;                                                      // lgkmcnt(0) only
 
-typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) void lds_void_t;
 
 // Workgroup barrier without the full memory fence of __syncthreads(): the callers order LDS traffic with
@@ -94,37 +108,41 @@ CS_DEVICE void static_for(F&& f) {
   static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
+// LDS organisation of a tile shape (shared by the kernel and its launcher).
+template <int BM, int BN>
+struct RingShape {
+  static constexpr int A_BYTES = BM * BK * 2, W_BYTES = BN * BK * 2;
+  static constexpr bool FIVE_UNITS = A_BYTES == W_BYTES && 5 * A_BYTES <= LDS_BYTES && 3 * (A_BYTES + W_BYTES) > LDS_BYTES;
+  static constexpr int BYTES = FIVE_UNITS ? 5 * A_BYTES : 3 * (A_BYTES + W_BYTES);
+  static_assert(BYTES <= LDS_BYTES, "tile does not fit a ring");
+};
+
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
-__global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const CsGemmArgs p, const int stagger) {
+__global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  constexpr int NW = WAVES_M * WAVES_N;
-  static_assert(NW == 8 || NW == 4, "8 waves (2 per SIMD, 256 registers each) or 4 waves (1 per SIMD, 512 registers)");
-  static_assert(NW == 8 || (BM / WAVES_M) * (BN / WAVES_N) <= 128 * 128, "the 4-wave form has 256 accumulation registers");
-  constexpr int A_BYTES = BM * BK * 2;
-  constexpr int W_BYTES = BN * BK * 2;
+  static_assert(WAVES_M * WAVES_N == NW, "four waves, one per SIMD");
+  using Ring = RingShape<BM, BN>;
+  constexpr int A_BYTES = Ring::A_BYTES, W_BYTES = Ring::W_BYTES;
+  constexpr bool RING5 = Ring::FIVE_UNITS;
+  // Byte offsets of operand tile slots.  Three-stage ring: slot s holds A at s*STAGE and W behind it.
+  // Five-unit ring: every unit is one operand tile.
   constexpr int STAGE = A_BYTES + W_BYTES;
   constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
   static_assert(WTM % 16 == 0 && WTN % 16 == 0 && BM % 8 == 0 && BN % 8 == 0, "tile shape");
   constexpr int MT = WTM / 16, NT = WTN / 16;
+  static_assert(MT * NT * 4 <= 256, "the accumulators of a wave live in its 256 accumulation registers");
   // W fragments come in groups of G: fragment j, fragment row 4q+r holds W row (j/G)*16G + q*4G + (j%G)*4 + r of
   // the wave's rows, so a lane owns 4G consecutive output columns per group and the four lanes q = 0..3 of
   // one output row own 16G consecutive columns.
   constexpr int G = (NT % 2 == 0) ? 2 : NT;
   auto piece_col = [](int j) { return (j / G) * 16 * G + (j % G) * 4; };  // first column of fragment j's piece
-  // Pinning a fine MFMA/LDS interleave costs registers; only tiles whose accumulators and two fragment
-  // sets leave room for it use it (the 256x256 tile would spill).
-  constexpr bool ILV = NW == 4 || (MT * NT * 4 + (MT + NT) * 8) <= 176;
-  constexpr int A_BLK = BM / 8, W_BLK = BN / 8;            // 8-row blocks = direct loads per stage
-  constexpr int A_LD = (A_BLK + NW - 1) / NW, W_LD = (W_BLK + NW - 1) / NW;  // per wave
-  // Tiles whose stage is small enough get a ring of THREE stages (one-wave-per-SIMD form only): the direct
-  // loads of a K tile are then spread over two half-iterations and have a whole iteration more to land.
-  constexpr bool RING = NW == 4 && 3 * STAGE <= 160 * 1024;
-  constexpr int NLD = A_LD + W_LD, H1 = NLD / 2, H2 = NLD - H1;  // direct loads per wave and K tile; its two halves
-  // The 256x256 tile (two 32 KB operand tiles per K tile) uses the whole 160 KB as a ring of FIVE 32 KB units
-  // holding A(kt), W(kt), A(kt+1), W(kt+1) and one unit in flight: A(kt+2) is requested in the first half
-  // of iteration kt, W(kt+2) in the second half into the unit the barrier has just freed.
-  constexpr bool RING5 = NW == 4 && !RING && A_BYTES == W_BYTES && 5 * A_BYTES <= 160 * 1024;
-  constexpr int UNIT = A_BYTES;
+  constexpr int A_BLK = BM / 8, W_BLK = BN / 8;  // 8-row blocks = direct loads per operand tile
+  static_assert(A_BLK % NW == 0 && W_BLK % NW == 0, "every wave issues the same number of direct loads");
+  constexpr int A_LD = A_BLK / NW, W_LD = W_BLK / NW;  // per wave
+  constexpr int NLD = A_LD + W_LD;                      // direct loads per wave and K tile
+  constexpr int NFR = MT + NT;                          // fragment reads per wave and k-step
+  constexpr int NMFMA = MT * NT;                        // MFMAs per wave and k-step
+  static_assert(2 * NFR <= NMFMA, "one slot after an MFMA per LDS read");
 
   // ---- tile coordinates of virtual block vb in [0, tiles): XCD-aware remap (workgroup i runs on XCD i%8,
   //      and the persistent stride gridDim.x is a multiple of 8, so a workgroup's tiles stay on its XCD),
@@ -143,17 +161,22 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
     n0 = (within / rows_in_band) * BN;
   };
 
-  if constexpr (NW == 4) asm volatile("" ::: CS_ALL_ACC_REGS);  // accounts a[0:255] to this kernel
+  // The accumulation registers a[0:255] belong to the inline assembly below (MFMAs in the main loop,
+  // v_accvgpr_read in the epilogue), accumulator (i, j) in a[4(i*NT+j) .. +3].  The compiler is told once
+  // that they are in use, so that the kernel's register allocation covers them; it has no reason to touch
+  // them itself as long as the rest of the kernel fits the 256 architectural registers, and the build
+  // checks the generated code for exactly that.
+  asm volatile("" ::: CS_ALL_ACC_REGS);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave % WAVES_M, wn = wave / WAVES_M;
 
-  // ---- global sources of the direct loads.  Row block rb = j*8 + wave covers tile rows 8rb..8rb+7; the
-  //      lane lands in slot lane%8 of row 8rb + lane/8 and fetches chunk (lane%8) ^ key(row).
+  // ---- global sources of the direct loads.  Row block rb = j*NW + wave covers tile rows 8rb..8rb+7; the
+  //      lane lands in slot lane%8 of row 8rb + lane/8 and fetches chunk (lane%8) ^ key(row).  Buffer
+  //      loads: a 32-bit per-lane byte offset plus a scalar K offset on a scalar descriptor, so an address
+  //      costs one register and no vector arithmetic.
   const int l_row = lane >> 3, l_slot = lane & 7;
-  // 32-bit byte offsets from the (scalar) matrix bases: half the registers of full pointers, and the K
-  // advance is one scalar add per operand instead of a vector add per load.
   uint32_t a_src[A_LD];
   uint32_t w_src[W_LD];
   auto setup_sources = [&](int m0, int n0) {
@@ -174,33 +197,25 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   };
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, -1, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void*)p.W, 0, -1, 0x00020000);
-  // Direct loads are buffer loads: a 32-bit per-lane byte offset plus a scalar K offset on a scalar descriptor,
-  // so an address costs one register and no vector arithmetic.
+  // (The builtin is called from non-generic lambdas on purpose: inside a generic lambda the host pass of the
+  // compiler rejects the device-only builtin, silently drops the kernel and leaves its launch stub undefined.)
   auto load_a = [&](int kt, char* lds_dst, uint32_t off) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t*)lds_dst, 16, off, kt * (BK * 2), 0, 0);
   };
   auto load_w = [&](int kt, char* lds_dst, uint32_t off) {
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void_t*)lds_dst, 16, off, kt * (BK * 2), 0, 0);
   };
-  // one direct load of K tile kt into `stage`: IDX < A_LD activation row blocks, then the W row blocks
-  auto issue_one_load = [&](int kt, int stage, auto idx_c) {
+  // Direct load number IDX (A row blocks first, then W row blocks) of K tile kt; a_base / w_base are the
+  // LDS byte offsets of the operand tiles it goes to.
+  auto direct_load = [&](int kt, int a_base, int w_base, auto idx_c) {
     constexpr int IDX = decltype(idx_c)::value;
-    char* As = smem + stage * STAGE;
     if constexpr (IDX < A_LD) {
-      if ((A_BLK % NW == 0) || IDX * NW + wave < A_BLK) load_a(kt, As + (IDX * NW + wave) * 1024, a_src[IDX]);
+      load_a(kt, smem + a_base + (IDX * NW + wave) * 1024, a_src[IDX]);
     } else {
       constexpr int J = IDX - A_LD;
-      if ((W_BLK % NW == 0) || J * NW + wave < W_BLK) load_w(kt, As + A_BYTES + (J * NW + wave) * 1024, w_src[J]);
+      load_w(kt, smem + w_base + (J * NW + wave) * 1024, w_src[J]);
     }
   };
-  // five-unit ring: one direct load of operand tile (A or W) of K tile kt into ring unit `slot`
-  auto issue_unit_load = [&](int kt, auto is_w_c, int slot, auto idx_c) {
-    constexpr int IDX = decltype(idx_c)::value;
-    char* dst = smem + slot * UNIT + (IDX * NW + wave) * 1024;
-    if constexpr (decltype(is_w_c)::value) load_w(kt, dst, w_src[IDX]);
-    else load_a(kt, dst, a_src[IDX]);
-  };
-  auto issue_loads = [&](int kt, int stage) { static_for<A_LD + W_LD>([&](auto n) { issue_one_load(kt, stage, n); }); };
 
   // ---- fragment addressing.  Lane (a = lane%16, kq = lane/16) reads chunk ks*4 + kq of its fragment row.
   //      Both keys depend only on the lane, so the per-lane part of the address is loop-invariant.
@@ -208,59 +223,27 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
   const int fq = fa >> 2, fr = fa & 3;
   const int x_key = (fa >> 1) & 7;
   const int w_key = (fq << 1) | ((fr >> 1) & 1);
-  // byte offset inside a stage of fragment (i or j), k-step ks: row*128 + (((ks*4 + kq) ^ key) << 4)
+  // byte offset inside an operand tile of fragment (i or j), k-step ks: row*128 + (((ks*4 + kq) ^ key) << 4)
   int x_off[2], w_off[2];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
     x_off[ks] = (wm * WTM + fa) * 128 + (((ks * 4 + kq) ^ x_key) << 4);
-    w_off[ks] = A_BYTES + (wn * WTN + fq * (4 * G) + fr) * 128 + (((ks * 4 + kq) ^ w_key) << 4);
+    w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * 128 + (((ks * 4 + kq) ^ w_key) << 4);
   }
-
-  f32x4_t acc[MT][NT];
   bf16x8_t wf[2][NT], xf[2][MT];
-  auto read_frags = [&](int stage, int ks, int b) {
-    const char* base = smem + stage * STAGE;
-#pragma unroll
-    for (int j = 0; j < NT; ++j) wf[b][j] = *(const bf16x8_t*)(base + w_off[ks] + piece_col(j) * 128);
-#pragma unroll
-    for (int i = 0; i < MT; ++i) xf[b][i] = *(const bf16x8_t*)(base + x_off[ks] + i * 16 * 128);
-  };
-  auto mfmas = [&](int b) {
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[b][j], xf[b][i], acc[i][j], 0, 0, 0);
-  };
-
-  // ---- one-wave-per-SIMD form (NW == 4, 8x8 fragments per wave, 512 registers per lane).  The 64
-  //      accumulators live in the accumulation registers a[0:255], accumulator (i, j) in a[4(8i+j) .. +3],
-  //      and are touched ONLY by the inline-asm statements below (MFMAs here, v_accvgpr_read in the
-  //      epilogue): the compiler sees no accumulator values at all, so it cannot copy, rotate or spill them.
-  //      It is told once that the 256 registers are in use (the clobber list at the top of the kernel) so
-  //      that the kernel's register allocation covers them, and it has no reason to use them itself as long
-  //      as the rest of the kernel fits the 256 architectural registers (the build checks the generated
-  //      code for that).  asm volatile statements keep their program order, so the hook called after each
-  //      MFMA places LDS reads and direct loads at fixed points of the instruction stream.  The first k-step
-  //      of an output tile takes a zero addend, which saves clearing the accumulators.
-  auto read_one = [&](int stage, int ks, int b, auto idx_c) {
+  // fragment read number IDX (W fragments first, then activation fragments) of k-step ks into set b
+  auto read_frag = [&](int a_base, int w_base, int ks, int b, auto idx_c) {
     constexpr int IDX = decltype(idx_c)::value;
-    const char* base = smem + stage * STAGE;
-    if constexpr (IDX < NT) wf[b][IDX] = *(const bf16x8_t*)(base + w_off[ks] + piece_col(IDX) * 128);
-    else xf[b][IDX - NT] = *(const bf16x8_t*)(base + x_off[ks] + (IDX - NT) * 16 * 128);
+    if constexpr (IDX < NT) wf[b][IDX] = *(const bf16x8_t*)(smem + w_base + w_off[ks] + piece_col(IDX) * 128);
+    else xf[b][IDX - NT] = *(const bf16x8_t*)(smem + a_base + x_off[ks] + (IDX - NT) * 16 * 128);
   };
-  // five-unit ring: fragment IDX of k-step ks from the units holding the A and W tiles
-  auto read_one5 = [&](int slot_a, int slot_w, int ks, int b, auto idx_c) {
-    constexpr int IDX = decltype(idx_c)::value;
-    if constexpr (IDX < NT)
-      wf[b][IDX] = *(const bf16x8_t*)(smem + slot_w * UNIT + (w_off[ks] - A_BYTES) + piece_col(IDX) * 128);
-    else
-      xf[b][IDX - NT] = *(const bf16x8_t*)(smem + slot_a * UNIT + x_off[ks] + (IDX - NT) * 16 * 128);
-  };
-  auto mfmas_pinned = [&](auto b_c, auto zero_c, auto&& hook) {
+  // The MFMAs of one k-step on fragment set B, in program order (asm volatile statements keep it), with a
+  // hook call after each: that is where LDS reads and direct loads are placed.  ZERO: the first k-step of an
+  // output tile takes a zero addend, which saves clearing the accumulators.
+  auto mfmas = [&](auto b_c, auto zero_c, auto&& hook) {
     constexpr int B = decltype(b_c)::value;
     constexpr bool ZERO = decltype(zero_c)::value;
-    static_for<MT * NT>([&](auto n) {
+    static_for<NMFMA>([&](auto n) {
       constexpr int N = decltype(n)::value, I = N / NT, J = N % NT, R = N * 4;
       if constexpr (ZERO)
         asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(wf[B][J]), "v"(xf[B][I]), "n"(R), "n"(R + 3));
@@ -270,415 +253,261 @@ __global__ __launch_bounds__(64 * WAVES_M * WAVES_N) void gemm_fast_kernel(const
     });
   };
 
-  const int nk = p.K / BK;
+  // ---- ring state.  `ring` is the slot of the current K tile: a stage number (three-stage ring) or the
+  //      unit of A(kt) with W(kt), A(kt+1), W(kt+1), A(kt+2) following cyclically (five-unit ring).  It
+  //      keeps rotating across output tiles.
+  constexpr int RING_N = RING5 ? 5 : 3;
+  auto slot_add = [](int s, int d) { return (s + d) % RING_N; };
+  auto a_base_of = [&](int tile_ahead, int ring) {  // LDS offset of the A tile of K tile kt + tile_ahead
+    return RING5 ? slot_add(ring, 2 * tile_ahead) * A_BYTES : slot_add(ring, tile_ahead) * STAGE;
+  };
+  auto w_base_of = [&](int tile_ahead, int ring) {
+    return RING5 ? slot_add(ring, 2 * tile_ahead + 1) * A_BYTES : slot_add(ring, tile_ahead) * STAGE + A_BYTES;
+  };
+  // Loads of a K tile are issued in two portions; PA of them in the first half of an iteration.
+  // Five-unit ring: A(kt+2) in the first half, W(kt+2) in the second (same K tile, AHEAD_B == AHEAD_A).
+  // Three-stage ring: the second portion of K tile kt+2 in the first half, the first portion of K tile kt+3
+  // in the second half.
+  constexpr int PA = RING5 ? A_LD : NLD - NLD / 2;  // loads issued in a first half
+  constexpr int PB = NLD - PA;                       // loads issued in a second half
+  constexpr int PA_FIRST = RING5 ? 0 : PB;           // index of the first load of the first-half portion
+  constexpr int PB_FIRST = RING5 ? A_LD : 0;
+  constexpr int AHEAD_A = 2, AHEAD_B = RING5 ? 2 : 3;
+  constexpr int EA = NMFMA / PA, EB = NMFMA / PB;    // MFMAs per direct load in each half
+  static_assert(EA >= 1 && EB >= 1, "one slot after an MFMA per direct load");
+  // Loads outstanding by design at the two wait points: everything issued after the K tile that is needed.
+  constexpr int PENDING_AT_BARRIER = RING5 ? PA : NLD;           // after K tile kt+1
+  constexpr int PENDING_AT_TILE_START = RING5 ? NLD : NLD + PB;  // after K tile 0 of an output tile
+
+  const int nk = p.K / BK;  // >= 3 (checked on the host)
   int vb = blockIdx.x;
-  if (stagger > 0) {
-    // Persistent launches: spread the 32 workgroups of each XCD in time (10 ns ticks per slot) so that the
-    // output bursts of the 256 CUs do not hit HBM in the same few microseconds of every round.
-    const long long until = wall_clock64() + (long long)((blockIdx.x >> 3) & 31) * stagger;
-    while (wall_clock64() < until) __builtin_amdgcn_s_sleep(4);
-  }
   int m0, n0;
   tile_origin(vb, m0, n0);
   setup_sources(m0, n0);
-  if constexpr (RING5) {  // units 0..3 = A(0), W(0), A(1), W(1); nk >= 3 (checked on the host)
-    static_for<A_LD>([&](auto n) { issue_unit_load(0, std::false_type{}, 0, n); });
-    static_for<W_LD>([&](auto n) { issue_unit_load(0, std::true_type{}, 1, n); });
-    static_for<A_LD>([&](auto n) { issue_unit_load(1, std::false_type{}, 2, n); });
-    static_for<W_LD>([&](auto n) { issue_unit_load(1, std::true_type{}, 3, n); });
-  } else {
-    issue_loads(0, 0);
-    if (nk > 1) issue_loads(1, 1);
-  }
-  int ua = 0;  // five-unit ring: unit of A(kt); W(kt), A(kt+1), W(kt+1), A(kt+2) follow cyclically
-  if constexpr (RING) static_for<H1>([&](auto n) { issue_one_load(2, 2, n); });  // nk >= 3 (checked on the host)
-  int st = 0;  // ring form: LDS stage of the current K tile; keeps rotating across output tiles
+  int ring = 0;
+  // in flight before the first iteration: K tiles 0 and 1, and what a second half would have requested
+  static_for<NLD>([&](auto n) { direct_load(0, a_base_of(0, ring), w_base_of(0, ring), n); });
+  static_for<NLD>([&](auto n) { direct_load(1, a_base_of(1, ring), w_base_of(1, ring), n); });
+  if constexpr (!RING5)
+    static_for<PB>([&](auto n) { direct_load(2, a_base_of(2, ring), w_base_of(2, ring), ic<PB_FIRST + decltype(n)::value>{}); });
 
-  // Persistent loop over this workgroup's tiles (vb, vb + gridDim.x, ...).  The first two K tiles of the
-  // NEXT output tile are requested inside the last K iteration of the current one, so they travel while
-  // the epilogue runs.
-  for (;;) {
-  if constexpr (NW == 8) {
-#pragma unroll
-    for (int i = 0; i < MT; ++i)
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
-  }
-  const int vb_next = vb + gridDim.x;
-  const bool has_next = vb_next < ntiles;
-  int m0_next = 0, n0_next = 0;
+  for (;;) {  // persistent loop over this workgroup's output tiles (vb, vb + gridDim.x, ...)
+    const int vb_next = vb + gridDim.x;
+    const bool has_next = vb_next < ntiles;
+    int m0_next = 0, n0_next = 0;
 
-  CS_TS(0);
-  if constexpr (RING5) {
-    CS_WAIT_VMCNT(NLD);  // K tile 0 has landed once at most K tile 1's loads are outstanding
+    CS_TS(0);
+    // K tile 0 has landed once at most the loads issued after it are outstanding.  (Loads complete in
+    // order; stores of the previous epilogue that are still in flight only make this wait longer.)
+    __builtin_amdgcn_s_waitcnt(waitcnt_vm(PENDING_AT_TILE_START));
     wg_barrier();
     CS_TS(1);
-    static_for<MT + NT>([&](auto n) { read_one5(ua, (ua + 1) % 5, 0, 0, n); });
-  } else if constexpr (RING) {
-    // K tile 0 has landed once at most the loads issued after it are outstanding: K tile 1 and the first
-    // half of K tile 2.  (Loads complete in order; stores of the previous epilogue that are still in
-    // flight only make this wait longer, never shorter.)
-    CS_WAIT_VMCNT(NLD + H1);
-    wg_barrier();
-    CS_TS(1);
-    read_frags(st, 0, 0);
-  } else {
-    CS_WAIT_VMCNT(0);  // K tiles 0 and 1 of this output tile (and the previous tile's stores)
-    wg_barrier();
-    CS_TS(1);
-    read_frags(0, 0, 0);
-  }
+    static_for<NFR>([&](auto n) { read_frag(a_base_of(0, ring), w_base_of(0, ring), 0, 0, n); });
 
-  // Ring form of one K iteration.  MODE 0: steady state; 3, 2, 1: that many iterations before the end of
-  // the output tile, where the loads switch over to the next output tile's first K tiles.  In iteration kt
-  // the first half requests the SECOND half of K tile kt+2 (stage freed one barrier ago) and the second
-  // half requests the FIRST half of K tile kt+3 (the stage this iteration's barrier has just freed).
-  auto body_ring = [&](int kt, auto first_c, auto mode_c) {
-    constexpr bool FIRST = decltype(first_c)::value;
-    constexpr int MODE = decltype(mode_c)::value;
-    constexpr int NFR = MT + NT;
-    constexpr int EA = (MT * NT) / H2, EB = (MT * NT) / H1;  // MFMAs per direct load in each half
-    static_assert(2 * NFR <= MT * NT && EA >= 1 && EB >= 1, "one slot after an MFMA per LDS read / direct load");
-    const int s_cur = st, s_nxt = st == 2 ? 0 : st + 1, s_prv = st == 0 ? 2 : st - 1;
-    const int k_a = (MODE == 0 || MODE == 3) ? kt + 2 : 2 - MODE;  // MODE 2 -> next tile's 0, MODE 1 -> 1
-    const int k_b = MODE == 0 ? kt + 3 : 3 - MODE;                 // MODE 3 -> next tile's 0, 2 -> 1, 1 -> 2
-    __builtin_amdgcn_sched_barrier(0);
-    mfmas_pinned(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
-      constexpr int N = decltype(n)::value;
-      if constexpr (N < NFR) read_one(s_cur, 1, 1, n);
-      if constexpr (N < EA * H2 && N % EA == EA - 1) {
-        if constexpr (MODE == 0 || MODE == 3) issue_one_load(k_a, s_prv, ic<H1 + N / EA>{});
-        else if (has_next) issue_one_load(k_a, s_prv, ic<H1 + N / EA>{});
-      }
-    });
-    // K tile kt+1 has landed once at most the NLD loads issued after it (K tile kt+2) are outstanding
-    if constexpr (MODE == 1) {
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): nothing more is read from LDS for this output tile
-    } else if (MODE == 2 && !has_next) {
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    } else {
-      __builtin_amdgcn_s_waitcnt(((NLD & 0xF) | ((NLD >> 4) << 14)) | 0x0070);  // vmcnt(NLD) lgkmcnt(0)
-    }
-    wg_barrier();
-    if constexpr (MODE == 3) {
-      if (has_next) {
-        tile_origin(vb_next, m0_next, n0_next);
-        setup_sources(m0_next, n0_next);
-      }
-    }
-    mfmas_pinned(ic<1>{}, std::false_type{}, [&](auto n) {
-      constexpr int N = decltype(n)::value;
-      if constexpr (MODE != 1 && N < 2 * NFR && N % 2 == 0) read_one(s_nxt, 0, 0, ic<N / 2>{});
-      if constexpr (N < EB * H1 && N % EB == EB - 1) {
-        if constexpr (MODE == 0) issue_one_load(k_b, s_cur, ic<N / EB>{});
-        else if (has_next) issue_one_load(k_b, s_cur, ic<N / EB>{});
-      }
-    });
-    st = s_nxt;
-  };
-
-  // Five-unit-ring form of one K iteration.  MODE 0: steady state; 2, 1: that many iterations before the
-  // end of the output tile, where the loads belong to the next output tile.
-  auto body_ring5 = [&](int kt, auto first_c, auto mode_c) {
-    constexpr bool FIRST = decltype(first_c)::value;
-    constexpr int MODE = decltype(mode_c)::value;
-    constexpr int NFR = MT + NT;
-    constexpr int EA = (MT * NT) / A_LD, EB = (MT * NT) / W_LD;
-    static_assert(2 * NFR <= MT * NT, "one slot after an MFMA per LDS read");
-    const int u_a0 = ua, u_w0 = (ua + 1) % 5, u_a1 = (ua + 2) % 5, u_w1 = (ua + 3) % 5, u_a2 = (ua + 4) % 5;
-    const int k_ld = MODE == 0 ? kt + 2 : 2 - MODE;  // MODE 2 -> next tile's K tile 0, MODE 1 -> 1
-    if constexpr (MODE == 2) {
-      if (has_next) {  // every load of this output tile has been issued
-        tile_origin(vb_next, m0_next, n0_next);
-        setup_sources(m0_next, n0_next);
-      }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    mfmas_pinned(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
-      constexpr int N = decltype(n)::value;
-      if constexpr (N < NFR) read_one5(u_a0, u_w0, 1, 1, n);
-      if constexpr (N < EA * A_LD && N % EA == EA - 1) {
-        if constexpr (MODE == 0) issue_unit_load(k_ld, std::false_type{}, u_a2, ic<N / EA>{});
-        else if (has_next) issue_unit_load(k_ld, std::false_type{}, u_a2, ic<N / EA>{});
-      }
-    });
-    // K tile kt+1 has landed once at most the A_LD loads issued after it (A of K tile kt+2) are outstanding
-    if constexpr (MODE == 1) {
-      __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): nothing more is read from LDS for this output tile
-    } else if (MODE == 2 && !has_next) {
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    } else {
-      __builtin_amdgcn_s_waitcnt(((A_LD & 0xF) | ((A_LD >> 4) << 14)) | 0x0070);  // vmcnt(A_LD) lgkmcnt(0)
-    }
-    wg_barrier();
-    mfmas_pinned(ic<1>{}, std::false_type{}, [&](auto n) {
-      constexpr int N = decltype(n)::value;
-      if constexpr (MODE != 1 && N < 2 * NFR && N % 2 == 0) read_one5(u_a1, u_w1, 0, 0, ic<N / 2>{});
-      if constexpr (N < EB * W_LD && N % EB == EB - 1) {
-        if constexpr (MODE == 0) issue_unit_load(k_ld, std::true_type{}, u_a0, ic<N / EB>{});
-        else if (has_next) issue_unit_load(k_ld, std::true_type{}, u_a0, ic<N / EB>{});
-      }
-    });
-    ua = u_a1;
-  };
-
-  // One K iteration.  LOADS: tile kt+2 exists and is fetched; NEXT: tile kt+1 exists; LAST: final iteration.
-  auto body = [&](int kt, auto first_c, auto loads_c, auto next_c) {
-    constexpr bool FIRST = decltype(first_c)::value, LOADS = decltype(loads_c)::value, NEXT = decltype(next_c)::value;
-    const int cur = kt & 1;
-    __builtin_amdgcn_sched_barrier(0);
-    if constexpr (NW == 4) {
-      constexpr int NLD = A_LD + W_LD, NFR = MT + NT;
-      static_assert(2 * NLD <= MT * NT && 2 * NFR <= MT * NT, "one slot after an MFMA per LDS read / direct load");
-      // first k-step; meanwhile the fragments of the second k-step
-      mfmas_pinned(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
+    // One K iteration.  TAIL 0: steady state.  TAIL t > 0: t iterations before the end of the output tile,
+    // where the K tiles being requested belong to the next output tile (if there is one).
+    auto iteration = [&](int kt, auto first_c, auto tail_c) {
+      constexpr bool FIRST = decltype(first_c)::value;
+      constexpr int TAIL = decltype(tail_c)::value;
+      // Does the portion requested in each half belong to this output tile?  K tile kt + AHEAD exists iff
+      // AHEAD < TAIL (or TAIL == 0).
+      constexpr bool CUR_A = TAIL == 0 || AHEAD_A < TAIL, CUR_B = TAIL == 0 || AHEAD_B < TAIL;
+      const int k_a = CUR_A ? kt + AHEAD_A : AHEAD_A - TAIL;  // K tile number inside its output tile
+      const int k_b = CUR_B ? kt + AHEAD_B : AHEAD_B - TAIL;
+      // The sources switch to the next output tile once, right before its first load is issued: that is the
+      // second-half portion when it runs further ahead than the first-half portion, else the first-half one.
+      constexpr bool SWITCH_BEFORE_B = AHEAD_B > AHEAD_A && TAIL == AHEAD_B;
+      constexpr bool SWITCH_BEFORE_A = AHEAD_B == AHEAD_A && TAIL == AHEAD_A;
+      auto switch_sources = [&]() {
+        if (has_next) {
+          tile_origin(vb_next, m0_next, n0_next);
+          setup_sources(m0_next, n0_next);
+        }
+      };
+      if constexpr (SWITCH_BEFORE_A) switch_sources();
+      __builtin_amdgcn_sched_barrier(0);
+      // first k-step; meanwhile the fragments of the second k-step and the first-half portion of loads
+      mfmas(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
         constexpr int N = decltype(n)::value;
-        if constexpr (N < NFR) read_one(cur, 1, 1, n);
-      });
-      // K tile kt+1 (requested one iteration ago) has landed in this wave's part of the other stage, and
-      // this wave has received its last fragments of the current stage
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-      wg_barrier();
-      if (!NEXT && has_next) {
-        tile_origin(vb_next, m0_next, n0_next);
-        setup_sources(m0_next, n0_next);
-      }
-      // second k-step; meanwhile the first fragments of K tile kt+1 and the request for K tile kt+2 into
-      // the stage that was just drained (or, at the end, for the next output tile's first two K tiles)
-      mfmas_pinned(ic<1>{}, std::false_type{}, [&](auto n) {
-        constexpr int N = decltype(n)::value;
-        if constexpr (NEXT && N < 2 * NFR && N % 2 == 0) read_one(cur ^ 1, 0, 0, ic<N / 2>{});
-        // four waves share the CU's one memory pipeline: space the direct loads as widely as the half allows
-        constexpr int LD_EVERY = (MT * NT) / NLD >= 4 ? 4 : ((MT * NT) / NLD >= 3 ? 3 : 2);
-        if constexpr (LOADS && N < LD_EVERY * NLD && N % LD_EVERY == LD_EVERY - 1)
-          issue_one_load(kt + 2, cur, ic<N / LD_EVERY>{});
-        constexpr int PF_EVERY = (MT * NT) / (2 * NLD);
-        if constexpr (!NEXT && N < PF_EVERY * 2 * NLD && N % PF_EVERY == PF_EVERY - 1) {
-          constexpr int L = N / PF_EVERY;
-          if (has_next && (nk > 1 || L < NLD)) issue_one_load(L / NLD, L / NLD, ic<L % NLD>{});
+        if constexpr (N < NFR) read_frag(a_base_of(0, ring), w_base_of(0, ring), 1, 1, n);
+        if constexpr (N < EA * PA && N % EA == EA - 1) {
+          auto ld = [&]() { direct_load(k_a, a_base_of(AHEAD_A, ring), w_base_of(AHEAD_A, ring), ic<PA_FIRST + N / EA>{}); };
+          if constexpr (CUR_A) ld();
+          else if (has_next) ld();
         }
       });
-      return;
-    }
-    read_frags(cur, 1, 1);
-    mfmas(0);
-    // Issue order: one fragment read after each of the first MFMAs, so the matrix cores never wait for
-    // the wave to get through a block of LDS instructions.
-    if (ILV) {
-#pragma unroll
-      for (int r = 0; r < MT + NT; ++r) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // DS read
+      // K tile kt+1 has landed in this wave's part of LDS once at most the loads issued after it are
+      // outstanding, and this wave has received its last fragments of K tile kt.
+      if constexpr (TAIL == 1) {
+        __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);  // nothing more is read from LDS for this output tile
+      } else if (!CUR_A && !has_next) {
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));  // nothing was requested after K tile kt+1
+      } else {
+        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(PENDING_AT_BARRIER));
       }
-      __builtin_amdgcn_sched_group_barrier(0x008, MT * NT - (MT + NT), 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-    // Tile kt+1 (issued one iteration ago) must have landed in every wave's part of the other stage, and
-    // every wave must have received its last fragments of this stage before it is refilled.
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-    wg_barrier();
-    __builtin_amdgcn_sched_barrier(0);
-    if (LOADS) issue_loads(kt + 2, cur);
-    if (NEXT) read_frags(cur ^ 1, 0, 0);
-    if (!NEXT && has_next) {  // both stages are free now: start on the next output tile
-      tile_origin(vb_next, m0_next, n0_next);
-      setup_sources(m0_next, n0_next);
-      issue_loads(0, 0);
-      if (nk > 1) issue_loads(1, 1);
-    }
-    mfmas(1);
-    if (ILV && LOADS && NEXT) {
-      constexpr int NLD = A_LD + W_LD;
-#pragma unroll
-      for (int r = 0; r < NLD; ++r) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
-        __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // direct-to-LDS load
-      }
-#pragma unroll
-      for (int r = 0; r < MT + NT; ++r) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-      __builtin_amdgcn_sched_group_barrier(0x008, MT * NT - NLD - (MT + NT), 0);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  };
-  if constexpr (RING5) {
-    constexpr std::true_type T{};
-    constexpr std::false_type F{};
-    body_ring5(0, T, ic<0>{});
-    for (int kt = 1; kt < nk - 2; ++kt) body_ring5(kt, F, ic<0>{});
-    body_ring5(nk - 2, F, ic<2>{});
-    body_ring5(nk - 1, F, ic<1>{});
-  } else if constexpr (RING) {
-    constexpr std::true_type T{};
-    constexpr std::false_type F{};
-    if (nk == 3) {
-      body_ring(0, T, ic<3>{});
-    } else {
-      body_ring(0, T, ic<0>{});
-      int kt = 1;
-      for (; kt < nk - 3; ++kt) body_ring(kt, F, ic<0>{});
-      body_ring(nk - 3, F, ic<3>{});
-    }
-    body_ring(nk - 2, F, ic<2>{});
-    body_ring(nk - 1, F, ic<1>{});
-  } else {
-    constexpr std::true_type T{};
-    constexpr std::false_type F{};
-    if (nk >= 3) {
-      body(0, T, T, T);
-      int kt = 1;
-      for (; kt + 2 < nk; ++kt) body(kt, F, T, T);
-      body(kt, F, F, T);
-      body(kt + 1, F, F, F);
-    } else if (nk == 2) {
-      body(0, T, F, T);
-      body(1, F, F, F);
-    } else {
-      body(0, T, F, F);
-    }
-  }
-  // inline-asm MFMAs are opaque to the compiler's hazard tracking: let the last results land before the
-  // epilogue reads the accumulation registers
-  if constexpr (NW == 4) asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  CS_TS(2);
-
-  // ---- epilogue.  acc[i][j][r] = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
-  //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
-  //      Every load the epilogue needs (row map, bias, residual / position rows) is issued up front, from
-  //      clamped addresses so that no branch guards a load: a load inside the store loop would make the
-  //      compiler wait for ALL outstanding memory operations (vmcnt counts stores too), i.e. for every
-  //      store issued so far and for the next tile's prefetch, once per row block.
-  {
-    const bf16_t* const pBias = (const bf16_t*)p.bias;
-    bf16_t* const pC = (bf16_t*)p.C;
-    const int n_lane = n0 + wn * WTN + kq * (4 * G);
-    int mrow[MT];
-    int crow[MT];  // 32-bit row numbers; the 64-bit address is formed at the store
-#pragma unroll
-    for (int i = 0; i < MT; ++i) {
-      mrow[i] = m0 + wm * WTM + i * 16 + fa;
-      const int mc = min(mrow[i], p.M - 1);
-      crow[i] = p.c_rows ? p.c_rows[mc] : mc;
-    }
-    bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
-#pragma unroll
-    for (int j = 0; j < NT; ++j) {
-      const int nc = min(n_lane + piece_col(j), p.N - 4);
-      bias_v[j] = bf16x4_t{0, 0, 0, 0};
-      if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + nc);
-    }
-    constexpr bool ADDEND = (EPI == CS_EPI_RESIDUAL) || (EPI == CS_EPI_BIAS_POS);
-    bf16x4_t addend[ADDEND ? MT : 1][ADDEND ? NT : 1];
-    auto load_addend = [&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
-      const int mc = min(mrow[i], p.M - 1);
-      const bf16_t* row = (EPI == CS_EPI_RESIDUAL)
-                              ? (const bf16_t*)p.residual + (int64_t)mc * p.ldr
-                              : (const bf16_t*)p.pos + (int64_t)(mc % p.pos_period) * p.ldpos;
-#pragma unroll
-      for (int j = 0; j < NT; ++j)
-        addend[ADDEND ? i : 0][ADDEND ? j : 0] = *(const bf16x4_t*)(row + min(n_lane + piece_col(j), p.N - 4));
+      wg_barrier();
+      if constexpr (SWITCH_BEFORE_B) switch_sources();
+      // second k-step; meanwhile the first fragments of K tile kt+1 and the second-half portion of loads,
+      // which goes to LDS space that the barrier has just freed
+      mfmas(ic<1>{}, std::false_type{}, [&](auto n) {
+        constexpr int N = decltype(n)::value;
+        if constexpr (TAIL != 1 && N < 2 * NFR && N % 2 == 0)
+          read_frag(a_base_of(1, ring), w_base_of(1, ring), 0, 0, ic<N / 2>{});
+        if constexpr (N < EB * PB && N % EB == EB - 1) {
+          auto ld = [&]() { direct_load(k_b, a_base_of(AHEAD_B, ring), w_base_of(AHEAD_B, ring), ic<PB_FIRST + N / EB>{}); };
+          if constexpr (CUR_B) ld();
+          else if (has_next) ld();
+        }
+      });
+      ring = slot_add(ring, RING5 ? 2 : 1);
     };
-    // The one-wave-per-SIMD form must stay inside the architectural registers (its accumulation registers
-    // are not the compiler's to use), so it fetches the addend rows in two batches.
-    constexpr int ADD_BATCH = (NW == 4) ? MT / 2 : MT;
-    if constexpr (ADDEND) static_for<ADD_BATCH>(load_addend);
-    static_for<MT>([&](auto i_c) {
-      constexpr int i = decltype(i_c)::value;
-      if constexpr (ADDEND && i == ADD_BATCH && ADD_BATCH < MT)
-        static_for<MT - ADD_BATCH>([&](auto k_c) { load_addend(ic<ADD_BATCH + decltype(k_c)::value>{}); });
-      const bool mok = mrow[i] < p.M;
-      f32x4_t racc[NT];
-      if constexpr (NW == 4) {
+    {
+      constexpr std::true_type T{};
+      constexpr std::false_type F{};
+      // the last AHEAD_B iterations are tails; everything before is steady state
+      if (nk == 3 && AHEAD_B == 3) {
+        iteration(0, T, ic<3>{});
+      } else {
+        iteration(0, T, ic<0>{});
+        for (int kt = 1; kt < nk - AHEAD_B; ++kt) iteration(kt, F, ic<0>{});
+        if constexpr (AHEAD_B == 3) iteration(nk - 3, F, ic<3>{});
+      }
+      iteration(nk - 2, F, ic<2>{});
+      iteration(nk - 1, F, ic<1>{});
+    }
+    // inline-asm MFMAs are opaque to the compiler's hazard tracking: let the last results land before the
+    // epilogue reads the accumulation registers
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    CS_TS(2);
+
+    // ---- epilogue.  Accumulator (i, j), element r = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
+    //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
+    //      The loads the epilogue needs (row map, bias, residual / position rows) are issued ahead of the
+    //      stores that follow them, from clamped addresses so that no branch guards a load: a load inside the
+    //      store loop would make the compiler wait for ALL outstanding memory operations (vmcnt counts stores
+    //      too), i.e. for every store issued so far and for the next tile's prefetch, once per row block.
+    {
+      const bf16_t* const pBias = (const bf16_t*)p.bias;
+      bf16_t* const pC = (bf16_t*)p.C;
+      const int n_lane = n0 + wn * WTN + kq * (4 * G);
+      int mrow[MT];
+      int crow[MT];  // 32-bit row numbers; the 64-bit address is formed at the store
+#pragma unroll
+      for (int i = 0; i < MT; ++i) {
+        mrow[i] = m0 + wm * WTM + i * 16 + fa;
+        const int mc = min(mrow[i], p.M - 1);
+        crow[i] = p.c_rows ? p.c_rows[mc] : mc;
+      }
+      bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const int nc = min(n_lane + piece_col(j), p.N - 4);
+        bias_v[j] = bf16x4_t{0, 0, 0, 0};
+        if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + nc);
+      }
+      constexpr bool ADDEND = (EPI == CS_EPI_RESIDUAL) || (EPI == CS_EPI_BIAS_POS);
+      bf16x4_t addend[ADDEND ? MT : 1][ADDEND ? NT : 1];
+      auto load_addend = [&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        const int mc = min(mrow[i], p.M - 1);
+        const bf16_t* row = (EPI == CS_EPI_RESIDUAL)
+                                ? (const bf16_t*)p.residual + (int64_t)mc * p.ldr
+                                : (const bf16_t*)p.pos + (int64_t)(mc % p.pos_period) * p.ldpos;
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          addend[ADDEND ? i : 0][ADDEND ? j : 0] = *(const bf16x4_t*)(row + min(n_lane + piece_col(j), p.N - 4));
+      };
+      // The kernel must stay inside the architectural registers (the accumulation registers are not the
+      // compiler's to use), so the addend rows are fetched in two batches.
+      constexpr int ADD_BATCH = MT / 2;
+      if constexpr (ADDEND) static_for<ADD_BATCH>(load_addend);
+      static_for<MT>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        if constexpr (ADDEND && i == ADD_BATCH)
+          static_for<MT - ADD_BATCH>([&](auto k_c) { load_addend(ic<ADD_BATCH + decltype(k_c)::value>{}); });
+        const bool mok = mrow[i] < p.M;
+        f32x4_t racc[NT];
         static_for<NT * 4>([&](auto e_c) {
           constexpr int E = decltype(e_c)::value;
           float t;
           asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(i * NT * 4 + E));
           racc[E / 4][E % 4] = t;
         });
-      } else {
+        bf16x4_t out[NT];
 #pragma unroll
-        for (int j = 0; j < NT; ++j) racc[j] = acc[i][j];
-      }
-      bf16x4_t out[NT];
+        for (int j = 0; j < NT; ++j) {
+          float v[4];
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        float v[4];
+          for (int r = 0; r < 4; ++r) v[r] = racc[j][r] + bf2f(bias_v[j][r]);
+          if (EPI == CS_EPI_SWIGLU) {
+            // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the
+            // product stay in fp32 until the single output rounding
+            const float g0 = silu(rbf(v[0])), u0 = rbf(v[1]);
+            const float g1 = silu(rbf(v[2])), u1 = rbf(v[3]);
+            out[j][0] = f2bf(g0 * u0);
+            out[j][1] = f2bf(g1 * u1);
+          } else {
+            if (EPI == CS_EPI_GELU_ERF) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = racc[j][r] + bf2f(bias_v[j][r]);
+              for (int r = 0; r < 4; ++r) v[r] = gelu_erf(rbf(v[r]));
+            } else if (EPI == CS_EPI_GELU_TANH) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(rbf(v[r]));
+            } else if (ADDEND) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) v[r] = rbf(v[r]) + bf2f(addend[ADDEND ? i : 0][ADDEND ? j : 0][r]);
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
+          }
+        }
+        // With G == 2 the pieces of fragments 2g and 2g+1 are adjacent: one 16-byte store per lane, and the
+        // four lanes of an output row write 64 consecutive bytes (32 with the halved SwiGLU output).
         if (EPI == CS_EPI_SWIGLU) {
-          // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the
-          // product stay in fp32 until the single output rounding
-          const float g0 = silu(rbf(v[0])), u0 = rbf(v[1]);
-          const float g1 = silu(rbf(v[2])), u1 = rbf(v[3]);
-          out[j][0] = f2bf(g0 * u0);
-          out[j][1] = f2bf(g1 * u1);
-        } else {
-          if (EPI == CS_EPI_GELU_ERF) {
+          bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + (n_lane >> 1);
+          if constexpr (G == 2) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] = gelu_erf(rbf(v[r]));
-          } else if (EPI == CS_EPI_GELU_TANH) {
+            for (int j = 0; j < NT; j += 2) {
+              if (mok && n_lane + piece_col(j) < p.N) {
+                bf16x4_t o = {out[j][0], out[j][1], out[j + 1][0], out[j + 1][1]};
+                *(bf16x4_t*)(dst + (piece_col(j) >> 1)) = o;
+              }
+            }
+          } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(rbf(v[r]));
-          } else if (ADDEND) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] = rbf(v[r]) + bf2f(addend[ADDEND ? i : 0][ADDEND ? j : 0][r]);
-          }
-#pragma unroll
-          for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
-        }
-      }
-      // With G == 2 the pieces of fragments 2g and 2g+1 are adjacent: one 16-byte store per lane, and the
-      // four lanes of an output row write 64 consecutive bytes (32 with the halved SwiGLU output).
-      if (EPI == CS_EPI_SWIGLU) {
-        bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + (n_lane >> 1);
-        if constexpr (G == 2) {
-#pragma unroll
-          for (int j = 0; j < NT; j += 2) {
-            if (mok && n_lane + piece_col(j) < p.N) {
-              bf16x4_t o = {out[j][0], out[j][1], out[j + 1][0], out[j + 1][1]};
-              *(bf16x4_t*)(dst + (piece_col(j) >> 1)) = o;
+            for (int j = 0; j < NT; ++j) {
+              if (mok && n_lane + piece_col(j) < p.N) {
+                bf16x2_t o;
+                o[0] = out[j][0];
+                o[1] = out[j][1];
+                *(bf16x2_t*)(dst + (piece_col(j) >> 1)) = o;
+              }
             }
           }
         } else {
+          bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + n_lane;
+          if constexpr (G == 2) {
 #pragma unroll
-          for (int j = 0; j < NT; ++j) {
-            if (mok && n_lane + piece_col(j) < p.N) {
-              bf16x2_t o;
-              o[0] = out[j][0];
-              o[1] = out[j][1];
-              *(bf16x2_t*)(dst + (piece_col(j) >> 1)) = o;
+            for (int j = 0; j < NT; j += 2) {
+              if (mok && n_lane + piece_col(j) < p.N) {
+                bf16x8_t o = {out[j][0], out[j][1], out[j][2], out[j][3], out[j + 1][0], out[j + 1][1], out[j + 1][2], out[j + 1][3]};
+                *(bf16x8_t*)(dst + piece_col(j)) = o;
+              }
             }
+          } else {
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+              if (mok && n_lane + piece_col(j) < p.N) *(bf16x4_t*)(dst + piece_col(j)) = out[j];
           }
         }
-      } else {
-        bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + n_lane;
-        if constexpr (G == 2) {
-#pragma unroll
-          for (int j = 0; j < NT; j += 2) {
-            if (mok && n_lane + piece_col(j) < p.N) {
-              bf16x8_t o = {out[j][0], out[j][1], out[j][2], out[j][3], out[j + 1][0], out[j + 1][1], out[j + 1][2], out[j + 1][3]};
-              *(bf16x8_t*)(dst + piece_col(j)) = o;
-            }
-          }
-        } else {
-#pragma unroll
-          for (int j = 0; j < NT; ++j)
-            if (mok && n_lane + piece_col(j) < p.N) *(bf16x4_t*)(dst + piece_col(j)) = out[j];
-        }
-      }
-    });
+      });
+    }
+    CS_TS(3);
+    if (!has_next) break;
+    vb = vb_next;
+    m0 = m0_next;
+    n0 = n0_next;
   }
-  CS_TS(3);
-  if (!has_next) break;
-  vb = vb_next;
-  m0 = m0_next;
-  n0 = n0_next;
-  }  // persistent tile loop
 }
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
@@ -686,10 +515,7 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   CsGemmArgs p = a;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  constexpr int stage_bytes = (BM + BN) * BK * 2;
-  constexpr bool ring3 = WAVES_M * WAVES_N == 4 && 3 * stage_bytes <= 160 * 1024;
-  constexpr bool ring5 = WAVES_M * WAVES_N == 4 && !ring3 && BM == BN && 5 * BM * BK * 2 <= 160 * 1024;
-  constexpr int lds = ring5 ? 5 * BM * BK * 2 : (ring3 ? 3 : 2) * stage_bytes;
+  constexpr int lds = RingShape<BM, BN>::BYTES;
   static bool attr_set = false;
   auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
   if (!attr_set) {
@@ -700,9 +526,7 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   const int tiles = p.tiles_m * p.tiles_n;
   // One resident workgroup per CU (LDS-bound); with more tiles than CUs the kernel is persistent.
   const int grid = tiles <= 256 ? tiles : 256;
-  static const char* st_env = getenv("CS_GEMM_STAGGER");  // experiment knob: ticks of 10 ns per slot
-  const int stagger = tiles > 256 ? (st_env ? atoi(st_env) : 0) : 0;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES_M * WAVES_N), lds, stream, p, stagger);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, p);
   return cs_launch_status();
 }
 
@@ -732,20 +556,19 @@ double rounds_cost(int M, int N, int bm, int bn) {
 // Called by cs_gemm after argument validation.  Sets *handled when this path took the problem.
 int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   *handled = false;
-  if (a.w_fp8 || a.K % BK || a.K < 3 * BK || a.M < 1 || a.w_scale || a.N < 8) return CS_OK;
-  // 16-byte output stores
-  if (a.N % 8 || a.ldc % 8 || ((uintptr_t)a.C & 15)) return CS_OK;
-  if (a.pos && a.epilogue != CS_EPI_BIAS) return CS_OK;
-  // per-lane source offsets are 32-bit byte offsets from the matrix bases
+  if (a.w_fp8 || a.w_scale || a.M < 1 || a.N < 8) return CS_OK;
+  if (a.K % BK || a.K < 3 * BK) return CS_OK;  // the ring pipeline is written for at least three K tiles
+  if (a.N % 8 || a.ldc % 8 || ((uintptr_t)a.C & 15)) return CS_OK;  // 16-byte output stores
+  if (a.pos && a.epilogue != CS_EPI_BIAS) return CS_OK;  // the position addend only pairs with the plain epilogue here
   if (a.a_rows) return CS_OK;  // gathered A rows can lie anywhere: the general kernel keeps 64-bit pointers
-  if ((int64_t)a.M * a.lda * 2 >= (int64_t)UINT32_MAX || (int64_t)a.N * a.ldw * 2 >= (int64_t)UINT32_MAX) return CS_OK;  // position addend only pairs with the plain epilogue here
+  // per-lane source offsets are 32-bit byte offsets from the matrix bases
+  if ((int64_t)a.M * a.lda * 2 >= (int64_t)UINT32_MAX || (int64_t)a.N * a.ldw * 2 >= (int64_t)UINT32_MAX) return CS_OK;
   *handled = true;
   // Tile shape: the one that needs the least chip time (tile quantisation over the 256 CUs).  The narrow
   // 256x160 tile exists for N = 1280 (8 column tiles: 8192 rows give exactly 256 workgroups).
   const double c256 = rounds_cost(a.M, a.N, 256, 256);
   const double c160 = rounds_cost(a.M, a.N, 256, 160) * 1.15;  // narrower tiles: more LDS and L2 traffic per FLOP
-  static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160", "256" or "8" (8-wave 256x256)
-  if (force && force[0] == '8') return dispatch_epi<256, 256, 2, 4>(a, stream);
+  static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160" or "256"
   if (force ? force[0] == '1' : c160 < c256) return dispatch_epi<256, 160, 4, 1>(a, stream);
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller
