@@ -99,8 +99,9 @@ int cs_layernorm(const void* x, int64_t ldx, const void* w, const void* b, void*
  * computation (:445-448):
  *   cu_window_host  int32, n_cu_window entries written (capacity cap_window)
  *   cu_full_host    int32, n_cu_full entries written   (capacity cap_full)
- *   item_meta_host  int32 [n_items][8]: t, h/merge, w/merge, first merged unit, first window-order
- *                   unit (== first merged unit), windows per row, windows per column, reserved
+ *   item_meta_host  int32 [n_items][8]: t, gh = h/merge, gw = w/merge, first merged unit of the item,
+ *                   ceil(gh/win), ceil(gw/win) (non-empty windows along h and w), first patch row of the
+ *                   item, reserved (0)
  * merge = spatial merge size (2), win = window side in merged units (window_size/merge/patch = 4).
  * Returns CS_ERR_TOO_LARGE if a capacity is too small.                                            */
 int cs_vit_seqlens_host(const int64_t* grid_thw_host, int32_t n_items, int32_t merge, int32_t win,
