@@ -226,6 +226,17 @@ class Qwen2_5_VisionTransformer(EricModel):
         ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, self.spatial_merge_size, win, pk["inv_freq"])
         return ix.window_index, sl.cu_window.tolist()
 
+    def _index(self, grid_thw: np.ndarray):
+        """Everything that depends on the grids only: window permutation, rotary table, attention work lists
+        (reference: rot_pos_emb :325-355, get_window_index :357-386, cu_seqlens :445-448)."""
+        merge = self.spatial_merge_size
+        win = self.window_size // merge // self.patch_size
+        dev = self.device
+        sl = ops.vit_seqlens_host(grid_thw, merge, win)
+        meta = torch.from_numpy(sl.item_meta).to(dev, non_blocking=True)
+        ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, merge, win, self._ensure_packed()["inv_freq"])
+        return ix, ops.attn_plan(sl.cu_window, dev), ops.attn_plan(sl.cu_full, dev), sl.total_patches
+
     def forward_device(self, pixel_values: torch.Tensor, grid_thw: np.ndarray, mark=None) -> list[torch.Tensor]:
         """pixel_values: bf16 [L, C*T*P*P] already on the device; grid_thw: host int64 [n,3].
 
@@ -241,14 +252,9 @@ class Qwen2_5_VisionTransformer(EricModel):
         dev = self.device
 
         mark("index")
-        sl = ops.vit_seqlens_host(grid_thw, merge, win)
-        L = sl.total_patches
+        ix, plan_win, plan_full, L = self._index(grid_thw)
         if pixel_values.shape[0] != L:
             raise ValueError(f"pixel_values has {pixel_values.shape[0]} rows but grid_thw describes {L} patches")
-        meta = torch.from_numpy(sl.item_meta).to(dev, non_blocking=True)
-        ix = ops.vit_index(meta, L, sl.max_units_per_item, merge, win, pk["inv_freq"])
-        plan_win = ops.attn_plan(sl.cu_window, dev)
-        plan_full = ops.attn_plan(sl.cu_full, dev)
 
         # patch embed; rows come out already in window order
         mark("patch_embed")
