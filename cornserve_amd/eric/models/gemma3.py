@@ -179,6 +179,22 @@ class Gemma3VisionEncoder(EricModel):
         kp = _round_up(kraw, 16)
         pe_w = torch.zeros((H, kp), dtype=self.dtype, device=self.device)
         pe_w[:, :kraw] = vm.embeddings.patch_embedding.weight.reshape(H, kraw)
+        # The MLP intermediate size (4304 for SigLIP-so400m) is padded to a multiple of 64 so that fc2's K loop is
+        # tail-free: the pad rows of fc1 (and their bias) are zero, GELU(0) = 0, and fc2's pad columns are zero,
+        # so the padded activations are exactly zero and the result is unchanged.
+        inter = vc.intermediate_size
+        ip = _round_up(inter, 64)
+
+        def pad_rows(w: torch.Tensor) -> torch.Tensor:
+            out = torch.zeros((ip, *w.shape[1:]), dtype=w.dtype, device=w.device)
+            out[:inter] = w
+            return out
+
+        def pad_cols(w: torch.Tensor) -> torch.Tensor:
+            out = torch.zeros((w.shape[0], ip), dtype=w.dtype, device=w.device)
+            out[:, :inter] = w
+            return out
+
         layers = []
         for lyr in vm.encoder.layers:
             a = lyr.self_attn
@@ -189,11 +205,11 @@ class Gemma3VisionEncoder(EricModel):
                     "qkv_w": torch.cat([a.q_proj.weight, a.k_proj.weight, a.v_proj.weight], dim=0).contiguous(),
                     "qkv_b": torch.cat([a.q_proj.bias, a.k_proj.bias, a.v_proj.bias], dim=0).contiguous(),
                     "out": (a.out_proj.weight, a.out_proj.bias),
-                    "fc1": (lyr.mlp.fc1.weight, lyr.mlp.fc1.bias),
-                    "fc2": (lyr.mlp.fc2.weight, lyr.mlp.fc2.bias),
+                    "fc1": (pad_rows(lyr.mlp.fc1.weight), pad_rows(lyr.mlp.fc1.bias)),
+                    "fc2": (pad_cols(lyr.mlp.fc2.weight), lyr.mlp.fc2.bias),
                 }
             )
-        return {"pe_w": pe_w, "pe_b": vm.embeddings.patch_embedding.bias, "kp": kp,
+        return {"pe_w": pe_w, "pe_b": vm.embeddings.patch_embedding.bias, "kp": kp, "ip": ip,
                 "pos": vm.embeddings.position_embedding.weight, "layers": layers,
                 "post": (vm.post_layernorm.weight, vm.post_layernorm.bias)}
 
@@ -222,7 +238,7 @@ class Gemma3VisionEncoder(EricModel):
         n = torch.empty_like(x)
         qkv = torch.empty((M, 3 * H), dtype=torch.bfloat16, device=x.device)
         att = torch.empty((M, H), dtype=torch.bfloat16, device=x.device)
-        hmid = torch.empty((M, vc.intermediate_size), dtype=torch.bfloat16, device=x.device)
+        hmid = torch.empty((M, pk["ip"]), dtype=torch.bfloat16, device=x.device)
         eps = vc.layer_norm_eps
         act = getattr(vc, "hidden_act", "gelu_pytorch_tanh")
         if act == "gelu_pytorch_tanh":
