@@ -172,6 +172,51 @@ def test_gemm_epilogues(ops, dev):
     close(ops.gemm(a, w, b, pos=pos), base + pos.float().cpu()[idx], 2**-7, "pos")
 
 
+def _epilogue_ref(ops, epi, base, res):
+    """fp32 reference of one fused epilogue on `base` = bf16-rounded A.W^T + bias."""
+    if epi == ops.EPI_BIAS:
+        return base
+    if epi == ops.EPI_RESIDUAL:
+        return base + res.float().cpu()
+    if epi == ops.EPI_GELU_ERF:
+        return F.gelu(base)
+    if epi == ops.EPI_GELU_TANH:
+        return F.gelu(base, approximate="tanh")
+    gate, up = base[:, 0::2], base[:, 1::2]
+    return F.silu(gate).bfloat16().float() * up
+
+
+# Shapes that reach every tile form and every schedule of the fast kernel: the 256x256 five-unit ring, the
+# 256x160 / 256x128 / 128x192 three-stage rings (N = 1280; remainders of a column split), the shortest K the
+# fast path takes (3 K tiles: the ring's tail iterations only) and 4, 5, 7 K tiles, row and column tails.
+@pytest.mark.parametrize("M,N,K", [
+    (8192, 3072, 192),    # 8 columns of 256x256 + 1024 columns of 256x128, 3 K tiles
+    (8192, 2304, 256),    # 8 columns of 256x256 + 256 columns of 128x192, 4 K tiles
+    (1000, 1280, 320),    # 256x160, row tail, 5 K tiles
+    (300, 520, 448),      # 256x256 with row and column tails, 7 K tiles
+    (8192, 1280, 192),    # 256x160, one tile per CU, 3 K tiles
+])
+def test_gemm_fast_path_forms(ops, dev, M, N, K):
+    a, w, b = rnd((M, K), 1.0, 11, dev), rnd((N, K), 0.05, 12, dev), rnd((N,), 0.02, 13, dev)
+    res = rnd((M, N), 1.0, 14, dev)
+    rows = torch.arange(0, M, max(1, M // 257))  # a sample of rows: the fp32 reference runs on the host
+    rows = torch.cat([rows, torch.tensor([M - 1])])
+    base = lin_ref(a[rows], w, b).bfloat16().float()
+    for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_SWIGLU):
+        got = ops.gemm(a, w, b, epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
+        close(got[rows], _epilogue_ref(ops, epi, base, res[rows]), 2**-7, f"{M}x{N}x{K} epilogue {epi}")
+    # repeated launches give identical bits (fixed accumulation order, no races between the two launches of
+    # a column split or between consecutive tiles of a persistent workgroup)
+    first = ops.gemm(a, w, b)
+    for _ in range(3):
+        assert torch.equal(ops.gemm(a, w, b), first)
+    perm = torch.randperm(M, generator=torch.Generator().manual_seed(2)).int().to(dev)
+    scat = ops.gemm(a, w, b, c_rows=perm)
+    ref = torch.empty_like(first)
+    ref[perm.long()] = first
+    assert torch.equal(scat, ref)
+
+
 def test_gemm_row_maps(ops, dev):
     M, N, K = 400, 512, 256
     a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
