@@ -17,7 +17,9 @@
 // product without touching LDS: accumulator rows 8kk..8kk+7 of a lane are keys
 // {16kk+4h+0..3, 16kk+8+4h+0..3} (h = lane/32); the V^T fragment is read from LDS with the same key
 // order, which is legal because a dot product does not care about the order of its terms.
-// V is transposed once per tile on its way into LDS (pairs of keys packed into 32-bit writes).
+// V goes to LDS row-major like K; the transposition happens in the LDS read: ds_read_b64_tr_b16 hands each
+// lane of a 16-lane group four 16-bit values gathered from four other lanes' addresses, which turns a
+// [4 keys x 16 dims] block into "lane l holds 4 consecutive keys of dim l".
 // Head dims that are not multiples of 16 (SigLIP's 72) are zero-padded in LDS only.
 #include <type_traits>
 
@@ -26,7 +28,27 @@
 namespace {
 
 constexpr int BKV = 64;        // keys per LDS tile
-constexpr int VT_STRIDE = 68;  // bf16 elements per V^T row (64 keys + 4 pad: conflict-free 8-byte reads)
+constexpr int V_RS = 192;      // bytes per key row of a V tile in LDS (96 head-dim slots).  192 = 64 mod 256: the four
+                               // key rows x 64 bytes that 32 lanes of a transposing read touch fall into distinct banks.
+
+typedef short s16x4_t __attribute__((ext_vector_type(4)));
+typedef short s16x8_t __attribute__((ext_vector_type(8)));
+typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;
+
+// A-operand fragment of V^T for the 32x32x16 MFMA: lane (fr = lane%32, hf = lane/32) gets dim 32t + fr and the
+// keys {16g + 4hf + 0..3, 16g + 8 + 4hf + 0..3} of key group g -- the key order in which the S^T accumulators
+// hold P.  ds_read_b64_tr_b16 works on groups of 16 lanes: destination lane l receives element l%4 of the
+// 8 bytes addressed by source lanes l/4 + 4e, e = 0..3.  So source lane s = 4e + j of a group addresses key
+// k0 + e, dims d0 + 4j .. 4j+3, and destination lane l ends up with dim d0 + l, keys k0 .. k0+3.
+CS_DEVICE bf16x8_t read_vt_frag(const char* v_tile, int t, int g, int lane) {
+  const int hf = lane >> 5, s = lane & 15;
+  const int key = 16 * g + 4 * hf + (s >> 2);
+  const int dim = 32 * t + 16 * ((lane >> 4) & 1) + 4 * (s & 3);
+  const char* p = v_tile + key * V_RS + dim * 2;
+  const s16x4_t lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)p);
+  const s16x4_t hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t*)(p + 8 * V_RS));
+  return __builtin_bit_cast(bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
 
 struct AttnArgs {
   const bf16_t* q;
@@ -54,7 +76,7 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
 
   __shared__ __attribute__((aligned(16))) char q_lds[BQ * RS];
   __shared__ __attribute__((aligned(16))) char k_lds[BKV * RS];
-  __shared__ __attribute__((aligned(16))) bf16_t vt_lds[DT * 32 * VT_STRIDE];
+  __shared__ __attribute__((aligned(16))) char v_lds[BKV * V_RS];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 31, hf = lane >> 5;
@@ -110,22 +132,14 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
     }
   };
 
-  // V tile -> V^T in LDS: thread takes a pair of keys and one 8-wide chunk of the head dim.
+  // V tile -> LDS, row-major; rows past the segment end are zero (they meet P = 0, which must not be 0 * NaN).
   auto stage_v = [&](int g0, int nvalid) {
     const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    for (int i = tid; i < (BKV / 2) * DC; i += NT) {
-      const int kp = i % (BKV / 2), c = i / (BKV / 2);
-      const int r0 = 2 * kp;
-      bf16x8_t x0 = zero, x1 = zero;
-      if (r0 < nvalid) x0 = *(const bf16x8_t*)(a.v + (int64_t)(g0 + r0) * a.ld + hoff + c * 8);
-      if (r0 + 1 < nvalid) x1 = *(const bf16x8_t*)(a.v + (int64_t)(g0 + r0 + 1) * a.ld + hoff + c * 8);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        bf16x2_t pr;
-        pr[0] = x0[e];
-        pr[1] = x1[e];
-        *(bf16x2_t*)(vt_lds + (c * 8 + e) * VT_STRIDE + r0) = pr;
-      }
+    for (int i = tid; i < BKV * DC; i += NT) {
+      const int r = i / DC, c = i - r * DC;
+      bf16x8_t x = zero;
+      if (r < nvalid) x = *(const bf16x8_t*)(a.v + (int64_t)(g0 + r) * a.ld + hoff + c * 8);
+      *(bf16x8_t*)(v_lds + r * V_RS + c * 16) = x;
     }
   };
 
@@ -222,15 +236,7 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-          const bf16_t* vp = vt_lds + (t * 32 + fr) * VT_STRIDE + kt * 32 + 16 * kk + 4 * hf;
-          const bf16x4_t v0 = *(const bf16x4_t*)vp;
-          const bf16x4_t v1 = *(const bf16x4_t*)(vp + 8);
-          bf16x8_t vf;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            vf[e] = v0[e];
-            vf[4 + e] = v1[e];
-          }
+          const bf16x8_t vf = read_vt_frag(v_lds, t, kt * 2 + kk, lane);
           oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][kk], oacc[t], 0, 0, 0);
         }
     }
@@ -243,9 +249,9 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
     // for all HPW heads, and the batch of head h+1 is requested before the matrix-core work on head h,
     // so after the first head the memory latency hides behind compute.
     constexpr int HC = DC / 2;
-    constexpr int NI = (BKV * HC + NT - 1) / NT, NV = ((BKV / 2) * DC + NT - 1) / NT;
+    constexpr int NI = (BKV * HC + NT - 1) / NT, NV = (BKV * DC + NT - 1) / NT;
     const bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8_t q1[NI], q2[NI], k1[NI], k2[NI], v0[NV], v1[NV];
+    bf16x8_t q1[NI], q2[NI], k1[NI], k2[NI], vx[NV];
     f32x4_t c0[NI], c1[NI], s0[NI], s1[NI];
     // Unconditional loads from clamped rows (no branch between them, so they are all in flight together).
     // Rows past the segment end therefore hold copies of the last row: as keys they are masked (P = 0, and
@@ -271,9 +277,8 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
       }
 #pragma unroll
       for (int it = 0; it < NV; ++it) {
-        const int i = min(tid + it * NT, (BKV / 2) * DC - 1), kp = i % (BKV / 2), c = i / (BKV / 2), r0 = 2 * kp;
-        v0[it] = *(const bf16x8_t*)(a.v + (int64_t)(seg_start + min(r0, seg_len - 1)) * a.ld + ho + c * 8);
-        v1[it] = *(const bf16x8_t*)(a.v + (int64_t)(seg_start + min(r0 + 1, seg_len - 1)) * a.ld + ho + c * 8);
+        const int i = min(tid + it * NT, BKV * DC - 1), r = i / DC, c = i - r * DC;
+        vx[it] = *(const bf16x8_t*)(a.v + (int64_t)(seg_start + min(r, seg_len - 1)) * a.ld + ho + c * 8);
       }
     };
     issue_qkv(hoff);
@@ -311,16 +316,8 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
       }
 #pragma unroll
       for (int it = 0; it < NV; ++it) {
-        const int i = tid + it * NT, kp = i % (BKV / 2), c = i / (BKV / 2), r0 = 2 * kp;
-        if (i < (BKV / 2) * DC) {
-#pragma unroll
-          for (int e = 0; e < 8; ++e) {
-            bf16x2_t pr;
-            pr[0] = v0[it][e];
-            pr[1] = v1[it][e];
-            *(bf16x2_t*)(vt_lds + (c * 8 + e) * VT_STRIDE + r0) = pr;
-          }
-        }
+        const int i = tid + it * NT, r = i / DC, c = i - r * DC;
+        if (i < BKV * DC) *(bf16x8_t*)(v_lds + r * V_RS + c * 16) = vx[it];
       }
       __syncthreads();
       if (hh + 1 < HPW) issue_qkv(hoff + D);  // the staging registers are free again
@@ -368,11 +365,11 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
   constexpr int HC = DC / 2;
   static_assert(D % 8 == 0 && D <= 96, "head dim");
   static_assert(!ROPE || D % 16 == 0, "rotary needs an even number of chunks per half");
-  constexpr int K_BYTES = BKV * RS, V_BYTES = DT * 32 * VT_STRIDE * 2, Q_BYTES = BQ * RS;
+  constexpr int K_BYTES = BKV * RS, V_BYTES = BKV * V_RS, Q_BYTES = BQ * RS;
   constexpr int REGION_B = (K_BYTES + V_BYTES) > Q_BYTES ? (K_BYTES + V_BYTES) : Q_BYTES;
   __shared__ __attribute__((aligned(16))) char lds[K_BYTES + V_BYTES + REGION_B];
   auto k_buf = [&](int b) -> char* { return lds + b * (K_BYTES + V_BYTES); };
-  auto v_buf = [&](int b) -> bf16_t* { return (bf16_t*)(lds + b * (K_BYTES + V_BYTES) + K_BYTES); };
+  auto v_buf = [&](int b) -> char* { return lds + b * (K_BYTES + V_BYTES) + K_BYTES; };
   char* const q_lds = lds + K_BYTES + V_BYTES;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -390,45 +387,43 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
   // ---- register staging of one K/V tile
   constexpr int K_ITEMS = ROPE ? BKV * HC : BKV * DC;
   constexpr int K_PER = (K_ITEMS + NT - 1) / NT;
-  constexpr int V_ITEMS = (BKV / 2) * DC;
+  constexpr int V_ITEMS = BKV * DC;
   constexpr int V_PER = (V_ITEMS + NT - 1) / NT;
   bf16x8_t kx1[K_PER], kx2[ROPE ? K_PER : 1];
   f32x4_t kc0[ROPE ? K_PER : 1], kc1[ROPE ? K_PER : 1], ks0[ROPE ? K_PER : 1], ks1[ROPE ? K_PER : 1];
-  bf16x8_t vx0[V_PER], vx1[V_PER];
+  bf16x8_t vx[V_PER];
 
+  // Unconditional loads from clamped rows and items (no branch between them, so they are all in flight
+  // together).  Rows past the segment end then hold copies of the last valid row: as keys they are masked
+  // (P = 0, and 0 times a finite V row is 0).
   auto gload_tile = [&](int kv0, int nvalid) {
 #pragma unroll
     for (int u = 0; u < K_PER; ++u) {
-      const int i = tid + u * NT;
+      const int i = min(tid + u * NT, K_ITEMS - 1);
       constexpr int PER_ROW = ROPE ? HC : DC;
       const int r = i / PER_ROW, jc = i - r * PER_ROW;
-      const bool ok = i < K_ITEMS && r < nvalid;
-      const int64_t g = seg_start + kv0 + (ok ? r : 0);
+      const int64_t g = seg_start + kv0 + min(r, nvalid - 1);
       const bf16_t* p = a.k + g * a.ld + hoff + jc * 8;
-      kx1[u] = ok ? *(const bf16x8_t*)p : zero8;
+      kx1[u] = *(const bf16x8_t*)p;
       if (ROPE) {
-        kx2[u] = ok ? *(const bf16x8_t*)(p + D / 2) : zero8;
+        kx2[u] = *(const bf16x8_t*)(p + D / 2);
         const float* cs = a.cos_sin + g * D + jc * 8;
-        kc0[u] = ok ? *(const f32x4_t*)cs : zero4;
-        kc1[u] = ok ? *(const f32x4_t*)(cs + 4) : zero4;
-        ks0[u] = ok ? *(const f32x4_t*)(cs + D / 2) : zero4;
-        ks1[u] = ok ? *(const f32x4_t*)(cs + D / 2 + 4) : zero4;
+        kc0[u] = *(const f32x4_t*)cs;
+        kc1[u] = *(const f32x4_t*)(cs + 4);
+        ks0[u] = *(const f32x4_t*)(cs + D / 2);
+        ks1[u] = *(const f32x4_t*)(cs + D / 2 + 4);
       }
     }
 #pragma unroll
     for (int u = 0; u < V_PER; ++u) {
-      const int i = tid + u * NT;
-      const int kp = i / DC, c = i - kp * DC;   // consecutive lanes: consecutive chunks of one key pair
-      const int r0 = 2 * kp;
-      const bool ok0 = i < V_ITEMS && r0 < nvalid, ok1 = i < V_ITEMS && r0 + 1 < nvalid;
-      const bf16_t* p = a.v + (int64_t)(seg_start + kv0 + (ok0 ? r0 : 0)) * a.ld + hoff + c * 8;
-      vx0[u] = ok0 ? *(const bf16x8_t*)p : zero8;
-      vx1[u] = ok1 ? *(const bf16x8_t*)(p + a.ld) : zero8;
+      const int i = min(tid + u * NT, V_ITEMS - 1);
+      const int r = i / DC, c = i - r * DC;   // consecutive lanes: consecutive chunks of one key row
+      vx[u] = *(const bf16x8_t*)(a.v + (int64_t)(seg_start + kv0 + min(r, nvalid - 1)) * a.ld + hoff + c * 8);
     }
   };
   auto lstore_tile = [&](int b) {
     char* kd = k_buf(b);
-    bf16_t* vd = v_buf(b);
+    char* vd = v_buf(b);
 #pragma unroll
     for (int u = 0; u < K_PER; ++u) {
       const int i = tid + u * NT;
@@ -462,14 +457,8 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
     for (int u = 0; u < V_PER; ++u) {
       const int i = tid + u * NT;
       if (i < V_ITEMS) {
-        const int kp = i / DC, c = i - kp * DC;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          bf16x2_t pr;
-          pr[0] = vx0[u][e];
-          pr[1] = vx1[u][e];
-          *(bf16x2_t*)(vd + (c * 8 + e) * VT_STRIDE + 2 * kp) = pr;
-        }
+        const int r = i / DC, c = i - r * DC;
+        *(bf16x8_t*)(vd + r * V_RS + c * 16) = vx[u];
       }
     }
   };
@@ -533,7 +522,7 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
     if (more) gload_tile(kv0 + BKV, min(BKV, seg_len - kv0 - BKV));
     if (wave_active) {
       const char* kd = k_buf(buf);
-      const bf16_t* vd = v_buf(buf);
+      const char* vd = v_buf(buf);
       f32x16_t sacc[2];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
@@ -588,15 +577,7 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int kk = 0; kk < 2; ++kk) {
-            const bf16_t* vp = vd + (t * 32 + fr) * VT_STRIDE + kt * 32 + 16 * kk + 4 * hf;
-            const bf16x4_t v0 = *(const bf16x4_t*)vp;
-            const bf16x4_t v1 = *(const bf16x4_t*)(vp + 8);
-            bf16x8_t vf;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              vf[e] = v0[e];
-              vf[4 + e] = v1[e];
-            }
+            const bf16x8_t vf = read_vt_frag(vd, t, kt * 2 + kk, lane);
             oacc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf, pf[kt][kk], oacc[t], 0, 0, 0);
           }
       }
