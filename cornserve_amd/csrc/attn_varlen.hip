@@ -60,6 +60,8 @@ struct AttnArgs {
   const int32_t* work;
   const float* cos_sin;
   float scale_log2e;
+  // full-attention kernel only: 1-D launch, see its workgroup mapping
+  int n_work, heads, chunk, n_chunks_x;
 };
 
 template <int D, int NWAVES, bool ROPE, int HPW>
@@ -374,11 +376,19 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int fr = lane & 31, hf = lane >> 5;
-  const int head = blockIdx.y;
-  const int seg_start = a.work[blockIdx.x * 4 + 0];
-  const int seg_end = a.work[blockIdx.x * 4 + 1];
-  const int q0 = a.work[blockIdx.x * 4 + 2];
-  const int nq = a.work[blockIdx.x * 4 + 3];
+  // Workgroup mapping.  Workgroup i runs on XCD i % 8, each with its own L2.  Query blocks of one segment
+  // and head read the same K/V, so they should meet in one L2: the (work item, head) space is cut into
+  // chunks of `chunk` consecutive work items of one head (a segment's query blocks are consecutive work
+  // items), chunk c goes to XCD c % 8, and an XCD walks its chunks in order.
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;
+  const int cid = (j / a.chunk) * 8 + xcd;           // chunk id in [0, n_chunks_x * heads)
+  const int item = (cid % a.n_chunks_x) * a.chunk + j % a.chunk;
+  const int head = cid / a.n_chunks_x;
+  if (item >= a.n_work || head >= a.heads) return;   // padding of the last chunks (uniform per workgroup)
+  const int seg_start = a.work[item * 4 + 0];
+  const int seg_end = a.work[item * 4 + 1];
+  const int q0 = a.work[item * 4 + 2];
+  const int nq = a.work[item * 4 + 3];
   const int64_t hoff = (int64_t)head * D;
   const int seg_len = seg_end - seg_start;
   const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -606,8 +616,14 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
 }
 
 template <int D>
-int launch_attn(const AttnArgs& a, int n_work, int heads, int block_q, bool rope, hipStream_t stream) {
+int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, bool rope, hipStream_t stream) {
   const dim3 grid(n_work, heads);
+  a.n_work = n_work;
+  a.heads = heads;
+  a.chunk = min(32, max(1, (max_seqlen + 127) / 128));  // query blocks of the longest segment
+  a.n_chunks_x = (n_work + a.chunk - 1) / a.chunk;
+  const int n_chunks = a.n_chunks_x * heads;
+  const dim3 grid_full(((n_chunks + 7) / 8) * 8 * a.chunk);
   if (block_q == 64) {
     if (rope) {
       // two heads per workgroup when that still leaves several workgroups per CU
@@ -623,10 +639,10 @@ int launch_attn(const AttnArgs& a, int n_work, int heads, int block_q, bool rope
     }
   } else {
     if (rope) {
-      if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_full_kernel<D, true>), grid, dim3(256), 0, stream, a);
+      if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_full_kernel<D, true>), grid_full, dim3(256), 0, stream, a);
       else return CS_ERR_UNSUPPORTED;
     } else {
-      hipLaunchKernelGGL((attn_full_kernel<D, false>), grid, dim3(256), 0, stream, a);
+      hipLaunchKernelGGL((attn_full_kernel<D, false>), grid_full, dim3(256), 0, stream, a);
     }
   }
   return cs_launch_status();
@@ -682,10 +698,10 @@ extern "C" int cs_attn_varlen(const void* q, const void* k, const void* v, int64
   const int bq = cs_attn_block_q(max_seqlen);
   const bool rope = cos_sin != nullptr;
   switch (head_dim) {
-    case 64: return launch_attn<64>(a, n_work, heads, bq, rope, stream);
-    case 72: return launch_attn<72>(a, n_work, heads, bq, rope, stream);
-    case 80: return launch_attn<80>(a, n_work, heads, bq, rope, stream);
-    case 96: return launch_attn<96>(a, n_work, heads, bq, rope, stream);
+    case 64: return launch_attn<64>(a, n_work, heads, bq, max_seqlen, rope, stream);
+    case 72: return launch_attn<72>(a, n_work, heads, bq, max_seqlen, rope, stream);
+    case 80: return launch_attn<80>(a, n_work, heads, bq, max_seqlen, rope, stream);
+    case 96: return launch_attn<96>(a, n_work, heads, bq, max_seqlen, rope, stream);
     default: return CS_ERR_UNSUPPORTED;
   }
 }
