@@ -109,19 +109,22 @@ CS_DEVICE void static_for(F&& f) {
 }
 
 // LDS organisation of a tile shape (shared by the kernel and its launcher).
-template <int BM, int BN>
+template <int BM, int BN, bool W_FP8>
 struct RingShape {
-  static constexpr int A_BYTES = BM * BK * 2, W_BYTES = BN * BK * 2;
+  static constexpr int A_BYTES = BM * BK * 2, W_BYTES = BN * BK * (W_FP8 ? 1 : 2);
   static constexpr bool FIVE_UNITS = A_BYTES == W_BYTES && 5 * A_BYTES <= LDS_BYTES && 3 * (A_BYTES + W_BYTES) > LDS_BYTES;
   static constexpr int BYTES = FIVE_UNITS ? 5 * A_BYTES : 3 * (A_BYTES + W_BYTES);
   static_assert(BYTES <= LDS_BYTES, "tile does not fit a ring");
 };
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+// W_FP8: the weights are e4m3 bytes with a per-output-channel fp32 scale.  W tiles travel and sit in LDS as bytes
+// (half the traffic); a fragment is converted to bf16 in registers right before its MFMAs (exact: every e4m3
+// value is a bf16 value) and the scale is applied to the fp32 accumulators in the epilogue.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8>
 __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   static_assert(WAVES_M * WAVES_N == NW, "four waves, one per SIMD");
-  using Ring = RingShape<BM, BN>;
+  using Ring = RingShape<BM, BN, W_FP8>;
   constexpr int A_BYTES = Ring::A_BYTES, W_BYTES = Ring::W_BYTES;
   constexpr bool RING5 = Ring::FIVE_UNITS;
   // Byte offsets of operand tile slots.  Three-stage ring: slot s holds A at s*STAGE and W behind it.
@@ -136,9 +139,15 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   // one output row own 16G consecutive columns.
   constexpr int G = (NT % 2 == 0) ? 2 : NT;
   auto piece_col = [](int j) { return (j / G) * 16 * G + (j % G) * 4; };  // first column of fragment j's piece
-  constexpr int A_BLK = BM / 8, W_BLK = BN / 8;  // 8-row blocks = direct loads per operand tile
-  static_assert(A_BLK % NW == 0 && W_BLK % NW == 0, "every wave issues the same number of direct loads");
-  constexpr int A_LD = A_BLK / NW, W_LD = W_BLK / NW;  // per wave
+  constexpr int W_ROW = W_FP8 ? BK : BK * 2;     // bytes per W tile row
+  constexpr int W_ROWS_LD = 1024 / W_ROW;         // W rows per direct load (one load moves 64 x 16 bytes)
+  static_assert(BN % W_ROWS_LD == 0, "tile shape");
+  constexpr int A_BLK = BM / 8, W_BLK = BN / W_ROWS_LD;  // row blocks = direct loads per operand tile
+  static_assert(A_BLK % NW == 0, "every wave issues the same number of direct loads");
+  // When W_BLK is not a multiple of the wave count, the waves that have no block left repeat the last one
+  // (the same bytes to the same place): every wave must issue the same number of loads, because the waits
+  // count loads.
+  constexpr int A_LD = A_BLK / NW, W_LD = (W_BLK + NW - 1) / NW;  // per wave
   constexpr int NLD = A_LD + W_LD;                      // direct loads per wave and K tile
   constexpr int NFR = MT + NT;                          // fragment reads per wave and k-step
   constexpr int NMFMA = MT * NT;                        // MFMAs per wave and k-step
@@ -189,10 +198,18 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     }
 #pragma unroll
     for (int j = 0; j < W_LD; ++j) {
-      const int row = (j * NW + wave) * 8 + l_row;
-      const int key = ((((row % (16 * G)) / (4 * G)) & 3) << 1) | ((row >> 1) & 1);
-      const int r = min(n0 + row, p.N - 1);
-      w_src[j] = (uint32_t)(((int64_t)r * p.ldw + ((l_slot ^ key) << 3)) * 2);
+      const int blk = min(j * NW + wave, W_BLK - 1);
+      if constexpr (W_FP8) {  // 64-byte rows: the lane lands in slot lane%4 of row 16 blk + lane/4
+        const int row = blk * 16 + (lane >> 2);
+        const int key = ((row % (16 * G)) / (4 * G)) & 3;
+        const int r = min(n0 + row, p.N - 1);
+        w_src[j] = (uint32_t)((int64_t)r * p.ldw + (((lane & 3) ^ key) << 4));
+      } else {
+        const int row = blk * 8 + l_row;
+        const int key = ((((row % (16 * G)) / (4 * G)) & 3) << 1) | ((row >> 1) & 1);
+        const int r = min(n0 + row, p.N - 1);
+        w_src[j] = (uint32_t)(((int64_t)r * p.ldw + ((l_slot ^ key) << 3)) * 2);
+      }
     }
   };
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, -1, 0x00020000);
@@ -203,7 +220,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t*)lds_dst, 16, off, kt * (BK * 2), 0, 0);
   };
   auto load_w = [&](int kt, char* lds_dst, uint32_t off) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void_t*)lds_dst, 16, off, kt * (BK * 2), 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void_t*)lds_dst, 16, off, kt * W_ROW, 0, 0);
   };
   // Direct load number IDX (A row blocks first, then W row blocks) of K tile kt; a_base / w_base are the
   // LDS byte offsets of the operand tiles it goes to.
@@ -213,7 +230,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       load_a(kt, smem + a_base + (IDX * NW + wave) * 1024, a_src[IDX]);
     } else {
       constexpr int J = IDX - A_LD;
-      load_w(kt, smem + w_base + (J * NW + wave) * 1024, w_src[J]);
+      load_w(kt, smem + w_base + min(J * NW + wave, W_BLK - 1) * 1024, w_src[J]);
     }
   };
 
@@ -228,14 +245,41 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks) {
     x_off[ks] = (wm * WTM + fa) * 128 + (((ks * 4 + kq) ^ x_key) << 4);
-    w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * 128 + (((ks * 4 + kq) ^ w_key) << 4);
+    if constexpr (W_FP8)  // 8 bytes: half (kq%2) of chunk 2ks + kq/2, which sits in slot chunk ^ q
+      w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 2 + (kq >> 1)) ^ fq) << 4) + (kq & 1) * 8;
+    else
+      w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 4 + kq) ^ w_key) << 4);
   }
-  bf16x8_t wf[2][NT], xf[2][MT];
-  // fragment read number IDX (W fragments first, then activation fragments) of k-step ks into set b
+  // Operand fragments: two sets.  fp8 weights are read as 8 raw bytes per fragment and converted into one of
+  // two bf16 registers sets right before use.
+  bf16x8_t wf[2][W_FP8 ? 1 : NT], xf[2][MT];
+  i32x2_t wraw[2][W_FP8 ? NT : 1];
+  bf16x8_t wcv[2];
+  // Fragment read number IDX of k-step ks into set b.  bf16 weights: W fragments first (MFMAs run i-major and
+  // need every W fragment at once); fp8 weights: activation fragments first (MFMAs run j-major).
   auto read_frag = [&](int a_base, int w_base, int ks, int b, auto idx_c) {
     constexpr int IDX = decltype(idx_c)::value;
-    if constexpr (IDX < NT) wf[b][IDX] = *(const bf16x8_t*)(smem + w_base + w_off[ks] + piece_col(IDX) * 128);
-    else xf[b][IDX - NT] = *(const bf16x8_t*)(smem + a_base + x_off[ks] + (IDX - NT) * 16 * 128);
+    if constexpr (W_FP8) {
+      if constexpr (IDX < MT) xf[b][IDX] = *(const bf16x8_t*)(smem + a_base + x_off[ks] + IDX * 16 * 128);
+      else wraw[b][IDX - MT] = *(const i32x2_t*)(smem + w_base + w_off[ks] + piece_col(IDX - MT) * W_ROW);
+    } else {
+      if constexpr (IDX < NT) wf[b][IDX] = *(const bf16x8_t*)(smem + w_base + w_off[ks] + piece_col(IDX) * W_ROW);
+      else xf[b][IDX - NT] = *(const bf16x8_t*)(smem + a_base + x_off[ks] + (IDX - NT) * 16 * 128);
+    }
+  };
+  auto convert_w = [&](int b, auto j_c) {  // 8 e4m3 bytes -> 8 bf16 (exact)
+    constexpr int J = decltype(j_c)::value;
+    bf16x8_t o;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const auto p0 = __builtin_amdgcn_cvt_pk_f32_fp8(wraw[b][W_FP8 ? J : 0][h], false);
+      const auto p1 = __builtin_amdgcn_cvt_pk_f32_fp8(wraw[b][W_FP8 ? J : 0][h], true);
+      o[4 * h + 0] = (bf16_t)p0[0];
+      o[4 * h + 1] = (bf16_t)p0[1];
+      o[4 * h + 2] = (bf16_t)p1[0];
+      o[4 * h + 3] = (bf16_t)p1[1];
+    }
+    wcv[J & 1] = o;
   };
   // The MFMAs of one k-step on fragment set B, in program order (asm volatile statements keep it), with a
   // hook call after each: that is where LDS reads and direct loads are placed.  ZERO: the first k-step of an
@@ -243,12 +287,21 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   auto mfmas = [&](auto b_c, auto zero_c, auto&& hook) {
     constexpr int B = decltype(b_c)::value;
     constexpr bool ZERO = decltype(zero_c)::value;
+    if constexpr (W_FP8) convert_w(B, ic<0>{});
     static_for<NMFMA>([&](auto n) {
-      constexpr int N = decltype(n)::value, I = N / NT, J = N % NT, R = N * 4;
+      constexpr int N = decltype(n)::value;
+      // bf16 weights: i-major; fp8 weights: j-major, the next W fragment is converted while this one is used
+      constexpr int I = W_FP8 ? N % MT : N / NT, J = W_FP8 ? N / MT : N % NT, R = (I * NT + J) * 4;
+      const bf16x8_t& w = W_FP8 ? wcv[J & 1] : wf[B][W_FP8 ? 0 : J];
+      // A register written by a vector instruction must not be read by an MFMA in the next few cycles; the
+      // compiler pads that for its own MFMAs but cannot see into these.  Only the first MFMA after a
+      // conversion can be that close.
+      if constexpr (W_FP8 && I == 0) asm volatile("s_nop 3");
       if constexpr (ZERO)
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(wf[B][J]), "v"(xf[B][I]), "n"(R), "n"(R + 3));
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
       else
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(wf[B][J]), "v"(xf[B][I]), "n"(R), "n"(R + 3));
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
+      if constexpr (W_FP8 && I == 0 && J + 1 < NT) convert_w(B, ic<J + 1>{});
       hook(n);
     });
   };
@@ -405,6 +458,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         bias_v[j] = bf16x4_t{0, 0, 0, 0};
         if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + nc);
       }
+      f32x4_t scale_v[W_FP8 ? NT : 1];
+      if constexpr (W_FP8) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) scale_v[j] = *(const f32x4_t*)(p.w_scale + min(n_lane + piece_col(j), p.N - 4));
+      }
       constexpr bool ADDEND = (EPI == CS_EPI_RESIDUAL) || (EPI == CS_EPI_BIAS_POS);
       bf16x4_t addend[ADDEND ? MT : 1][ADDEND ? NT : 1];
       auto load_addend = [&](auto i_c) {
@@ -438,7 +496,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         for (int j = 0; j < NT; ++j) {
           float v[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r) v[r] = racc[j][r] + bf2f(bias_v[j][r]);
+          for (int r = 0; r < 4; ++r)
+            v[r] = (W_FP8 ? racc[j][r] * scale_v[W_FP8 ? j : 0][r] : racc[j][r]) + bf2f(bias_v[j][r]);
           if (EPI == CS_EPI_SWIGLU) {
             // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the
             // product stay in fp32 until the single output rounding
@@ -510,14 +569,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8>
 int launch(const CsGemmArgs& a, hipStream_t stream) {
   CsGemmArgs p = a;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
-  constexpr int lds = RingShape<BM, BN>::BYTES;
+  constexpr int lds = RingShape<BM, BN, W_FP8>::BYTES;
   static bool attr_set = false;
-  auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI>;
+  auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8>;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return CS_ERR_LAUNCH;
@@ -530,18 +589,28 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   return cs_launch_status();
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-int dispatch_epi(const CsGemmArgs& a, hipStream_t s) {
+template <int BM, int BN, int WAVES_M, int WAVES_N, bool W_FP8>
+int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
   switch (a.epilogue) {
     case CS_EPI_BIAS:
-      if (a.pos) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS_POS>(a, s);
-      return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS>(a, s);
-    case CS_EPI_RESIDUAL: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL>(a, s);
-    case CS_EPI_SWIGLU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_SWIGLU>(a, s);
-    case CS_EPI_GELU_ERF: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_ERF>(a, s);
-    case CS_EPI_GELU_TANH: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_TANH>(a, s);
+      if constexpr (!W_FP8) {
+        if (a.pos) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS_POS, false>(a, s);
+      }
+      return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, W_FP8>(a, s);
+    case CS_EPI_RESIDUAL: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, W_FP8>(a, s);
+    case CS_EPI_SWIGLU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_SWIGLU, W_FP8>(a, s);
+    case CS_EPI_GELU_ERF:
+      if constexpr (W_FP8 && BN == 160) return CS_ERR_UNSUPPORTED;  // never dispatched, see cs_gemm_fast
+      else return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_ERF, W_FP8>(a, s);
+    case CS_EPI_GELU_TANH: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_TANH, W_FP8>(a, s);
     default: return CS_ERR_INVALID_ARG;
   }
+}
+
+template <int BM, int BN, int WAVES_M, int WAVES_N>
+int dispatch_epi(const CsGemmArgs& a, hipStream_t s) {
+  if (a.w_fp8) return dispatch_epi_w<BM, BN, WAVES_M, WAVES_N, true>(a, s);
+  return dispatch_epi_w<BM, BN, WAVES_M, WAVES_N, false>(a, s);
 }
 
 // Time of a launch in units of "one 256x256 tile on every CU": rounds of 256 workgroups times tile area.
@@ -556,20 +625,24 @@ double rounds_cost(int M, int N, int bm, int bn) {
 // Called by cs_gemm after argument validation.  Sets *handled when this path took the problem.
 int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   *handled = false;
-  if (a.w_fp8 || a.w_scale || a.M < 1 || a.N < 8) return CS_OK;
+  if (a.M < 1 || a.N < 8) return CS_OK;
+  if (a.w_fp8 ? (!a.w_scale || a.pos) : (a.w_scale != nullptr)) return CS_OK;
   if (a.K % BK || a.K < 3 * BK) return CS_OK;  // the ring pipeline is written for at least three K tiles
   if (a.N % 8 || a.ldc % 8 || ((uintptr_t)a.C & 15)) return CS_OK;  // 16-byte output stores
   if (a.pos && a.epilogue != CS_EPI_BIAS) return CS_OK;  // the position addend only pairs with the plain epilogue here
   if (a.a_rows) return CS_OK;  // gathered A rows can lie anywhere: the general kernel keeps 64-bit pointers
   // per-lane source offsets are 32-bit byte offsets from the matrix bases
-  if ((int64_t)a.M * a.lda * 2 >= (int64_t)UINT32_MAX || (int64_t)a.N * a.ldw * 2 >= (int64_t)UINT32_MAX) return CS_OK;
+  if ((int64_t)a.M * a.lda * 2 >= (int64_t)UINT32_MAX || (int64_t)a.N * a.ldw * (a.w_fp8 ? 1 : 2) >= (int64_t)UINT32_MAX)
+    return CS_OK;
   *handled = true;
   // Tile shape: the one that needs the least chip time (tile quantisation over the 256 CUs).  The narrow
   // 256x160 tile exists for N = 1280 (8 column tiles: 8192 rows give exactly 256 workgroups).
   const double c256 = rounds_cost(a.M, a.N, 256, 256);
   const double c160 = rounds_cost(a.M, a.N, 256, 160) * 1.15;  // narrower tiles: more LDS and L2 traffic per FLOP
   static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160" or "256"
-  if (force ? force[0] == '1' : c160 < c256) return dispatch_epi<256, 160, 4, 1>(a, stream);
+  // (the erf GELU epilogue with fp8 scales does not fit the architectural registers of the 256x160 form)
+  const bool fits160 = !(a.w_fp8 && a.epilogue == CS_EPI_GELU_ERF);
+  if (fits160 && (force ? force[0] == '1' : c160 < c256)) return dispatch_epi<256, 160, 4, 1>(a, stream);
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller
   // tiles (256x128 or 128x192: more workgroups, each shorter).  The two launches write disjoint column
@@ -600,7 +673,8 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
       CsGemmArgs lo = a, hi = a;
       lo.N = n1;
       hi.N = a.N - n1;
-      hi.W = (const char*)a.W + (int64_t)n1 * a.ldw * 2;
+      hi.W = (const char*)a.W + (int64_t)n1 * a.ldw * (a.w_fp8 ? 1 : 2);
+      if (a.w_scale) hi.w_scale = a.w_scale + n1;
       if (a.bias) hi.bias = (const char*)a.bias + (int64_t)n1 * 2;
       if (a.residual) hi.residual = (const char*)a.residual + (int64_t)n1 * 2;
       if (a.pos) hi.pos = (const char*)a.pos + (int64_t)n1 * 2;

@@ -217,6 +217,29 @@ def test_gemm_fast_path_forms(ops, dev, M, N, K):
     assert torch.equal(scat, ref)
 
 
+@pytest.mark.parametrize("M,N,K", [
+    (8192, 3072, 192),    # 256x256 (three-stage ring with byte-wide W tiles) + 256x128 remainder, 3 K tiles
+    (8192, 2304, 256),    # 256x256 + 128x192 remainder
+    (1000, 1280, 320),    # 256x160: 10 W row blocks over 4 waves (two waves repeat the last block)
+    (300, 520, 448),      # row and column tails
+])
+def test_gemm_fast_path_forms_fp8_weights(ops, dev, M, N, K):
+    a, b = rnd((M, K), 1.0, 21, dev), rnd((N,), 0.02, 23, dev)
+    res = rnd((M, N), 1.0, 24, dev)
+    w = torch.randn(N, K, generator=torch.Generator().manual_seed(22)) * 0.05
+    scale = w.abs().amax(dim=1) / 448.0
+    q = (w / scale[:, None]).to(torch.float8_e4m3fn)
+    wd = q.float() * scale[:, None]          # de-quantised fp32 weights: the comparator of the fp8 path
+    rows = torch.cat([torch.arange(0, M, max(1, M // 257)), torch.tensor([M - 1])])
+    base = (a[rows].float().cpu() @ wd.t() + b.float().cpu()).bfloat16().float()
+    qd, sd = q.to(dev), scale.to(dev)
+    for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_SWIGLU):
+        got = ops.gemm(a, qd, b, w_scale=sd, epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
+        close(got[rows], _epilogue_ref(ops, epi, base, res[rows]), 2**-7, f"fp8 {M}x{N}x{K} epilogue {epi}")
+    first = ops.gemm(a, qd, b, w_scale=sd)
+    assert torch.equal(ops.gemm(a, qd, b, w_scale=sd), first)
+
+
 def test_gemm_row_maps(ops, dev):
     M, N, K = 400, 512, 256
     a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
