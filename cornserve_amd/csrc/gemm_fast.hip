@@ -120,7 +120,13 @@ struct RingShape {
 // W_FP8: the weights are e4m3 bytes with a per-output-channel fp32 scale.  W tiles travel and sit in LDS as bytes
 // (half the traffic); a fragment is converted to bf16 in registers right before its MFMAs (exact: every e4m3
 // value is a bf16 value) and the scale is applied to the fp32 accumulators in the epilogue.
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8>
+//
+// FUSE: 0 = plain; FUSE_NORM_A = the rows of A stand for their RMS-normalised form: the accumulators are multiplied
+// by rsqrt(sum of squares of the A row / K + eps) before the bias (the norm's weight is folded into W by the
+// caller); FUSE_SUMSQ_C = besides C, the sum of squares of every output row over this tile's columns goes to
+// c_row_sumsq (what the next FUSE_NORM_A launch reads).
+constexpr int FUSE_NORM_A = 1, FUSE_SUMSQ_C = 2;
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE>
 __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   static_assert(WAVES_M * WAVES_N == NW, "four waves, one per SIMD");
@@ -451,6 +457,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         const int mc = min(mrow[i], p.M - 1);
         crow[i] = p.c_rows ? p.c_rows[mc] : mc;
       }
+      float rstd[FUSE == FUSE_NORM_A ? MT : 1];
+      if constexpr (FUSE == FUSE_NORM_A) {
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const float* parts = p.a_row_sumsq + (int64_t)min(mrow[i], p.M - 1) * CS_SUMSQ_PARTS;
+          const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
+          const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
+          rstd[i] = rsqrtf(ss / (float)p.K + p.norm_eps);
+        }
+      }
       bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
@@ -496,8 +512,12 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         for (int j = 0; j < NT; ++j) {
           float v[4];
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            v[r] = (W_FP8 ? racc[j][r] * scale_v[W_FP8 ? j : 0][r] : racc[j][r]) + bf2f(bias_v[j][r]);
+          for (int r = 0; r < 4; ++r) {
+            float t = racc[j][r];
+            if constexpr (W_FP8) t *= scale_v[W_FP8 ? j : 0][r];
+            if constexpr (FUSE == FUSE_NORM_A) t *= rstd[FUSE == FUSE_NORM_A ? i : 0];
+            v[r] = t + bf2f(bias_v[j][r]);
+          }
           if (EPI == CS_EPI_SWIGLU) {
             // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the
             // product stay in fp32 until the single output rounding
@@ -519,6 +539,24 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
 #pragma unroll
             for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
           }
+        }
+        if constexpr (FUSE == FUSE_SUMSQ_C) {
+          // Sum of squares of the row's ROUNDED outputs over this wave's columns: lane-local over the lane's
+          // pieces, then over the four lanes of the row (fixed order: the result does not depend on timing).
+          static_assert(WAVES_N == 1 && EPI != CS_EPI_SWIGLU, "one wave spans the tile's columns: one part per tile");
+          float ss = 0.f;
+#pragma unroll
+          for (int j = 0; j < NT; ++j) {
+            const bool nok = n_lane + piece_col(j) < p.N;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float o = bf2f(out[j][r]);
+              ss += nok ? o * o : 0.f;
+            }
+          }
+          ss += __shfl_xor(ss, 16);
+          ss += __shfl_xor(ss, 32);
+          if (mok && kq == 0) p.c_row_sumsq[(int64_t)crow[i] * CS_SUMSQ_PARTS + n0 / BN] = ss;
         }
         // With G == 2 the pieces of fragments 2g and 2g+1 are adjacent: one 16-byte store per lane, and the
         // four lanes of an output row write 64 consecutive bytes (32 with the halved SwiGLU output).
@@ -569,14 +607,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE = 0>
 int launch(const CsGemmArgs& a, hipStream_t stream) {
   CsGemmArgs p = a;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   constexpr int lds = RingShape<BM, BN, W_FP8>::BYTES;
   static bool attr_set = false;
-  auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8>;
+  auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE>;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return CS_ERR_LAUNCH;
@@ -591,6 +629,24 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
 
 template <int BM, int BN, int WAVES_M, int WAVES_N, bool W_FP8>
 int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
+  if constexpr (!W_FP8) {
+    // the fused-norm forms exist for the epilogues an encoder block pairs them with
+    if (a.a_row_sumsq) {
+      if (a.pos || a.c_row_sumsq) return CS_ERR_UNSUPPORTED;
+      if (a.epilogue == CS_EPI_BIAS) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_NORM_A>(a, s);
+      if (a.epilogue == CS_EPI_SWIGLU) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_SWIGLU, false, FUSE_NORM_A>(a, s);
+      return CS_ERR_UNSUPPORTED;
+    }
+    if (a.c_row_sumsq) {
+      if constexpr (BN == 160 && WAVES_N == 1) {
+        if (a.epilogue == CS_EPI_RESIDUAL) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_SUMSQ_C>(a, s);
+        if (a.epilogue == CS_EPI_BIAS && !a.pos) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_SUMSQ_C>(a, s);
+      }
+      return CS_ERR_UNSUPPORTED;
+    }
+  } else {
+    if (a.a_row_sumsq || a.c_row_sumsq) return CS_ERR_UNSUPPORTED;
+  }
   switch (a.epilogue) {
     case CS_EPI_BIAS:
       if constexpr (!W_FP8) {
@@ -642,6 +698,11 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160" or "256"
   // (the erf GELU epilogue with fp8 scales does not fit the architectural registers of the 256x160 form)
   const bool fits160 = !(a.w_fp8 && a.epilogue == CS_EPI_GELU_ERF);
+  // Row sums of squares come in CS_SUMSQ_PARTS parts, one per column tile of the 256x160 form.
+  if (a.c_row_sumsq) {
+    if (a.N > CS_SUMSQ_PARTS * 160 || a.w_fp8) return CS_ERR_UNSUPPORTED;
+    return dispatch_epi<256, 160, 4, 1>(a, stream);
+  }
   if (fits160 && (force ? force[0] == '1' : c160 < c256)) return dispatch_epi<256, 160, 4, 1>(a, stream);
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller

@@ -109,7 +109,13 @@ def quantize_fp8_rows(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
 
 
 class Qwen2_5_VisionTransformer(EricModel):
-    def __init__(self, config: Any, weight_format: str = "bf16") -> None:
+    def __init__(self, config: Any, weight_format: str = "bf16", fold_norm: bool = True) -> None:
+        """`fold_norm`: apply norm1 / norm2 of every block inside the GEMM that follows them (the norm weight is
+        folded into that GEMM's weight columns at pack time, the per-row rsqrt is applied to the fp32
+        accumulators, and the row sums of squares come out of the GEMM that wrote the residual stream).  The
+        normalised activations are then never rounded to bf16 on their own, unlike the reference
+        (norm.py:35-70 followed by F.linear): results stay inside the parity tolerance but are not
+        bit-identical to the unfolded path.  Only with bf16 weights and a hidden size the fast GEMM takes."""
         super().__init__()
         vc = config.vision_config if hasattr(config, "vision_config") else config
         if weight_format not in ("bf16", "fp8_e4m3"):
@@ -130,6 +136,8 @@ class Qwen2_5_VisionTransformer(EricModel):
         if getattr(vc, "hidden_act", "silu") != "silu":
             raise NotImplementedError("only the SiLU-gated MLP of Qwen2.5-VL is implemented")
         self.head_dim = self.hidden_size // self.num_heads
+        H = self.hidden_size
+        self.fold_norm = bool(fold_norm) and weight_format == "bf16" and H % 64 == 0 and 192 <= H <= 160 * ops.SUMSQ_PARTS
 
         self.patch_embed = _PatchEmbed(self.in_channels, self.hidden_size, self.temporal_patch_size, self.patch_size)
         self.blocks = nn.ModuleList([_Block(self.hidden_size, self.intermediate_size) for _ in range(vc.depth)])
@@ -182,11 +190,15 @@ class Qwen2_5_VisionTransformer(EricModel):
             gu_b[1 : 2 * I : 2] = blk.mlp.up_proj.bias
             down_w = torch.zeros((H, Ip), dtype=self.dtype, device=dev)
             down_w[:, :I] = blk.mlp.down_proj.weight
+            qkv_w = blk.attn.qkv.weight
+            if self.fold_norm:
+                qkv_w = (qkv_w.float() * blk.norm1.weight.float()[None, :]).to(self.dtype)
+                gu_w = (gu_w.float() * blk.norm2.weight.float()[None, :]).to(self.dtype)
             blocks.append(
                 {
                     "n1": blk.norm1.weight,
                     "n2": blk.norm2.weight,
-                    "qkv": self._lin(blk.attn.qkv.weight, blk.attn.qkv.bias),
+                    "qkv": self._lin(qkv_w, blk.attn.qkv.bias),
                     "proj": self._lin(blk.attn.proj.weight, blk.attn.proj.bias),
                     "gu": self._lin(gu_w, gu_b),
                     "down": self._lin(down_w, blk.mlp.down_proj.bias),
@@ -260,6 +272,15 @@ class Qwen2_5_VisionTransformer(EricModel):
         mark("patch_embed")
         x = ops.gemm(pixel_values, pk["pe_w"], None, a_rows=ix.src_rows)
         n = torch.empty_like(x)
+        # the folded-norm GEMMs exist in the fast kernel only, whose per-lane byte offsets are 32-bit
+        fold = self.fold_norm
+        if fold and L * max(3 * H, pk["Ip"]) * 2 >= 2**32:
+            raise ValueError(f"{L} patches in one forward exceed what the folded-norm GEMMs address; split the batch "
+                             "or construct the model with fold_norm=False")
+        eps = self.norm_eps
+        if fold:
+            mark("norm")
+            ss = ops.row_sumsq(x, out=torch.zeros((L, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev))
         qkv = torch.empty((L, 3 * H), dtype=torch.bfloat16, device=dev)
         att = torch.empty((L, H), dtype=torch.bfloat16, device=dev)
         hmid = torch.empty((L, pk["Ip"]), dtype=torch.bfloat16, device=dev)
@@ -267,20 +288,31 @@ class Qwen2_5_VisionTransformer(EricModel):
         for i, b in enumerate(pk["blocks"]):
             full = i in self.fullatt_block_indexes
             plan = plan_full if full else plan_win
-            mark("norm")
-            ops.rmsnorm(x, b["n1"], self.norm_eps, out=n)
-            mark("gemm_qkv")
-            self._g(n, b["qkv"], out=qkv)
+            if fold:
+                mark("gemm_qkv")
+                self._g(x, b["qkv"], out=qkv, a_row_sumsq=ss, norm_eps=eps)
+            else:
+                mark("norm")
+                ops.rmsnorm(x, b["n1"], eps, out=n)
+                mark("gemm_qkv")
+                self._g(n, b["qkv"], out=qkv)
             mark("attn_full" if full else "attn_window")
             ops.attn_varlen(qkv[:, :H], qkv[:, H : 2 * H], qkv[:, 2 * H :], plan, nh, d, scale, cos_sin=ix.cos_sin, out=att)
             mark("gemm_proj")
-            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
-            mark("norm")
-            ops.rmsnorm(x, b["n2"], self.norm_eps, out=n)
-            mark("gemm_gate_up")
-            self._g(n, b["gu"], epilogue=ops.EPI_SWIGLU, out=hmid)
-            mark("gemm_down")
-            self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+            if fold:
+                self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss)
+                mark("gemm_gate_up")
+                self._g(x, b["gu"], epilogue=ops.EPI_SWIGLU, out=hmid, a_row_sumsq=ss, norm_eps=eps)
+                mark("gemm_down")
+                self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss)
+            else:
+                self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+                mark("norm")
+                ops.rmsnorm(x, b["n2"], eps, out=n)
+                mark("gemm_gate_up")
+                self._g(n, b["gu"], epilogue=ops.EPI_SWIGLU, out=hmid)
+                mark("gemm_down")
+                self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
 
         mark("norm")
         ops.rmsnorm(x, pk["ln_q"], self.norm_eps, out=n)

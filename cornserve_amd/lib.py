@@ -17,7 +17,7 @@ CS_ERR_INVALID_ARG = 1
 CS_ERR_UNSUPPORTED = 2
 CS_ERR_LAUNCH = 3
 CS_ERR_TOO_LARGE = 4
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH = range(5)
 
@@ -48,6 +48,9 @@ class CsGemmArgs(ctypes.Structure):
         ("w_fp8", c_int32),
         ("tiles_m", c_int32),
         ("tiles_n", c_int32),
+        ("a_row_sumsq", c_void_p),
+        ("c_row_sumsq", c_void_p),
+        ("norm_eps", ctypes.c_float),
     ]
 
 
@@ -55,6 +58,7 @@ class CsGemmArgs(ctypes.Structure):
 _SIGNATURES: dict[str, list] = {
     "cs_abi_version": [],
     "cs_gemm": [POINTER(CsGemmArgs), c_void_p],
+    "cs_row_sumsq": [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p],
     "cs_rmsnorm": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_float, c_int32, c_void_p],
     "cs_layernorm": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_float, c_void_p],
     "cs_vit_seqlens_host": [

@@ -54,8 +54,15 @@ def gemm(
     c_rows: torch.Tensor | None = None,
     out: torch.Tensor | None = None,
     k: int | None = None,
+    a_row_sumsq: torch.Tensor | None = None,
+    c_row_sumsq: torch.Tensor | None = None,
+    norm_eps: float = 0.0,
 ) -> torch.Tensor:
-    """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`."""
+    """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`.
+
+    `a_row_sumsq` (fp32 [M, SUMSQ_PARTS]) scales row m of the product by rsqrt(sum(parts)/K + norm_eps): an
+    RMSNorm of `a` whose weight the caller has folded into the columns of `w`.  `c_row_sumsq` (same layout,
+    indexed by output row) receives the sums of squares of the output rows."""
     lib = _l.load()
     _req(a, torch.bfloat16, "a")
     if a.dim() != 2 or w.dim() != 2:
@@ -89,11 +96,34 @@ def gemm(
     args.M, args.N, args.K = M, N, K
     args.epilogue = epilogue
     args.w_fp8 = 1 if fp8 else 0
+    for name, t in (("a_row_sumsq", a_row_sumsq), ("c_row_sumsq", c_row_sumsq)):
+        if t is not None:
+            _req(t, torch.float32, name)
+            if t.dim() != 2 or t.shape[1] != SUMSQ_PARTS or not t.is_contiguous() or t.shape[0] < M:
+                raise ValueError(f"{name} must be a contiguous fp32 [>=M, {SUMSQ_PARTS}] tensor")
+    args.a_row_sumsq = _ptr(a_row_sumsq)
+    args.c_row_sumsq = _ptr(c_row_sumsq)
+    args.norm_eps = norm_eps
     _l.check(lib.cs_gemm(ctypes.byref(args), _stream()), "cs_gemm")
     return out
 
 
 # -------------------------------------------------------------------------------------------- norms
+SUMSQ_PARTS = 8  # CS_SUMSQ_PARTS
+
+
+def row_sumsq(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 [rows, SUMSQ_PARTS]: sums of squares of the rows of `x` in parts of 160 columns."""
+    lib = _l.load()
+    _req(x, torch.bfloat16, "x")
+    if x.dim() != 2:
+        raise ValueError("row_sumsq takes a 2-D tensor")
+    if out is None:
+        out = torch.empty((x.shape[0], SUMSQ_PARTS), dtype=torch.float32, device=x.device)
+    _l.check(lib.cs_row_sumsq(x.data_ptr(), x.stride(0), x.shape[0], x.shape[1], out.data_ptr(), _stream()), "cs_row_sumsq")
+    return out
+
+
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, *, gemma: bool = False,
             out: torch.Tensor | None = None) -> torch.Tensor:
     lib = _l.load()

@@ -36,7 +36,7 @@ extern "C" {
 #define CS_ERR_TOO_LARGE 4
 
 /* ABI version of this header; cs_abi_version() returns the value the library was built with. */
-#define CS_ABI_VERSION 1
+#define CS_ABI_VERSION 2
 int cs_abi_version(void);
 
 /* ------------------------------------------------------------------------------------------------
@@ -75,7 +75,21 @@ typedef struct CsGemmArgs {
   int32_t epilogue;      /* enum CsEpilogue                                                      */
   int32_t w_fp8;
   int32_t tiles_m, tiles_n; /* filled in by the library                                          */
+  /* RMSNorm folded into the neighbouring GEMMs (qwen2_5_vl.py:173-177: norm1 -> qkv, norm2 -> gate|up).
+   * rsqrt(mean(x^2) + eps) is a per-row scalar, so  bf16(x*rstd) * w_norm . W^T  ==  rstd * (x . (W*w_norm)^T)
+   * up to the rounding of the normalised activations: the caller folds w_norm into W's columns, passes the
+   * residual stream itself as A, and the row scalar is applied to the fp32 accumulators.
+   * a_row_sumsq: optional fp32 [M][CS_SUMSQ_PARTS]; the parts of row m add up to sum_k A[m,k]^2.  The
+   *   epilogue becomes  y = acc * rsqrt(sum/K + norm_eps) (+ bias) ...   (CS_EPI_BIAS and CS_EPI_SWIGLU, bf16 W).
+   * c_row_sumsq: optional fp32 [M][CS_SUMSQ_PARTS], indexed by OUTPUT row; part p receives the sum of squares
+   *   of the rounded outputs C[m, 160p .. 160p+159], for the parts N covers (the caller zeroes the others once).
+   *   CS_EPI_BIAS and CS_EPI_RESIDUAL, bf16 W, N <= 160 * CS_SUMSQ_PARTS.
+   * Unsupported combinations return CS_ERR_UNSUPPORTED (nothing is launched).                      */
+  const float* a_row_sumsq;
+  float* c_row_sumsq;
+  float norm_eps;
 } CsGemmArgs;
+#define CS_SUMSQ_PARTS 8
 
 /* Constraints: K % 8 == 0 (16 with fp8), lda/ldw % 8 == 0, N % 4 == 0, A and W 16-byte aligned. */
 int cs_gemm(const CsGemmArgs* args, void* stream);
@@ -87,6 +101,10 @@ int cs_gemm(const CsGemmArgs* args, void* stream);
  * gemma = 1 selects GemmaRMSNorm, norm.py:90-113: y = bf16(x * rsqrt(..) * (1 + w)).              */
 int cs_rmsnorm(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, int32_t rows, int32_t H,
                float eps, int32_t gemma, void* stream);
+/* Sum of squares of every row of x (bf16 [rows,H], H <= 160 * CS_SUMSQ_PARTS) in the layout of
+ * CsGemmArgs.c_row_sumsq: out[m][p] = sum of x[m, 160p .. 160p+159]^2, parts beyond H are written as 0.
+ * The variance term of RMSNorm (norm.py:35-70) for a GEMM launched with a_row_sumsq.               */
+int cs_row_sumsq(const void* x, int64_t ldx, int32_t rows, int32_t H, float* out, void* stream);
 /* nn.LayerNorm with affine, siglip.py:173-175,333.                                                */
 int cs_layernorm(const void* x, int64_t ldx, const void* w, const void* b, void* y, int64_t ldy,
                  int32_t rows, int32_t H, float eps, void* stream);

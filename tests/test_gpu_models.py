@@ -40,12 +40,12 @@ def check(got: torch.Tensor, ref: torch.Tensor, rel: float, what: str):
     assert err <= rel, f"{what}: max rel err {err:.4g} > {rel}"
 
 
-def build_qwen(dev, depth, fullatt, seed, weight_format="bf16"):
+def build_qwen(dev, depth, fullatt, seed, weight_format="bf16", fold_norm=True):
     from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
 
     cfg = synth.qwen_vision_config(depth=depth, fullatt_block_indexes=fullatt)
     sd = synth.qwen_state_dict(cfg, seed=seed)
-    model = Qwen2_5_VisionTransformer(cfg, weight_format=weight_format)
+    model = Qwen2_5_VisionTransformer(cfg, weight_format=weight_format, fold_norm=fold_norm)
     inc = model.load_state_dict(sd, strict=False)
     assert not inc.missing_keys and not inc.unexpected_keys
     model = model.to(device=dev, dtype=torch.bfloat16).eval()
@@ -65,6 +65,23 @@ def test_qwen_cfg1_shape_against_oracle_and_golden(dev, golden_dir):
     check(out[0], ref_f32, REL_BF16, "cfg1 vs fp32 oracle")
     gold = np.load(golden_dir / "qwen2_5_vl_cfg1.npz")   # Hugging Face fp32 output, every 16th column
     check(out[0][:, ::16], torch.from_numpy(gold["sample"]), REL_BF16, "cfg1 vs committed golden sample")
+
+
+def test_qwen_without_folded_norms(dev, golden_dir):
+    """The same network with every RMSNorm as its own kernel (the reference's rounding points exactly), and
+    the distance between the two forms."""
+    model, sd, ocfg = build_qwen(dev, 4, (3,), seed=1, fold_norm=False)
+    assert not model.fold_norm
+    px, grid = synth.qwen_inputs([(1, 32, 32)], seed=1)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})[0]
+    check(out, oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)[0], REL_BF16, "unfolded vs bf16 oracle")
+    check(out, oq.forward(sd, ocfg, px, grid, dtype=torch.float32)[0], REL_BF16, "unfolded vs fp32 oracle")
+    gold = np.load(golden_dir / "qwen2_5_vl_cfg1.npz")
+    check(out[:, ::16], torch.from_numpy(gold["sample"]), REL_BF16, "unfolded vs committed golden sample")
+    folded, _, _ = build_qwen(dev, 4, (3,), seed=1)
+    assert folded.fold_norm
+    out_f = folded(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})[0]
+    check(out_f, out, REL_BF16, "folded vs unfolded")
 
 
 def test_qwen_multi_image_ragged_and_video(dev):

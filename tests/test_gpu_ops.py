@@ -240,6 +240,84 @@ def test_gemm_fast_path_forms_fp8_weights(ops, dev, M, N, K):
     assert torch.equal(ops.gemm(a, qd, b, w_scale=sd), first)
 
 
+def _sumsq_parts_ref(x: torch.Tensor) -> torch.Tensor:
+    """fp32 [rows, 8]: sums of squares of 160-column blocks of x (zero where x has no such columns)."""
+    rows, H = x.shape
+    pad = torch.zeros((rows, 1280), dtype=torch.float32)
+    pad[:, :H] = x.float().cpu()
+    return (pad * pad).view(rows, 8, 160).sum(-1)
+
+
+@pytest.mark.parametrize("rows,H", [(1, 1280), (1000, 1280), (77, 1152), (5, 64), (3, 160)])
+def test_row_sumsq(ops, dev, rows, H):
+    x = rnd((rows, H), 2.0, 31, dev)
+    got = ops.row_sumsq(x)
+    ref = _sumsq_parts_ref(x)
+    assert got.shape == (rows, 8) and got.dtype == torch.float32
+    torch.testing.assert_close(got.cpu(), ref, rtol=1e-5, atol=1e-6)
+    assert (got.cpu()[:, (H + 159) // 160:] == 0).all()
+    with pytest.raises(RuntimeError):
+        ops.row_sumsq(rnd((4, 1288), 1.0, 1, dev))
+
+
+# RMSNorm folded into the GEMMs on both sides of it: the producer (residual epilogue) emits the sums of squares
+# of the rows it writes, the consumer scales its accumulators by rsqrt(mean square + eps).
+@pytest.mark.parametrize("M,N,K", [(8192, 1280, 192), (1000, 1280, 320), (300, 1152, 448), (257, 168, 192)])
+def test_gemm_emits_row_sums_of_squares(ops, dev, M, N, K):
+    a, w, b = rnd((M, K), 1.0, 41, dev), rnd((N, K), 0.05, 42, dev), rnd((N,), 0.02, 43, dev)
+    res = rnd((M, N), 1.0, 44, dev)
+    for epi in (ops.EPI_RESIDUAL, ops.EPI_BIAS):
+        kw = dict(epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
+        plain = ops.gemm(a, w, b, **kw)
+        ss = torch.full((M, 8), 7.0, dtype=torch.float32, device=dev)
+        got = ops.gemm(a, w, b, c_row_sumsq=ss, **kw)
+        assert torch.equal(got, plain)                       # C itself is unchanged by the extra output
+        ref = _sumsq_parts_ref(plain)                        # ... and the sums are those of the ROUNDED outputs
+        parts = (N + 159) // 160
+        torch.testing.assert_close(ss.cpu()[:, :parts], ref[:, :parts], rtol=1e-5, atol=1e-6)
+        assert (ss.cpu()[:, parts:] == 7.0).all()            # parts beyond N are left to the caller
+        ss2 = torch.zeros_like(ss)
+        ops.gemm(a, w, b, c_row_sumsq=ss2, **kw)
+        assert torch.equal(ss2[:, :parts], ss[:, :parts])    # fixed summation order: identical bits
+    perm = torch.randperm(M, generator=torch.Generator().manual_seed(3)).int().to(dev)
+    ss = torch.zeros((M, 8), dtype=torch.float32, device=dev)
+    scat = ops.gemm(a, w, b, c_rows=perm, c_row_sumsq=ss)
+    torch.testing.assert_close(ss.cpu(), _sumsq_parts_ref(scat), rtol=1e-5, atol=1e-6)   # indexed by output row
+
+
+@pytest.mark.parametrize("M,N,K", [(8192, 3072, 192), (8192, 2304, 256), (1000, 1280, 320), (300, 520, 448)])
+def test_gemm_with_folded_rmsnorm(ops, dev, M, N, K):
+    eps = 1e-6
+    a, w, b = rnd((M, K), 3.0, 51, dev), rnd((N, K), 0.05, 52, dev), rnd((N,), 0.02, 53, dev)
+    g = (1.0 + rnd((K,), 0.1, 54)).bfloat16()                           # the norm's weight
+    wf = (w.float().cpu() * g.float()[None, :]).bfloat16().to(dev)     # folded into W's columns
+    ss = ops.row_sumsq(a)
+    rows = torch.cat([torch.arange(0, M, max(1, M // 257)), torch.tensor([M - 1])])
+    af = a[rows].float().cpu()
+    rstd = torch.rsqrt((af * af).mean(-1, keepdim=True) + eps)
+    # closed form of the fused op in fp32 ...
+    base = ((af @ wf.float().cpu().t()) * rstd + b.float().cpu()).bfloat16().float()
+    # ... and the unfused reference sequence (norm.py:35-70 then F.linear): cast, multiply by the weight, cast
+    n_ref = ((af * rstd).bfloat16().float() * g.float()).bfloat16()
+    base_unfused = lin_ref(n_ref, w, b).bfloat16().float()
+    for epi in (ops.EPI_BIAS, ops.EPI_SWIGLU):
+        if epi == ops.EPI_SWIGLU and (N // 2) % 8:   # output rows the fast kernel's 16-byte stores cannot take
+            with pytest.raises(RuntimeError):
+                ops.gemm(a, wf, b, epilogue=epi, a_row_sumsq=ss, norm_eps=eps)
+            continue
+        got = ops.gemm(a, wf, b, epilogue=epi, a_row_sumsq=ss, norm_eps=eps)
+        close(got[rows], _epilogue_ref(ops, epi, base, None), 2**-7, f"folded norm {M}x{N}x{K} epilogue {epi}")
+        close(got[rows], _epilogue_ref(ops, epi, base_unfused, None), 2**-6, f"folded vs unfused {M}x{N}x{K} epilogue {epi}")
+    # against the library's own unfused pair
+    unfused = ops.gemm(ops.rmsnorm(a, g.to(dev), eps), w, b)
+    close(ops.gemm(a, wf, b, a_row_sumsq=ss, norm_eps=eps), unfused.float().cpu(), 2**-6, "folded vs rmsnorm + gemm")
+    # combinations that do not exist are refused, not silently computed without the norm
+    with pytest.raises(RuntimeError):
+        ops.gemm(a, wf, b, epilogue=ops.EPI_GELU_ERF, a_row_sumsq=ss, norm_eps=eps)
+    with pytest.raises(RuntimeError):
+        ops.gemm(a[:, :72].contiguous(), wf[:, :72].contiguous(), b, a_row_sumsq=ss, norm_eps=eps)   # K the fast kernel does not take
+
+
 def test_gemm_row_maps(ops, dev):
     M, N, K = 400, 512, 256
     a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
