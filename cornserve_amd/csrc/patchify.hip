@@ -1,4 +1,5 @@
-// Strided patch gather for the SigLIP patch embedding (gfx950).
+// Patch layout kernels (gfx950): strided patch gather for the SigLIP patch embedding, and uint8 frames ->
+// normalised patch rows for the Qwen2-VL family.
 //
 // nn.Conv2d(C, E, kernel=stride=p, padding="valid") (eric/models/layers/siglip.py:30-36,94-95) over
 // NCHW pixels equals a GEMM between the flattened non-overlapping patches and the [E, C*p*p] weight.
@@ -34,7 +35,82 @@ __global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict_
   }
 }
 
+// Qwen2-VL family: resized uint8 frames [T,H,W,3] -> the flat patch rows the encoder consumes, with the
+// rescale + normalise step applied through a per-channel table of the 256 byte values (so the arithmetic of
+// the caller's image processor is reproduced bit for bit whatever its operation order: the caller computes
+// the table with it).  Rows are ordered (t, block row, block col, row in block, col in block) with blocks of
+// merge x merge patches, columns (channel, temporal, y, x); temporal slot tt of row group t shows frame
+// min(t*temporal + tt, T-1): an image is one frame repeated, a video's last frame is repeated to fill a group.
+// One thread writes two neighbouring x of one output row; the table sits in LDS.
+template <typename OUT>
+__global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __restrict__ frames, int T, int H, int W,
+                                                               int p, int m, int tps, const float* __restrict__ table,
+                                                               OUT* __restrict__ out, int64_t ldo, int64_t total_pairs) {
+  __shared__ float lut[3 * 256];
+  for (int i = threadIdx.x; i < 3 * 256; i += 256) lut[i] = table[i];
+  __syncthreads();
+  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total_pairs) return;
+  const int hp = p >> 1;
+  const int xp = (int)(i % hp);
+  i /= hp;
+  const int py = (int)(i % p);
+  i /= p;
+  const int tt = (int)(i % tps);
+  i /= tps;
+  const int c = (int)(i % 3);
+  int64_t row = i / 3;
+  const int col = ((c * tps + tt) * p + py) * p + 2 * xp;
+  const int bw = W / (p * m), bh = H / (p * m);
+  int64_t r = row;
+  const int mx = (int)(r % m);
+  r /= m;
+  const int my = (int)(r % m);
+  r /= m;
+  const int bx = (int)(r % bw);
+  r /= bw;
+  const int by = (int)(r % bh);
+  const int t = (int)(r / bh);
+  const int f = min(t * tps + tt, T - 1);
+  const int y = (by * m + my) * p + py, x = (bx * m + mx) * p + 2 * xp;
+  const uint8_t* src = frames + (((int64_t)f * H + y) * W + x) * 3 + c;
+  const float v0 = lut[c * 256 + src[0]], v1 = lut[c * 256 + src[3]];
+  OUT* dst = out + row * ldo + col;
+  if constexpr (sizeof(OUT) == 2) {
+    bf16x2_t o;
+    o[0] = f2bf(v0);
+    o[1] = f2bf(v1);
+    *(bf16x2_t*)dst = o;
+  } else {
+    dst[0] = v0;
+    dst[1] = v1;
+  }
+}
+
 }  // namespace
+
+extern "C" int cs_qwen_patchify_u8(const void* frames, int32_t T, int32_t H, int32_t W, int32_t patch, int32_t merge,
+                                   int32_t temporal, const float* table, void* out, int64_t ldo, int32_t out_fp32,
+                                   void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!frames || !table || !out || T < 0 || H <= 0 || W <= 0 || patch <= 0 || patch % 2 || merge <= 0 || temporal <= 0)
+    return CS_ERR_INVALID_ARG;
+  if (H % (patch * merge) || W % (patch * merge)) return CS_ERR_INVALID_ARG;
+  const int64_t cols = (int64_t)3 * temporal * patch * patch;
+  if (ldo < cols || ldo % 2 || ((uintptr_t)out & (out_fp32 ? 7 : 3)) || ((uintptr_t)table & 3)) return CS_ERR_INVALID_ARG;
+  if (T == 0) return CS_OK;
+  const int64_t rows = (int64_t)((T + temporal - 1) / temporal) * (H / patch) * (W / patch);
+  const int64_t pairs = rows * cols / 2;
+  if ((pairs + 255) / 256 > 0x7fffffff) return CS_ERR_TOO_LARGE;
+  const dim3 grid((unsigned)((pairs + 255) / 256)), block(256);
+  if (out_fp32)
+    hipLaunchKernelGGL(qwen_patchify_u8_kernel<float>, grid, block, 0, stream, (const uint8_t*)frames, T, H, W, patch,
+                       merge, temporal, table, (float*)out, ldo, pairs);
+  else
+    hipLaunchKernelGGL(qwen_patchify_u8_kernel<bf16_t>, grid, block, 0, stream, (const uint8_t*)frames, T, H, W, patch,
+                       merge, temporal, table, (bf16_t*)out, ldo, pairs);
+  return cs_launch_status();
+}
 
 extern "C" int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_t H, int32_t W, int32_t patch,
                                 void* out, int64_t ldo, void* stream_) {

@@ -11,6 +11,7 @@ on torch's current stream:
     per block:  RMSNorm -> QKV GEMM(+bias) -> varlen MFMA attention with rotary fused into the q/k load
                 -> proj GEMM(+bias,+residual) -> RMSNorm -> gate|up GEMM(+bias, SiLU*mul)
                 -> down GEMM(+bias,+residual)                                :168-178
+                (by default the two RMSNorms are folded into the GEMMs around them: see `fold_norm`)
     merger:     RMSNorm -> GEMM(+bias, GELU) -> GEMM(+bias) with the inverse window permutation fused
                 as a row scatter of C                                        :225-233,:478-479
 
@@ -29,6 +30,7 @@ import torch
 import torch.nn as nn
 
 from cornserve_amd import ops
+from cornserve_amd.eric import frames as frame_ops
 from cornserve_amd.eric.api import Modality
 from cornserve_amd.eric.models.base import BaseModalityProcessor, EricModel
 
@@ -326,16 +328,51 @@ class Qwen2_5_VisionTransformer(EricModel):
         seqlens = (g[:, 0] * g[:, 1] * g[:, 2]) // unit
         return list(out.split([int(s) for s in seqlens], dim=0))
 
+    def patchify_frames(self, frames: list[torch.Tensor], arithmetic: str = "fused") -> tuple[torch.Tensor, np.ndarray]:
+        """uint8 frames of every item ([T,H,W,3] or [H,W,3], already at the processor's target size, on the host
+        or the device) -> (pixel_values [L, C*T*P*P] in the model dtype on the device, grid_thw int64 [n,3]): what
+        the Hugging Face processor the reference runs (:488-512) produces from the same frames, with rescale,
+        normalise and the patch layout done on the GPU."""
+        p, m, tps, dev = self.patch_size, self.spatial_merge_size, self.temporal_patch_size, self.device
+        key = ("byte_table", arithmetic)
+        pk = self._ensure_packed()
+        if key not in pk:
+            pk[key] = frame_ops.byte_table(arithmetic=arithmetic).to(dev)
+        items, grids = [], []
+        for f in frames:
+            f = torch.as_tensor(f)
+            if f.dim() == 3:
+                f = f[None]
+            if f.dtype != torch.uint8 or f.dim() != 4 or f.shape[-1] != 3:
+                raise ValueError("frames must be uint8 [T,H,W,3] or [H,W,3] (RGB)")
+            T, H, W, _ = f.shape
+            if H % (p * m) or W % (p * m) or T < 1:
+                raise ValueError(f"frame size {H}x{W} is not a multiple of {p * m}: resize first (frames.resize_frames)")
+            items.append(f.contiguous().to(dev, non_blocking=True))
+            grids.append((-(-T // tps), H // p, W // p))
+        grid = np.asarray(grids, dtype=np.int64).reshape(-1, 3)
+        L = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
+        px = torch.empty((L, self.in_channels * tps * p * p), dtype=self.dtype, device=dev)
+        row = 0
+        for f, (gt, gh, gw) in zip(items, grids):
+            ops.qwen_patchify_u8(f, pk[key], p, m, tps, out=px[row : row + gt * gh * gw])
+            row += gt * gh * gw
+        return px, grid
+
     @torch.inference_mode()
     def forward(self, modality: Modality, adapter_name: str, batch: dict[str, list[torch.Tensor]]) -> list[torch.Tensor]:
         """See the reference docstring (:402-413): `pixel_values` + `image_grid_thw` for images,
-        `pixel_values_videos` + `video_grid_thw` for videos."""
+        `pixel_values_videos` + `video_grid_thw` for videos.  In addition to the reference's format, a batch
+        may carry `pixel_frames` / `pixel_frames_videos` instead: one uint8 [T,H,W,3] tensor of resized frames
+        per item (see `FrameModalityProcessor`); the grids follow from the shapes."""
         if modality == Modality.IMAGE:
-            px_key, grid_key = "pixel_values", "image_grid_thw"
+            px_key, grid_key, frame_key = "pixel_values", "image_grid_thw", "pixel_frames"
         elif modality == Modality.VIDEO:
-            px_key, grid_key = "pixel_values_videos", "video_grid_thw"
+            px_key, grid_key, frame_key = "pixel_values_videos", "video_grid_thw", "pixel_frames_videos"
         else:
             raise ValueError(f"Unsupported modality: {modality}")
+        if frame_key in batch:
+            return self.forward_device(*self.patchify_frames(batch[frame_key]))
         pixel_values = torch.cat(batch[px_key], dim=0).to(device=self.device, dtype=self.dtype)
         grid = torch.cat([g.reshape(-1, 3) for g in batch[grid_key]], dim=0).cpu().numpy().astype(np.int64)
         return self.forward_device(pixel_values, grid)
@@ -362,3 +399,22 @@ class ModalityProcessor(BaseModalityProcessor):
             return self.hf_processor(images=None, videos=[video], return_tensors="pt").data
 
         return processor
+
+
+class FrameModalityProcessor(BaseModalityProcessor):
+    """Processor for the uint8-frame input format: resizes only (the Hugging Face processor's target size and
+    PIL bicubic resampling) and emits `pixel_frames` / `pixel_frames_videos`; rescale, normalise and the patch
+    layout run on the GPU inside the model's forward.  Needs no model files."""
+
+    def __init__(self, model_id: str, min_pixels: int = 56 * 56, max_pixels: int = 14 * 14 * 4 * 1280) -> None:
+        super().__init__(model_id=model_id)
+        self.min_pixels, self.max_pixels = min_pixels, max_pixels
+
+    def _resized(self, frames) -> torch.Tensor:
+        return torch.from_numpy(frame_ops.resize_frames(frames, 28, self.min_pixels, self.max_pixels))
+
+    def get_image_processor(self) -> Callable | None:
+        return lambda image: {"pixel_frames": self._resized(image)}
+
+    def get_video_processor(self) -> Callable | None:
+        return lambda video: {"pixel_frames_videos": self._resized(video)}

@@ -79,6 +79,8 @@ _SIGNATURES: dict[str, list] = {
     ],
     "cs_attn_block_q": [c_int32],
     "cs_attn_work_host": [c_void_p, c_int32, c_int32, c_void_p, c_int32, POINTER(c_int32)],
+    "cs_qwen_patchify_u8": [c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64,
+                            c_int32, c_void_p],
     "cs_patchify_nchw": [c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_int64, c_void_p],
     "cs_avgpool_gemma_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_float, c_void_p],
     "cs_cast_f32_bf16": [c_void_p, c_void_p, c_int64, c_void_p],

@@ -337,6 +337,32 @@ def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPla
 
 
 # ------------------------------------------------------------------------------------------ SigLIP
+def qwen_patchify_u8(frames: torch.Tensor, table: torch.Tensor, patch: int, merge: int, temporal: int, *,
+                     out: torch.Tensor | None = None, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+    """uint8 frames [T,H,W,3] -> normalised patch rows [ceil(T/temporal)*(H/patch)*(W/patch), 3*temporal*patch^2]
+    in the Qwen2-VL processor's layout; `table` is the fp32 [3,256] byte table.  `out` may be a row slice of a
+    larger buffer."""
+    lib = _l.load()
+    _req(frames, torch.uint8, "frames")
+    _req(table, torch.float32, "table")
+    if frames.dim() != 4 or frames.shape[-1] != 3 or not frames.is_contiguous():
+        raise ValueError("frames must be contiguous uint8 [T,H,W,3]")
+    if tuple(table.shape) != (3, 256) or not table.is_contiguous():
+        raise ValueError("table must be contiguous fp32 [3,256]")
+    T, H, W, _ = frames.shape
+    if H % (patch * merge) or W % (patch * merge):
+        raise ValueError(f"frame size {H}x{W} is not a multiple of patch*merge = {patch * merge}")
+    rows, cols = -(-T // temporal) * (H // patch) * (W // patch), 3 * temporal * patch * patch
+    if out is None:
+        out = torch.empty((rows, cols), dtype=dtype, device=frames.device)
+    elif out.dtype not in (torch.bfloat16, torch.float32) or tuple(out.shape) != (rows, cols) or out.stride(1) != 1:
+        raise ValueError(f"out must be bf16 or fp32 [{rows},{cols}]")
+    _l.check(lib.cs_qwen_patchify_u8(frames.data_ptr(), T, H, W, patch, merge, temporal, table.data_ptr(),
+                                     out.data_ptr(), out.stride(0), int(out.dtype == torch.float32), _stream()),
+             "cs_qwen_patchify_u8")
+    return out
+
+
 def patchify_nchw(pixels: torch.Tensor, patch: int, ldo: int) -> torch.Tensor:
     """[B,C,H,W] bf16 -> [B*(H/p)*(W/p), ldo] rows of (c,ky,kx)-ordered patch values, zero padded."""
     lib = _l.load()

@@ -181,6 +181,18 @@ int cs_attn_work_host(const int32_t* cu_seqlens_host, int32_t n_seg, int32_t blo
  * ordered (c, ky, kx) and zero padding up to ldo.                                                 */
 int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_t H, int32_t W, int32_t patch,
                      void* out, int64_t ldo, void* stream);
+/* The step before the Qwen2.5-VL encoder, for callers that hand over resized uint8 frames instead of float
+ * pixel_values (the reference runs the Hugging Face image processor on the CPU: ModalityProcessor,
+ * qwen2_5_vl.py:488-512, called from router/processor.py:46-131, and ships 1176 floats per patch).
+ * frames: uint8 [T,H,W,3] on the device, H and W multiples of patch*merge (the processor's resize is the caller's).
+ * table:  fp32 [3][256] on the device: the processor's rescale + normalise applied to every byte value per
+ *         channel, computed by the caller in the processor's own arithmetic.
+ * out:    bf16 (or fp32 if out_fp32) [ceil(T/temporal)*(H/patch)*(W/patch), ldo], the processor's layout:
+ *         rows (t, block row, block col, row in block, col in block) with merge x merge blocks, columns
+ *         (channel, temporal, y, x); temporal slot tt of row group t shows frame min(t*temporal+tt, T-1).   */
+int cs_qwen_patchify_u8(const void* frames, int32_t T, int32_t H, int32_t W, int32_t patch, int32_t merge,
+                        int32_t temporal, const float* table, void* out, int64_t ldo, int32_t out_fp32,
+                        void* stream);
 /* Gemma3MultiModalProjector front half, gemma3.py:36-46: AvgPool2d(k) over the side x side token grid
  * followed by GemmaRMSNorm.  x: bf16 [B, side*side, H] -> y: bf16 [B, (side/k)^2, H].             */
 int cs_avgpool_gemma_rmsnorm(const void* x, const void* w, void* y, int32_t B, int32_t side, int32_t k,

@@ -84,6 +84,32 @@ def test_qwen_without_folded_norms(dev, golden_dir):
     check(out_f, out, REL_BF16, "folded vs unfolded")
 
 
+def test_qwen_uint8_frames_equal_float_pixel_values(dev):
+    """The uint8-frame input format gives bit-identical embeddings to the reference's format fed with what the
+    image processor makes of the same frames (oracle restatement of the processor)."""
+    from oracle import qwen_preprocess as qp
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=7)
+    rng = np.random.default_rng(7)
+    images = [rng.integers(0, 256, (1, h, w, 3), dtype=np.uint8) for h, w in [(56, 84), (224, 112), (28, 28)]]
+    table = qp.normalization_table(arithmetic="fused")
+    px = [torch.from_numpy(qp.patchify_frames(f, table)[0]) for f in images]
+    grids = [torch.tensor([[1, f.shape[1] // 14, f.shape[2] // 14]]) for f in images]
+    ref = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grids})
+    got = model(Modality.IMAGE, "", {"pixel_frames": [torch.from_numpy(f) for f in images]})
+    assert len(got) == 3 and all(torch.equal(a, b) for a, b in zip(got, ref))
+    got = model(Modality.IMAGE, "", {"pixel_frames": [torch.from_numpy(f[0]).to(dev) for f in images]})   # [H,W,3], on the device
+    assert all(torch.equal(a, b) for a, b in zip(got, ref))
+    video = rng.integers(0, 256, (5, 56, 112, 3), dtype=np.uint8)
+    vpx, vgrid = qp.patchify_frames(video, table)
+    assert vgrid == (3, 4, 8)
+    ref = model(Modality.VIDEO, "", {"pixel_values_videos": [torch.from_numpy(vpx)], "video_grid_thw": [torch.tensor([vgrid])]})
+    got = model(Modality.VIDEO, "", {"pixel_frames_videos": [torch.from_numpy(video)]})
+    assert torch.equal(got[0], ref[0]) and got[0].shape == (3 * 4 * 8 // 4, 3584)
+    with pytest.raises(ValueError):
+        model(Modality.IMAGE, "", {"pixel_frames": [torch.zeros((1, 30, 28, 3), dtype=torch.uint8)]})
+
+
 def test_qwen_multi_image_ragged_and_video(dev):
     """Ragged image grids (window padding at non-multiple-of-8 edges) and a video (per-frame segments)."""
     model, sd, ocfg = build_qwen(dev, 3, (1,), seed=2)

@@ -94,6 +94,30 @@ def test_patchify_bit_exact(ops, dev):
 
 
 # ------------------------------------------------------------------------------------------- norms
+@pytest.mark.parametrize("t,h,w,patch,merge,temporal", [
+    (1, 448, 448, 14, 2, 2),    # one image of the benchmark's size
+    (1, 28, 1344, 14, 2, 2),    # one block row
+    (8, 336, 588, 14, 2, 2),    # config-5 style video
+    (5, 56, 84, 14, 2, 2),      # odd frame count: the last frame fills the last group
+    (7, 24, 36, 2, 3, 3),       # other patch / merge / temporal sizes
+])
+def test_qwen_patchify_u8_bit_exact(ops, dev, t, h, w, patch, merge, temporal):
+    from cornserve_amd.eric import frames as fr
+    from oracle import qwen_preprocess as qp
+
+    frames = np.random.default_rng(t * 1000 + h + w).integers(0, 256, (t, h, w, 3), dtype=np.uint8)
+    for arithmetic in ("fused", "numpy"):
+        table = fr.byte_table(arithmetic=arithmetic)
+        ref, grid = qp.patchify_frames(frames, qp.normalization_table(arithmetic=arithmetic), patch, merge, temporal)
+        got32 = ops.qwen_patchify_u8(torch.from_numpy(frames).to(dev), table.to(dev), patch, merge, temporal, dtype=torch.float32)
+        assert got32.shape == ref.shape == (grid[0] * grid[1] * grid[2], 3 * temporal * patch * patch)
+        assert np.array_equal(got32.cpu().numpy(), ref)
+        got16 = ops.qwen_patchify_u8(torch.from_numpy(frames).to(dev), table.to(dev), patch, merge, temporal)
+        assert torch.equal(got16.cpu(), torch.from_numpy(ref).bfloat16())   # the reference's .to(dtype), :415-419
+    with pytest.raises(ValueError):
+        ops.qwen_patchify_u8(torch.zeros((1, 30, 28, 3), dtype=torch.uint8, device=dev), table.to(dev), 14, 2, 2)
+
+
 @pytest.mark.parametrize("rows,H", [(1, 1280), (1023, 1280), (64, 1152), (5, 64), (7, 5120)])
 def test_rmsnorm(ops, dev, rows, H):
     x = rnd((rows, H), 2.0, 1, dev)

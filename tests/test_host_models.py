@@ -82,3 +82,35 @@ def test_gemma3_names_adapters_and_errors():
 
 def test_modality_is_a_str_enum():
     assert Modality.IMAGE == "image" and str(Modality.VIDEO) == "video" and Modality("audio") is Modality.AUDIO
+
+
+# ------------------------------------------------------------------ uint8-frame input format (host side)
+def test_frame_processor_resize_and_table_match_the_hf_pil_processor():
+    """FrameModalityProcessor's resize + the byte table + the oracle's layout reproduce the Hugging Face PIL
+    processor's pixel_values bit for bit on images that DO need resampling."""
+    import numpy as np
+    pytest.importorskip("PIL")
+    mod = pytest.importorskip("transformers.models.qwen2_vl.image_processing_pil_qwen2_vl")
+    from cornserve_amd.eric import frames as fr
+    from cornserve_amd.eric.api import Modality
+    from cornserve_amd.eric.models.qwen2_5_vl import FrameModalityProcessor
+    from oracle import qwen_preprocess as qp
+
+    hf = mod.Qwen2VLImageProcessorPil()
+    proc = FrameModalityProcessor("unused")
+    rng = np.random.default_rng(5)
+    for h, w in [(50, 70), (33, 200), (448, 448), (301, 517)]:
+        img = rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+        ref = hf(images=[img], return_tensors="np")
+        out = proc.process(Modality.IMAGE, img)["pixel_frames"]
+        assert out.dtype == torch.uint8 and out.shape[0] == 1 and out.shape[3] == 3
+        assert tuple(out.shape[1:3]) == fr.target_size(h, w) == qp.smart_resize(h, w)
+        table = fr.byte_table(arithmetic="numpy").numpy()
+        assert np.array_equal(table, qp.normalization_table(arithmetic="numpy"))
+        px, grid = qp.patchify_frames(out.numpy(), table)
+        assert grid == tuple(ref["image_grid_thw"][0]) and np.array_equal(px, ref["pixel_values"])
+    assert np.array_equal(fr.byte_table(arithmetic="fused").numpy(), qp.normalization_table(arithmetic="fused"))
+    with pytest.raises(ValueError):
+        fr.resize_frames(np.zeros((4, 4), np.uint8))
+    with pytest.raises(ValueError):
+        fr.target_size(1, 500)

@@ -1,0 +1,103 @@
+"""Pins oracle/qwen_preprocess.py (the step before the encoder: resized uint8 frames -> flat pixel_values)."""
+
+import itertools
+
+import numpy as np
+import pytest
+
+from oracle import qwen_preprocess as qp
+
+
+def _rand_frames(t, h, w, seed):
+    return np.random.default_rng(seed).integers(0, 256, (t, h, w, 3), dtype=np.uint8)
+
+
+def _hf_pil_processor():
+    mod = pytest.importorskip("transformers.models.qwen2_vl.image_processing_pil_qwen2_vl")
+    pytest.importorskip("PIL")
+    return mod.Qwen2VLImageProcessorPil()
+
+
+@pytest.mark.parametrize("h,w", [(56, 84), (448, 448), (28, 140), (252, 1344)])
+def test_numpy_arithmetic_and_layout_match_the_package_bit_for_bit(h, w):
+    """Sizes that are multiples of 28 inside the pixel budget: the processor's resize keeps every pixel."""
+    proc = _hf_pil_processor()
+    img = _rand_frames(1, h, w, seed=h * 7 + w)[0]
+    out = proc(images=[img], return_tensors="np")
+    got, grid = qp.patchify_frames(img[None], qp.normalization_table(arithmetic="numpy"))
+    assert tuple(out["image_grid_thw"][0]) == grid == (1, h // 14, w // 14)
+    assert out["pixel_values"].dtype == np.float32
+    assert np.array_equal(out["pixel_values"], got)
+
+
+def test_smart_resize_matches_the_package():
+    mod = pytest.importorskip("transformers.models.qwen2_vl.image_processing_pil_qwen2_vl")
+    rng = np.random.default_rng(0)
+    cases = [(1, 1), (27, 29), (28, 28), (5000, 4000), (100, 19000), (3, 600), (1344, 1344), (10000, 10000)]
+    cases += [tuple(int(v) for v in rng.integers(1, 6000, 2)) for _ in range(300)]
+    for h, w in cases:
+        if max(h, w) / min(h, w) > 200:
+            with pytest.raises(ValueError):
+                qp.smart_resize(h, w)
+            continue
+        assert qp.smart_resize(h, w) == mod.smart_resize(h, w)
+        assert qp.smart_resize(h, w, 28, 3136, 12845056) == mod.smart_resize(h, w, 28, 3136, 12845056)
+    hb, wb = qp.smart_resize(5000, 4000)
+    assert hb % 28 == 0 and wb % 28 == 0 and hb * wb <= 14 * 14 * 4 * 1280
+
+
+def test_tables():
+    a, b = qp.normalization_table(arithmetic="numpy"), qp.normalization_table(arithmetic="fused")
+    assert a.shape == b.shape == (3, 256) and a.dtype == b.dtype == np.float32
+    # worked values: byte 0 and byte 255 of the red channel
+    assert a[0, 0] == np.float32(-0.48145466) / np.float32(0.26862954)
+    assert a[0, 255] == (np.float32(1.0) - np.float32(0.48145466)) / np.float32(0.26862954)
+    assert np.all(np.diff(a, axis=1) > 0) and np.all(np.diff(b, axis=1) > 0)          # monotone in the byte value
+    # the two arithmetic sequences agree to 2 units in the last place of the largest values ...
+    assert np.all(np.abs(a - b) <= 2 * np.spacing(np.float32(2.0)))
+    # ... so after the encoder's cast to bfloat16 they agree for (nearly) all byte values
+    import torch
+    ta, tb = torch.from_numpy(a).bfloat16(), torch.from_numpy(b).bfloat16()
+    assert (ta != tb).sum().item() <= 3
+
+
+def _brute_force(frames, table, patch, merge, temporal):
+    """Every output element from its definition, with plain index arithmetic (no reshape / transpose)."""
+    T, H, W, _ = frames.shape
+    gt, gh, gw = -(-T // temporal), H // patch, W // patch
+    out = np.zeros((gt * gh * gw, 3 * temporal * patch * patch), np.float32)
+    for t, by, bx, my, mx in itertools.product(range(gt), range(gh // merge), range(gw // merge), range(merge), range(merge)):
+        row = (((t * (gh // merge) + by) * (gw // merge) + bx) * merge + my) * merge + mx
+        for c, tt, py, px in itertools.product(range(3), range(temporal), range(patch), range(patch)):
+            f = min(t * temporal + tt, T - 1)
+            y, x = (by * merge + my) * patch + py, (bx * merge + mx) * patch + px
+            out[row, ((c * temporal + tt) * patch + py) * patch + px] = table[c, frames[f, y, x, c]]
+    return out
+
+
+@pytest.mark.parametrize("t,h,w,patch,merge,temporal", [(1, 8, 12, 2, 2, 2), (3, 8, 4, 2, 2, 2), (4, 12, 12, 2, 3, 2),
+                                                        (5, 4, 8, 2, 2, 3), (2, 28, 56, 14, 2, 2)])
+def test_layout_against_brute_force(t, h, w, patch, merge, temporal):
+    frames = _rand_frames(t, h, w, seed=t + h + w)
+    table = qp.normalization_table()
+    got, grid = qp.patchify_frames(frames, table, patch, merge, temporal)
+    assert grid == (-(-t // temporal), h // patch, w // patch)
+    assert np.array_equal(got, _brute_force(frames, table, patch, merge, temporal))
+
+
+def test_video_of_repeated_frames_is_the_image():
+    img = _rand_frames(1, 56, 84, seed=9)
+    table = qp.normalization_table()
+    one, _ = qp.patchify_frames(img, table)
+    vid, grid = qp.patchify_frames(np.repeat(img, 4, axis=0), table)
+    assert grid == (2, 4, 6)
+    assert np.array_equal(vid[:24], one) and np.array_equal(vid[24:], one)
+    odd, grid = qp.patchify_frames(np.repeat(img, 3, axis=0), table)   # 3 frames: the last one is repeated
+    assert grid == (2, 4, 6) and np.array_equal(odd, vid)
+
+
+def test_rejects_bad_input():
+    with pytest.raises(ValueError):
+        qp.patchify_frames(np.zeros((1, 30, 28, 3), np.uint8), qp.normalization_table())
+    with pytest.raises(ValueError):
+        qp.patchify_frames(np.zeros((1, 28, 28, 3), np.float32), qp.normalization_table())
