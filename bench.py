@@ -12,9 +12,12 @@ with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
                         ranges): algorithmic FLOPs per call / average duration of the call's launches, measured
                         with HIP events on the launch stream inside the timed region, against the bf16 dense
                         MFMA peak
-  breakdown             per-stage device time from a separately instrumented pass, and the MFMA fraction
-                        over GEMM+attention time (the target the build is held to)
+  breakdown             per-stage device time from a separately instrumented pass (an event between stages,
+                        which makes that pass a little longer than a timed step), and the MFMA fraction over
+                        GEMM+attention time (the target the build is held to) = the GEMM+attention share of
+                        the instrumented pass applied to the timed step
   host_inputs           the same step with the batch handed over as fp32 host tensors (PCIe-inclusive)
+  host_inputs_uint8_frames  the same step from resized uint8 frames on the host (PCIe-inclusive; GPU patch layout)
   cpu_baseline          the CPU oracle (a port of the reference's algorithm, plain PyTorch) timed on this
                         host's cores on a bounded sample of the same workload
 """
@@ -36,9 +39,9 @@ if str(ROOT) not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak (2.5 PFLOP/s, the published figure at 2.4 GHz)
 N_IMAGES = 8
 # HBM-side bytes per gate|up call (its two launches together), measured with rocprofv3 --pmc (not live):
-# FETCH_SIZE 92,378 + 18,044 KiB scaled by 2.00 (what the same counter reads for a plain 1 GiB copy) +
+# FETCH_SIZE 93,167 + 18,180 KiB scaled by 2.00 (what the same counter reads for a plain 1 GiB copy) +
 # WRITE_SIZE 49,152 + 6,144 KiB scaled by 1.00.
-GATE_UP_HBM_BYTES_PER_LAUNCH = int(((92378 + 18044) * 2.00 + (49152 + 6144) * 1.00) * 1024)
+GATE_UP_HBM_BYTES_PER_LAUNCH = int(((93167 + 18180) * 2.00 + (49152 + 6144) * 1.00) * 1024)
 GRID = (1, 32, 32)          # 448 x 448, patch 14
 
 
@@ -181,10 +184,24 @@ def main() -> None:
             model.forward(Modality.IMAGE, "", host_batch)
         torch.cuda.synchronize()
         host_ms = (time.perf_counter() - t0) / 5 * 1e3
+        # the same batch as resized uint8 frames (8x fewer bytes over PCIe; rescale, normalise and the patch
+        # layout run on the GPU): random bytes, so the embeddings differ from the float batch above
+        frames = [torch.randint(0, 256, (1, GRID[1] * 14, GRID[2] * 14, 3), dtype=torch.uint8) for _ in range(N_IMAGES)]
+        frame_batch = {"pixel_frames": frames}
+        model.forward(Modality.IMAGE, "", frame_batch)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            model.forward(Modality.IMAGE, "", frame_batch)
+        torch.cuda.synchronize()
+        frames_ms = (time.perf_counter() - t0) / 5 * 1e3
     stage_ms = {k: sum(v) / 3 for k, v in full.durations_ms().items()}
     mfma_keys = [k for k in stage_ms if k.startswith("gemm_") or k.startswith("attn_") or k == "patch_embed"]
-    mfma_ms = sum(stage_ms[k] for k in mfma_keys)
+    # The instrumented pass records an event between stages, which costs a little device time per mark: its
+    # stage SHARES are applied to the timed step (whose duration has no such overhead).
+    mfma_share = sum(stage_ms[k] for k in mfma_keys) / sum(stage_ms.values())
     ms_per_step = dt / args.steps * 1e3
+    mfma_ms = ms_per_step * mfma_share
     achieved = flops["gemm_gate_up"] / (gu_ms * 1e-3) / 1e12
 
     result = {
@@ -214,6 +231,7 @@ def main() -> None:
         },
         "breakdown": {
             "stage_ms_per_step": {k: round(v, 4) for k, v in sorted(stage_ms.items())},
+            "instrumented_pass_ms": sum(stage_ms.values()),
             "gemm_attention_ms": mfma_ms,
             "algorithmic_tflop_per_step": flops["total"] / 1e12,
             "mfma_frac_over_gemm_attention_time": flops["total"] / (mfma_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
@@ -223,6 +241,11 @@ def main() -> None:
     result["host_inputs"] = {
         "ms_per_step": host_ms, "patches_per_s": L / (host_ms * 1e-3),
         "note": "same batch handed over as pageable fp32 host tensors (PCIe copy + cast inside the call)",
+    }
+    result["host_inputs_uint8_frames"] = {
+        "ms_per_step": frames_ms, "patches_per_s": L / (frames_ms * 1e-3),
+        "note": "same shapes handed over as pageable uint8 host frames [1,448,448,3] (PCIe copy, then rescale + "
+                "normalise + patch layout on the GPU inside the call)",
     }
     if args.calibrate_copy:
         src = torch.zeros(256 * 1024 * 1024, dtype=torch.int32, device=dev)  # 1 GiB read + 1 GiB written per copy
