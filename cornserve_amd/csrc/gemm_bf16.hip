@@ -221,6 +221,7 @@ int dispatch_epi(const CsGemmArgs& a, hipStream_t s) {
     case CS_EPI_SWIGLU: return launch<BM, BN, CS_EPI_SWIGLU, W_FP8>(a, s);
     case CS_EPI_GELU_ERF: return launch<BM, BN, CS_EPI_GELU_ERF, W_FP8>(a, s);
     case CS_EPI_GELU_TANH: return launch<BM, BN, CS_EPI_GELU_TANH, W_FP8>(a, s);
+    case CS_EPI_QUICK_GELU: return launch<BM, BN, CS_EPI_QUICK_GELU, W_FP8>(a, s);
     default: return CS_ERR_INVALID_ARG;
   }
 }

@@ -21,6 +21,8 @@ CS_DEVICE float gelu_tanh(float x) {
   const float u = k0 * (x + k1 * x * x * x);
   return x * __builtin_amdgcn_rcpf(1.0f + __expf(-2.0f * u));
 }
+// x * sigmoid(1.702 x)
+CS_DEVICE float quick_gelu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-1.702f * x)); }
 // x * sigmoid(x) with the hardware reciprocal (1 ulp) instead of an IEEE division sequence.
 CS_DEVICE float silu(float x) { return x * __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
 
@@ -73,6 +75,9 @@ CS_DEVICE void epilogue(const CsGemmArgs& p, const f32x16_t (&acc)[MT][NT], int 
           } else if (EPI == CS_EPI_GELU_TANH) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) v[q] = gelu_tanh(rbf(v[q]));
+          } else if (EPI == CS_EPI_QUICK_GELU) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = quick_gelu(rbf(v[q]));
           } else if (EPI == CS_EPI_RESIDUAL) {
             const bf16x4_t r = *(const bf16x4_t*)(pRes + (int64_t)m * p.ldr + n);
 #pragma unroll

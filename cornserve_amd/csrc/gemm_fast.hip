@@ -532,6 +532,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
             } else if (EPI == CS_EPI_GELU_TANH) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(rbf(v[r]));
+            } else if (EPI == CS_EPI_QUICK_GELU) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) v[r] = quick_gelu(rbf(v[r]));
             } else if (ADDEND) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] = rbf(v[r]) + bf2f(addend[ADDEND ? i : 0][ADDEND ? j : 0][r]);
@@ -659,6 +662,7 @@ int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
       if constexpr (W_FP8 && BN == 160) return CS_ERR_UNSUPPORTED;  // never dispatched, see cs_gemm_fast
       else return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_ERF, W_FP8>(a, s);
     case CS_EPI_GELU_TANH: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_TANH, W_FP8>(a, s);
+    case CS_EPI_QUICK_GELU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_QUICK_GELU, W_FP8>(a, s);
     default: return CS_ERR_INVALID_ARG;
   }
 }

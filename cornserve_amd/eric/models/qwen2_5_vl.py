@@ -110,7 +110,108 @@ def quantize_fp8_rows(w: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     return q, scale.contiguous()
 
 
-class Qwen2_5_VisionTransformer(EricModel):
+class QwenVisionBase(EricModel):
+    """What the Qwen2-VL family encoders share: parameter placement, lazy repacking of the weights into their
+    device form, the batch formats of `forward` and the uint8-frame input path.  Subclasses provide `_pack`,
+    `forward_device`, `chunk_shape` and the attributes patch_size, temporal_patch_size, spatial_merge_size,
+    in_channels, weight_format and patch_embed."""
+
+    def __init__(self) -> None:
+        super().__init__()
+        self._packed: dict | None = None
+        self.register_load_state_dict_post_hook(lambda module, incompatible: module._invalidate())
+
+    # ------------------------------------------------------------------ EricModel properties
+    @property
+    def dtype(self) -> torch.dtype:
+        return self.patch_embed.proj.weight.dtype
+
+    @property
+    def device(self) -> torch.device:
+        return self.patch_embed.proj.weight.device
+
+    # ------------------------------------------------------------------ weight repacking
+    def _invalidate(self) -> None:
+        self._packed = None
+
+    def _apply(self, fn, recurse=True):  # .to()/.cuda()/.bfloat16() move the parameters: repack lazily
+        self._packed = None
+        return super()._apply(fn, recurse)
+
+    def _lin(self, w: torch.Tensor, b: torch.Tensor | None) -> dict:
+        """Device form of one linear layer: bf16 [N,K] or fp8 [N,K] + fp32 scale [N]."""
+        w = w.contiguous()
+        if self.weight_format == "fp8_e4m3":
+            q, s = quantize_fp8_rows(w)
+            return {"w": q.contiguous(), "s": s, "b": b}
+        return {"w": w, "s": None, "b": b}
+
+    def _ensure_packed(self) -> dict:
+        if self._packed is None:
+            if self.dtype != torch.bfloat16 or self.device.type != "cuda":
+                raise RuntimeError(
+                    "the gfx950 kernels need the model in bfloat16 on a GPU "
+                    f"(got {self.dtype} on {self.device}); there is no CPU path"
+                )
+            self._packed = self._pack()
+        return self._packed
+
+    # ------------------------------------------------------------------ forward
+    @staticmethod
+    def _g(a: torch.Tensor, lin: dict, **kw) -> torch.Tensor:
+        return ops.gemm(a, lin["w"], lin["b"], w_scale=lin["s"], **kw)
+
+    def patchify_frames(self, frames: list[torch.Tensor], arithmetic: str = "fused") -> tuple[torch.Tensor, np.ndarray]:
+        """uint8 frames of every item ([T,H,W,3] or [H,W,3], already at the processor's target size, on the host
+        or the device) -> (pixel_values [L, C*T*P*P] in the model dtype on the device, grid_thw int64 [n,3]): what
+        the Hugging Face processor the reference runs (:488-512) produces from the same frames, with rescale,
+        normalise and the patch layout done on the GPU."""
+        p, m, tps, dev = self.patch_size, self.spatial_merge_size, self.temporal_patch_size, self.device
+        key = ("byte_table", arithmetic)
+        pk = self._ensure_packed()
+        if key not in pk:
+            pk[key] = frame_ops.byte_table(arithmetic=arithmetic).to(dev)
+        items, grids = [], []
+        for f in frames:
+            f = torch.as_tensor(f)
+            if f.dim() == 3:
+                f = f[None]
+            if f.dtype != torch.uint8 or f.dim() != 4 or f.shape[-1] != 3:
+                raise ValueError("frames must be uint8 [T,H,W,3] or [H,W,3] (RGB)")
+            T, H, W, _ = f.shape
+            if H % (p * m) or W % (p * m) or T < 1:
+                raise ValueError(f"frame size {H}x{W} is not a multiple of {p * m}: resize first (frames.resize_frames)")
+            items.append(f.contiguous().to(dev, non_blocking=True))
+            grids.append((-(-T // tps), H // p, W // p))
+        grid = np.asarray(grids, dtype=np.int64).reshape(-1, 3)
+        L = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
+        px = torch.empty((L, self.in_channels * tps * p * p), dtype=self.dtype, device=dev)
+        row = 0
+        for f, (gt, gh, gw) in zip(items, grids):
+            ops.qwen_patchify_u8(f, pk[key], p, m, tps, out=px[row : row + gt * gh * gw])
+            row += gt * gh * gw
+        return px, grid
+
+    @torch.inference_mode()
+    def forward(self, modality: Modality, adapter_name: str, batch: dict[str, list[torch.Tensor]]) -> list[torch.Tensor]:
+        """See the reference docstring (:402-413): `pixel_values` + `image_grid_thw` for images,
+        `pixel_values_videos` + `video_grid_thw` for videos.  In addition to the reference's format, a batch
+        may carry `pixel_frames` / `pixel_frames_videos` instead: one uint8 [T,H,W,3] tensor of resized frames
+        per item (see `FrameModalityProcessor`); the grids follow from the shapes."""
+        if modality == Modality.IMAGE:
+            px_key, grid_key, frame_key = "pixel_values", "image_grid_thw", "pixel_frames"
+        elif modality == Modality.VIDEO:
+            px_key, grid_key, frame_key = "pixel_values_videos", "video_grid_thw", "pixel_frames_videos"
+        else:
+            raise ValueError(f"Unsupported modality: {modality}")
+        if frame_key in batch:
+            return self.forward_device(*self.patchify_frames(batch[frame_key]))
+        pixel_values = torch.cat(batch[px_key], dim=0).to(device=self.device, dtype=self.dtype)
+        grid = torch.cat([g.reshape(-1, 3) for g in batch[grid_key]], dim=0).cpu().numpy().astype(np.int64)
+        return self.forward_device(pixel_values, grid)
+
+
+class Qwen2_5_VisionTransformer(QwenVisionBase):
     def __init__(self, config: Any, weight_format: str = "bf16", fold_norm: bool = True) -> None:
         """`fold_norm`: apply norm1 / norm2 of every block inside the GEMM that follows them (the norm weight is
         folded into that GEMM's weight columns at pack time, the per-row rsqrt is applied to the fp32
@@ -144,38 +245,13 @@ class Qwen2_5_VisionTransformer(EricModel):
         self.patch_embed = _PatchEmbed(self.in_channels, self.hidden_size, self.temporal_patch_size, self.patch_size)
         self.blocks = nn.ModuleList([_Block(self.hidden_size, self.intermediate_size) for _ in range(vc.depth)])
         self.merger = _Merger(self.out_hidden_size, self.hidden_size, self.spatial_merge_size)
-        self._packed: dict | None = None
-        self.register_load_state_dict_post_hook(lambda module, incompatible: module._invalidate())
 
     # ------------------------------------------------------------------ EricModel properties
-    @property
-    def dtype(self) -> torch.dtype:
-        return self.patch_embed.proj.weight.dtype
-
-    @property
-    def device(self) -> torch.device:
-        return self.patch_embed.proj.weight.device
-
     @property
     def chunk_shape(self) -> tuple[int, ...]:
         return (1, self.out_hidden_size)
 
     # ------------------------------------------------------------------ weight repacking
-    def _invalidate(self) -> None:
-        self._packed = None
-
-    def _apply(self, fn, recurse=True):  # .to()/.cuda()/.bfloat16() move the parameters: repack lazily
-        self._packed = None
-        return super()._apply(fn, recurse)
-
-    def _lin(self, w: torch.Tensor, b: torch.Tensor | None) -> dict:
-        """Device form of one linear layer: bf16 [N,K] or fp8 [N,K] + fp32 scale [N]."""
-        w = w.contiguous()
-        if self.weight_format == "fp8_e4m3":
-            q, s = quantize_fp8_rows(w)
-            return {"w": q.contiguous(), "s": s, "b": b}
-        return {"w": w, "s": None, "b": b}
-
     @torch.no_grad()
     def _pack(self) -> dict:
         dev, H, I = self.device, self.hidden_size, self.intermediate_size
@@ -215,21 +291,7 @@ class Qwen2_5_VisionTransformer(EricModel):
         pk["inv_freq"] = inv_freq.to(dev)
         return pk
 
-    def _ensure_packed(self) -> dict:
-        if self._packed is None:
-            if self.dtype != torch.bfloat16 or self.device.type != "cuda":
-                raise RuntimeError(
-                    "the gfx950 kernels need the model in bfloat16 on a GPU "
-                    f"(got {self.dtype} on {self.device}); there is no CPU path"
-                )
-            self._packed = self._pack()
-        return self._packed
-
     # ------------------------------------------------------------------ forward
-    @staticmethod
-    def _g(a: torch.Tensor, lin: dict, **kw) -> torch.Tensor:
-        return ops.gemm(a, lin["w"], lin["b"], w_scale=lin["s"], **kw)
-
     def get_window_index(self, grid_thw) -> tuple[torch.Tensor, list[int]]:
         """Same results as the reference method (:357-386) followed by unique_consecutive (:436)."""
         g = np.asarray(torch.as_tensor(grid_thw).cpu(), dtype=np.int64).reshape(-1, 3)
@@ -327,56 +389,6 @@ class Qwen2_5_VisionTransformer(EricModel):
         g = grid_thw.reshape(-1, 3)
         seqlens = (g[:, 0] * g[:, 1] * g[:, 2]) // unit
         return list(out.split([int(s) for s in seqlens], dim=0))
-
-    def patchify_frames(self, frames: list[torch.Tensor], arithmetic: str = "fused") -> tuple[torch.Tensor, np.ndarray]:
-        """uint8 frames of every item ([T,H,W,3] or [H,W,3], already at the processor's target size, on the host
-        or the device) -> (pixel_values [L, C*T*P*P] in the model dtype on the device, grid_thw int64 [n,3]): what
-        the Hugging Face processor the reference runs (:488-512) produces from the same frames, with rescale,
-        normalise and the patch layout done on the GPU."""
-        p, m, tps, dev = self.patch_size, self.spatial_merge_size, self.temporal_patch_size, self.device
-        key = ("byte_table", arithmetic)
-        pk = self._ensure_packed()
-        if key not in pk:
-            pk[key] = frame_ops.byte_table(arithmetic=arithmetic).to(dev)
-        items, grids = [], []
-        for f in frames:
-            f = torch.as_tensor(f)
-            if f.dim() == 3:
-                f = f[None]
-            if f.dtype != torch.uint8 or f.dim() != 4 or f.shape[-1] != 3:
-                raise ValueError("frames must be uint8 [T,H,W,3] or [H,W,3] (RGB)")
-            T, H, W, _ = f.shape
-            if H % (p * m) or W % (p * m) or T < 1:
-                raise ValueError(f"frame size {H}x{W} is not a multiple of {p * m}: resize first (frames.resize_frames)")
-            items.append(f.contiguous().to(dev, non_blocking=True))
-            grids.append((-(-T // tps), H // p, W // p))
-        grid = np.asarray(grids, dtype=np.int64).reshape(-1, 3)
-        L = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
-        px = torch.empty((L, self.in_channels * tps * p * p), dtype=self.dtype, device=dev)
-        row = 0
-        for f, (gt, gh, gw) in zip(items, grids):
-            ops.qwen_patchify_u8(f, pk[key], p, m, tps, out=px[row : row + gt * gh * gw])
-            row += gt * gh * gw
-        return px, grid
-
-    @torch.inference_mode()
-    def forward(self, modality: Modality, adapter_name: str, batch: dict[str, list[torch.Tensor]]) -> list[torch.Tensor]:
-        """See the reference docstring (:402-413): `pixel_values` + `image_grid_thw` for images,
-        `pixel_values_videos` + `video_grid_thw` for videos.  In addition to the reference's format, a batch
-        may carry `pixel_frames` / `pixel_frames_videos` instead: one uint8 [T,H,W,3] tensor of resized frames
-        per item (see `FrameModalityProcessor`); the grids follow from the shapes."""
-        if modality == Modality.IMAGE:
-            px_key, grid_key, frame_key = "pixel_values", "image_grid_thw", "pixel_frames"
-        elif modality == Modality.VIDEO:
-            px_key, grid_key, frame_key = "pixel_values_videos", "video_grid_thw", "pixel_frames_videos"
-        else:
-            raise ValueError(f"Unsupported modality: {modality}")
-        if frame_key in batch:
-            return self.forward_device(*self.patchify_frames(batch[frame_key]))
-        pixel_values = torch.cat(batch[px_key], dim=0).to(device=self.device, dtype=self.dtype)
-        grid = torch.cat([g.reshape(-1, 3) for g in batch[grid_key]], dim=0).cpu().numpy().astype(np.int64)
-        return self.forward_device(pixel_values, grid)
-
 
 class ModalityProcessor(BaseModalityProcessor):
     """Qwen2.5-VL modality processor (reference: :488-512). Wraps the HF image processor, which has to be

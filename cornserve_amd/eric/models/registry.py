@@ -1,6 +1,6 @@
 """Registry entries for the MI355X-native encoders (reference: eric/models/registry.py:11-233).
 
-Same record types and the same two entries the reference keeps for these model types, so that
+Same record types and the same entries the reference keeps for these model types, so that
 `loader.load_model` (eric/executor/loader.py:62-96) can resolve them by `hf_config.model_type`.
 """
 
@@ -47,6 +47,14 @@ class RegistryEntry:
 
 
 MODEL_REGISTRY: dict[str, RegistryEntry] = {
+    "qwen2_vl": RegistryEntry(
+        module="qwen2_vl",
+        class_name="Qwen2VisionTransformer",
+        adapter_attr=None,
+        vit_resolution_type=ViTResolutionType.DYNAMIC,
+        weight=WeightInfo(required_prefixes=["visual."], strip_prefixes=True),
+        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
+    ),
     "qwen2_5_vl": RegistryEntry(
         module="qwen2_5_vl",
         class_name="Qwen2_5_VisionTransformer",

@@ -19,7 +19,7 @@ CS_ERR_LAUNCH = 3
 CS_ERR_TOO_LARGE = 4
 ABI_VERSION = 2
 
-EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH = range(5)
+EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH, EPI_QUICK_GELU = range(6)
 
 
 class CsGemmArgs(ctypes.Structure):

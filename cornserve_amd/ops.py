@@ -18,6 +18,7 @@ from .lib import (  # noqa: F401  (re-exported)
     EPI_BIAS,
     EPI_GELU_ERF,
     EPI_GELU_TANH,
+    EPI_QUICK_GELU,
     EPI_RESIDUAL,
     EPI_SWIGLU,
 )

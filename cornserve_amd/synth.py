@@ -106,6 +106,52 @@ def ragged_grids(n: int = 16, seed: int = 0, lo: int = 224, hi: int = 1344) -> l
     return [(1, int(h) // 14, int(w) // 14) for h, w in sizes]
 
 
+# ------------------------------------------------------------------------------------------ Qwen2-VL
+def qwen2_vision_config(depth: int = 32, embed_dim: int = 1280, hidden_size: int = 3584, num_heads: int = 16,
+                        mlp_ratio: float = 4.0) -> SimpleNamespace:
+    """The Qwen2-VL-7B vision tower's hyper-parameters (only `vision_config` and `rms_norm_eps` are read)."""
+    vc = SimpleNamespace(depth=depth, embed_dim=embed_dim, hidden_size=hidden_size, num_heads=num_heads,
+                         mlp_ratio=mlp_ratio, in_channels=3, patch_size=14, temporal_patch_size=2, spatial_merge_size=2)
+    return SimpleNamespace(vision_config=vc, rms_norm_eps=1e-6, model_type="qwen2_vl")
+
+
+def qwen2_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
+    """fp32 state dict with the Qwen2-VL checkpoint's names (after `visual.` is stripped)."""
+    vc = config.vision_config
+    E, I, O = vc.embed_dim, int(vc.embed_dim * vc.mlp_ratio), vc.hidden_size
+    M = E * vc.spatial_merge_size**2
+    sd: dict[str, torch.Tensor] = {}
+
+    def mat(name, *shape):
+        sd[name] = normal(seed, name, shape, 0.02)
+
+    def ln(prefix):
+        sd[prefix + ".weight"] = normal(seed, prefix + ".weight", (E,), 0.02, 1.0)
+        sd[prefix + ".bias"] = normal(seed, prefix + ".bias", (E,), 0.02)
+
+    mat("patch_embed.proj.weight", E, vc.in_channels, vc.temporal_patch_size, vc.patch_size, vc.patch_size)
+    for i in range(vc.depth):
+        p = f"blocks.{i}."
+        ln(p + "norm1")
+        ln(p + "norm2")
+        for name, n, k in (("attn.qkv", 3 * E, E), ("attn.proj", E, E), ("mlp.fc1", I, E), ("mlp.fc2", E, I)):
+            mat(p + name + ".weight", n, k)
+            mat(p + name + ".bias", n)
+    ln("merger.ln_q")
+    mat("merger.mlp.0.weight", M, M)
+    mat("merger.mlp.0.bias", M)
+    mat("merger.mlp.2.weight", O, M)
+    mat("merger.mlp.2.bias", O)
+    return sd
+
+
+def qwen2_linear_weight_keys(config) -> list[str]:
+    keys = []
+    for i in range(config.vision_config.depth):
+        keys += [f"blocks.{i}.{n}.weight" for n in ("attn.qkv", "attn.proj", "mlp.fc1", "mlp.fc2")]
+    return keys + ["merger.mlp.0.weight", "merger.mlp.2.weight"]
+
+
 # --------------------------------------------------------------------------------------- Gemma-3 / SigLIP
 def gemma3_config(num_hidden_layers: int = 27, image_size: int = 896, text_hidden: int = 2560,
                   mm_tokens_per_image: int = 256) -> SimpleNamespace:

@@ -52,7 +52,9 @@ enum CsEpilogue {
   CS_EPI_SWIGLU = 2,    /* W rows interleaved gate_j,up_j; y[m,j] = silu(g)*u; C is N/2 wide
                            qwen2_5_vl.py:143-148                                               */
   CS_EPI_GELU_ERF = 3,  /* y = gelu(acc + bias), erf form               qwen2_5_vl.py:220       */
-  CS_EPI_GELU_TANH = 4  /* y = gelu(acc + bias), tanh form              siglip.py:155-163       */
+  CS_EPI_GELU_TANH = 4, /* y = gelu(acc + bias), tanh form              siglip.py:155-163       */
+  CS_EPI_QUICK_GELU = 5 /* y = x * sigmoid(1.702 x), x = acc + bias     layers/activations.py:9-12
+                           (Qwen2-VL MLP, qwen2_vl.py:112-128)                                   */
 };
 
 typedef struct CsGemmArgs {

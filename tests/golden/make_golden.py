@@ -13,6 +13,8 @@ of cornserve_amd.synth, fp32, CPU, eager/sdpa attention.  Outputs:
                              (full arrays for small grids, sha256 + head for large ones)
     qwen2_5_vl_cfg1.npz      config 1 (4 blocks, one 448x448 image): every 16th column of the [256,3584]
                              output, per-row L2 norms, sum and abs-sum
+    qwen2_vl_small.npz       2-block Qwen2-VL tower (width 1280), an image (1,16,16) and a video (2,8,12): every 8th
+                             column of the [112,3584] output, per-row L2 norms, sum
     gemma3_small.npz         2-layer SigLIP (224x224, 256 tokens) + projector to 16 tokens x 640: full output
 """
 
@@ -108,6 +110,32 @@ def make_qwen_cfg1() -> None:
     print("qwen2_5_vl_cfg1.npz", out.shape, float(np.abs(out).mean()))
 
 
+def make_qwen2_vl_small() -> None:
+    from transformers.models.qwen2_vl.configuration_qwen2_vl import Qwen2VLVisionConfig
+    from transformers.models.qwen2_vl.modeling_qwen2_vl import Qwen2VisionTransformerPretrainedModel
+
+    cfg = synth.qwen2_vision_config(depth=2)
+    vc = cfg.vision_config
+    hf_cfg = Qwen2VLVisionConfig(depth=vc.depth, embed_dim=vc.embed_dim, hidden_size=vc.hidden_size, num_heads=vc.num_heads,
+                                 mlp_ratio=int(vc.mlp_ratio), patch_size=vc.patch_size, spatial_merge_size=vc.spatial_merge_size,
+                                 temporal_patch_size=vc.temporal_patch_size, hidden_act="quick_gelu")
+    hf_cfg._attn_implementation = "sdpa"
+    model = Qwen2VisionTransformerPretrainedModel(hf_cfg).float().eval()
+    sd = synth.qwen2_state_dict(cfg, seed=3)
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys, inc
+    grids = [(1, 16, 16), (2, 8, 12)]
+    px, grid = synth.qwen_inputs(grids, seed=3)
+    with torch.no_grad():
+        out = model(torch.cat(px), grid_thw=torch.cat(grid))
+    out = (out.pooler_output if hasattr(out, "pooler_output") else out).float().numpy()
+    assert out.shape == ((256 + 192) // 4, 3584), out.shape
+    np.savez_compressed(HERE / "qwen2_vl_small.npz", sample=out[:, ::8].astype(np.float32),
+                        row_l2=np.linalg.norm(out.astype(np.float64), axis=1).astype(np.float32),
+                        total=np.float64(out.astype(np.float64).sum()), seed=np.int64(3))
+    print("qwen2_vl_small.npz", out.shape, float(np.abs(out).mean()))
+
+
 def make_gemma3_small() -> None:
     from transformers.models.gemma3.configuration_gemma3 import Gemma3Config, Gemma3TextConfig
     from transformers.models.gemma3.modeling_gemma3 import Gemma3MultiModalProjector
@@ -148,4 +176,5 @@ def make_gemma3_small() -> None:
 if __name__ == "__main__":
     make_index()
     make_qwen_cfg1()
+    make_qwen2_vl_small()
     make_gemma3_small()

@@ -162,6 +162,66 @@ def test_qwen_errors_on_gpu(dev):
     assert wi[:8].tolist() == [0, 1, 2, 3, 16, 17, 18, 19] and cu == list(range(0, 1025, 64))
 
 
+# ------------------------------------------------------------------------------------------ Qwen2-VL
+def build_qwen2(dev, depth, seed, weight_format="bf16"):
+    from cornserve_amd.eric.models.qwen2_vl import Qwen2VisionTransformer
+    from oracle import qwen2_vl as o2
+
+    cfg = synth.qwen2_vision_config(depth=depth)
+    sd = synth.qwen2_state_dict(cfg, seed=seed)
+    model = Qwen2VisionTransformer(cfg, weight_format=weight_format)
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys
+    return model.to(device=dev, dtype=torch.bfloat16).eval(), sd, o2.Qwen2VisionConfig(depth=depth), cfg
+
+
+def test_qwen2_vl_against_oracle_and_golden(dev, golden_dir):
+    from oracle import qwen2_vl as o2
+
+    model, sd, ocfg, _ = build_qwen2(dev, 2, seed=3)
+    grids = [(1, 16, 16), (2, 8, 12)]
+    px, grid = synth.qwen_inputs(grids, seed=3)
+    img = model(Modality.IMAGE, "", {"pixel_values": px[:1], "image_grid_thw": grid[:1]})
+    vid = model(Modality.VIDEO, "", {"pixel_values_videos": px[1:], "video_grid_thw": grid[1:]})
+    assert img[0].shape == (64, 3584) and vid[0].shape == (48, 3584) and img[0].dtype == torch.bfloat16
+    both = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    assert torch.equal(both[0], img[0]) and torch.equal(both[1], vid[0])        # items are independent
+    ref16 = o2.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
+    ref32 = o2.forward(sd, ocfg, px, grid, dtype=torch.float32)
+    for i in range(2):
+        check(both[i], ref16[i], REL_BF16, f"qwen2-vl item {i} vs bf16 oracle")
+        check(both[i], ref32[i], REL_BF16, f"qwen2-vl item {i} vs fp32 oracle")
+    gold = np.load(golden_dir / "qwen2_vl_small.npz")      # Hugging Face fp32 output, every 8th column
+    check(torch.cat(both)[:, ::8], torch.from_numpy(gold["sample"]), REL_BF16, "qwen2-vl vs committed golden sample")
+
+
+def test_qwen2_vl_ragged_frames_and_fp8(dev):
+    from oracle import qwen2_vl as o2
+    from oracle import qwen2_5_vl as oq5
+    from oracle import qwen_preprocess as qp
+
+    model, sd, ocfg, cfg = build_qwen2(dev, 3, seed=4)
+    grids = [(1, 18, 14), (1, 2, 2), (1, 6, 34), (3, 4, 8)]
+    px, grid = synth.qwen_inputs(grids, seed=4)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    ref = o2.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
+    assert [tuple(o.shape) for o in out] == [tuple(r.shape) for r in ref]
+    for i, (o, r) in enumerate(zip(out, ref)):
+        check(o, r, REL_BF16, f"qwen2-vl ragged item {i} {grids[i]}")
+    # the uint8-frame input format, shared with the Qwen2.5-VL encoder
+    frames = np.random.default_rng(4).integers(0, 256, (3, 56, 84, 3), dtype=np.uint8)
+    fpx, fgrid = qp.patchify_frames(frames, qp.normalization_table(arithmetic="fused"))
+    a = model(Modality.VIDEO, "", {"pixel_values_videos": [torch.from_numpy(fpx)], "video_grid_thw": [torch.tensor([fgrid])]})
+    b = model(Modality.VIDEO, "", {"pixel_frames_videos": [torch.from_numpy(frames)]})
+    assert torch.equal(a[0], b[0])
+    # fp8 weights against the de-quantised fp32 oracle
+    model8, sd8, ocfg8, cfg8 = build_qwen2(dev, 2, seed=5, weight_format="fp8_e4m3")
+    sd_dq = oq5.dequantized_state_dict(sd8, synth.qwen2_linear_weight_keys(cfg8))
+    px, grid = synth.qwen_inputs([(2, 12, 20)], seed=5)
+    out = model8(Modality.VIDEO, "", {"pixel_values_videos": px, "video_grid_thw": grid})
+    check(out[0], o2.forward(sd_dq, ocfg8, px, grid, dtype=torch.float32)[0], REL_FP8, "qwen2-vl fp8 vs de-quantised fp32 oracle")
+
+
 def build_gemma(dev, layers, image_size, text_hidden, tokens, seed):
     from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
 

@@ -185,6 +185,11 @@ def test_gemm_epilogues(ops, dev):
     close(ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res), base + res.float().cpu(), 2**-7, "residual")
     close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_ERF), F.gelu(base), 2**-7, "gelu erf")
     close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_TANH), F.gelu(base, approximate="tanh"), 2**-7, "gelu tanh")
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_QUICK_GELU), base * torch.sigmoid(1.702 * base), 2**-7, "quick gelu")
+    # the general kernel's copy of the same epilogue (K = 72 is not a shape the fast kernel takes)
+    a72, w72 = a[:, :72].contiguous(), w[:, :72].contiguous()
+    base72 = lin_ref(a72, w72, b).bfloat16().float()
+    close(ops.gemm(a72, w72, b, epilogue=ops.EPI_QUICK_GELU), base72 * torch.sigmoid(1.702 * base72), 2**-7, "quick gelu, general kernel")
     gate, up = base[:, 0::2], base[:, 1::2]
     close(ops.gemm(a, w, b, epilogue=ops.EPI_SWIGLU), F.silu(gate).bfloat16().float() * up, 2**-7, "swiglu")
     # in-place residual (out aliases residual), as the model uses it
@@ -206,6 +211,8 @@ def _epilogue_ref(ops, epi, base, res):
         return F.gelu(base)
     if epi == ops.EPI_GELU_TANH:
         return F.gelu(base, approximate="tanh")
+    if epi == ops.EPI_QUICK_GELU:
+        return base * torch.sigmoid(1.702 * base)
     gate, up = base[:, 0::2], base[:, 1::2]
     return F.silu(gate).bfloat16().float() * up
 
@@ -226,7 +233,7 @@ def test_gemm_fast_path_forms(ops, dev, M, N, K):
     rows = torch.arange(0, M, max(1, M // 257))  # a sample of rows: the fp32 reference runs on the host
     rows = torch.cat([rows, torch.tensor([M - 1])])
     base = lin_ref(a[rows], w, b).bfloat16().float()
-    for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_SWIGLU):
+    for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU, ops.EPI_SWIGLU):
         got = ops.gemm(a, w, b, epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
         close(got[rows], _epilogue_ref(ops, epi, base, res[rows]), 2**-7, f"{M}x{N}x{K} epilogue {epi}")
     # repeated launches give identical bits (fixed accumulation order, no races between the two launches of
@@ -257,7 +264,7 @@ def test_gemm_fast_path_forms_fp8_weights(ops, dev, M, N, K):
     rows = torch.cat([torch.arange(0, M, max(1, M // 257)), torch.tensor([M - 1])])
     base = (a[rows].float().cpu() @ wd.t() + b.float().cpu()).bfloat16().float()
     qd, sd = q.to(dev), scale.to(dev)
-    for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_SWIGLU):
+    for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU, ops.EPI_SWIGLU):
         got = ops.gemm(a, qd, b, w_scale=sd, epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
         close(got[rows], _epilogue_ref(ops, epi, base, res[rows]), 2**-7, f"fp8 {M}x{N}x{K} epilogue {epi}")
     first = ops.gemm(a, qd, b, w_scale=sd)

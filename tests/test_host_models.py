@@ -114,3 +114,22 @@ def test_frame_processor_resize_and_table_match_the_hf_pil_processor():
         fr.resize_frames(np.zeros((4, 4), np.uint8))
     with pytest.raises(ValueError):
         fr.target_size(1, 500)
+
+
+def test_qwen2_vl_class_surface():
+    from cornserve_amd import synth
+    from cornserve_amd.eric.models.qwen2_vl import Qwen2VisionTransformer
+    from cornserve_amd.eric.models.registry import MODEL_REGISTRY
+
+    cfg = synth.qwen2_vision_config(depth=2)
+    model = Qwen2VisionTransformer(cfg)
+    sd = synth.qwen2_state_dict(cfg, seed=0)
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys          # the checkpoint's names, nothing else
+    assert model.chunk_shape == (1, 3584) and model.dtype == torch.float32 and model.device.type == "cpu"
+    entry = MODEL_REGISTRY["qwen2_vl"]
+    assert entry.module == "qwen2_vl" and entry.class_name == "Qwen2VisionTransformer" and entry.weight.required_prefixes == ["visual."]
+    with pytest.raises(RuntimeError):                                # no CPU path
+        model._ensure_packed()
+    with pytest.raises(ValueError):
+        Qwen2VisionTransformer(cfg, weight_format="int4")

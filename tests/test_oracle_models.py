@@ -106,3 +106,73 @@ def test_bf16_stepwise_close_to_fp32():
     b = oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)[0].float()
     cos = F.cosine_similarity(a.flatten(), b.flatten(), dim=0).item()
     assert cos > 0.999
+
+
+# ------------------------------------------------------------------------------------------ Qwen2-VL
+def _qwen2_small(depth=2, seed=3):
+    from oracle import qwen2_vl as o2
+
+    cfg = synth.qwen2_vision_config(depth=depth)
+    return o2, cfg, o2.Qwen2VisionConfig(depth=depth), synth.qwen2_state_dict(cfg, seed=seed)
+
+
+def test_qwen2_vl_against_golden(golden_dir):
+    gold = np.load(golden_dir / "qwen2_vl_small.npz")
+    o2, cfg, ocfg, sd = _qwen2_small(seed=int(gold["seed"]))
+    px, grid = synth.qwen_inputs([(1, 16, 16), (2, 8, 12)], seed=int(gold["seed"]))
+    out = o2.forward(sd, ocfg, px, grid, dtype=torch.float32)
+    assert [tuple(o.shape) for o in out] == [(64, 3584), (48, 3584)]
+    o = torch.cat(out).numpy()
+    assert np.abs(o[:, ::8] - gold["sample"]).max() <= 2e-4 * np.abs(gold["sample"]).max()
+    assert np.allclose(np.linalg.norm(o.astype(np.float64), axis=1), gold["row_l2"], rtol=1e-4)
+    assert abs(o.astype(np.float64).sum() - float(gold["total"])) <= 1e-4 * np.abs(o.astype(np.float64)).sum()
+
+
+def test_qwen2_vl_live_against_hugging_face():
+    """The same comparison against the installed third-party implementation on another shape (a ragged image and a
+    three-frame-group video), when it is importable."""
+    cm = pytest.importorskip("transformers.models.qwen2_vl.configuration_qwen2_vl")
+    mm = pytest.importorskip("transformers.models.qwen2_vl.modeling_qwen2_vl")
+    o2, cfg, ocfg, sd = _qwen2_small(depth=1, seed=8)
+    vc = cfg.vision_config
+    hf_cfg = cm.Qwen2VLVisionConfig(depth=1, embed_dim=vc.embed_dim, hidden_size=vc.hidden_size, num_heads=vc.num_heads,
+                                    mlp_ratio=int(vc.mlp_ratio), patch_size=14, spatial_merge_size=2, temporal_patch_size=2,
+                                    hidden_act="quick_gelu")
+    hf_cfg._attn_implementation = "sdpa"
+    model = mm.Qwen2VisionTransformerPretrainedModel(hf_cfg).float().eval()
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys
+    px, grid = synth.qwen_inputs([(1, 6, 10), (3, 4, 4)], seed=8)
+    with torch.no_grad():
+        ref = model(torch.cat(px), grid_thw=torch.cat(grid))
+    ref = ref.pooler_output if hasattr(ref, "pooler_output") else ref
+    got = torch.cat(o2.forward(sd, ocfg, px, grid, dtype=torch.float32))
+    assert got.shape == ref.shape == ((60 + 48) // 4, 3584)
+    assert (got - ref).abs().max().item() <= 2e-4 * ref.abs().max().item()
+
+
+def test_qwen2_vl_pieces():
+    from oracle import qwen2_vl as o2
+
+    x = torch.linspace(-6, 6, 25)
+    assert torch.allclose(o2.quick_gelu(x), x / (1 + torch.exp(-1.702 * x)), atol=1e-6)
+    assert o2.quick_gelu(torch.tensor(0.0)).item() == 0.0 and abs(o2.quick_gelu(torch.tensor(20.0)).item() - 20.0) < 1e-5
+    # rotary angles: position (h, w) times inv_freq, h-half then w-half, rows in 2x2-block-major order
+    cfg = o2.Qwen2VisionConfig()
+    ang = o2.rotary_angles(cfg, np.array([[1, 4, 4]]))
+    inv = 1.0 / (10000.0 ** (torch.arange(0, 40, 2, dtype=torch.float) / 40))
+    assert ang.shape == (16, 40)
+    assert torch.equal(ang[0], torch.zeros(40))                                  # patch (0,0)
+    assert torch.allclose(ang[1], torch.cat([torch.zeros(20), inv]))             # patch (0,1)
+    assert torch.allclose(ang[2], torch.cat([inv, torch.zeros(20)]))             # patch (1,0)
+    assert torch.allclose(ang[4], torch.cat([torch.zeros(20), 2 * inv]))         # next block: patch (0,2)
+    # items are independent and frames of a video do not attend to each other
+    o2_, cfg_s, ocfg, sd = _qwen2_small(depth=1, seed=9)
+    px, grid = synth.qwen_inputs([(2, 4, 4), (1, 4, 6)], seed=9)
+    both = o2.forward(sd, ocfg, px, grid)
+    alone = o2.forward(sd, ocfg, px[1:], grid[1:])
+    assert torch.allclose(both[1], alone[0], atol=1e-6)
+    px2 = [px[0].clone(), px[1]]
+    px2[0][16:] += 1.0                                                           # change the second frame group only
+    pert = o2.forward(sd, ocfg, px2, grid)
+    assert torch.equal(pert[0][:4], both[0][:4]) and not torch.allclose(pert[0][4:], both[0][4:])
