@@ -367,6 +367,10 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
   constexpr int HC = DC / 2;
   static_assert(D % 8 == 0 && D <= 96, "head dim");
   static_assert(!ROPE || D % 16 == 0, "rotary needs an even number of chunks per half");
+  // When the head dim does not fill its last 32-row block of O^T, one of the spare V columns is set to 1:
+  // row D of O^T is then sum_k P[k], the softmax denominator, accumulated (and rescaled) by the matrix cores
+  // together with O instead of 32 vector additions and a shuffle per tile.
+  constexpr bool L_FROM_MFMA = (D % 32) != 0;
   constexpr int K_BYTES = BKV * RS, V_BYTES = BKV * V_RS, Q_BYTES = BQ * RS;
   constexpr int REGION_B = (K_BYTES + V_BYTES) > Q_BYTES ? (K_BYTES + V_BYTES) : Q_BYTES;
   __shared__ __attribute__((aligned(16))) char lds[K_BYTES + V_BYTES + REGION_B];
@@ -473,6 +477,15 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
     }
   };
 
+  // chunk DC (dims D .. D+7) of every key row of V buffer b := (1, 0, ..., 0); lstore_tile never writes there
+  auto store_ones_column = [&](int b) {
+    if constexpr (L_FROM_MFMA) {
+      bf16x8_t one = zero8;
+      one[0] = f2bf(1.0f);
+      for (int r = tid; r < BKV; r += NT) *(bf16x8_t*)(v_buf(b) + r * V_RS + DC * 16) = one;
+    }
+  };
+
   // ---- prologue: Q -> LDS (rotated), tile 0 -> LDS buffer 0
   gload_tile(0, min(BKV, seg_len));
   {
@@ -510,11 +523,13 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
     }
   }
   lstore_tile(0);
+  store_ones_column(0);
   __syncthreads();
   bf16x8_t qf[KS];
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8_t*)(q_lds + (wave * 32 + fr) * RS + (2 * ks + hf) * 16);
   __syncthreads();  // every wave holds its Q fragments: the Q region may now become K/V buffer 1
+  store_ones_column(1);  // (ordered before the first read of buffer 1 by the barrier that ends iteration 0)
 
   f32x16_t oacc[DT];
 #pragma unroll
@@ -559,9 +574,23 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run, mx);
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
-      const float mb = m_new * sl2;
+      // Lazy reference maximum: P = exp2((s - m_run) * scale) with an m_run that is only raised when some
+      // query of the wave sees a score more than LAZY_LOG2 (in log2 units) above it.  P then ranges up to
+      // 2^LAZY_LOG2 instead of 1, which fp32 accumulation and bf16's exponent range do not care about, the
+      // final division by the denominator (built from the same P) cancels the reference, and the rescale of
+      // O -- DT*16 multiplies and an exponential per tile -- runs only in the first tiles of a segment.
+      constexpr float LAZY_LOG2 = 6.0f;
+      float alpha = 1.0f;
+      if (__any((mx - m_run) * sl2 > LAZY_LOG2)) {  // m_run starts at -inf: always taken for the first tile
+        const float m_new = fmaxf(m_run, mx);
+        alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
+#pragma unroll
+        for (int t = 0; t < DT; ++t)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+        m_run = m_new;
+      }
+      const float mb = m_run * sl2;
       float psum = 0.f;
       bf16x8_t pf[2][2];
 #pragma unroll
@@ -569,18 +598,13 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * sl2 - mb);
-          psum += pv;
+          if constexpr (!L_FROM_MFMA) psum += pv;
           pf[kt][r >> 3][r & 7] = f2bf(pv);
         }
-      psum += __shfl_xor(psum, 32, 64);
-      l_run = l_run * alpha + psum;
-      if (__any(m_new != m_run)) {  // the running maximum moved for some query of this wave: rescale O
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+      if constexpr (!L_FROM_MFMA) {
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * alpha + psum;
       }
-      m_run = m_new;
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
 #pragma unroll
@@ -596,6 +620,13 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
     __syncthreads();
   }
 
+  if constexpr (L_FROM_MFMA) {
+    // row D of O^T: block D/32, row D%32 = 8g + 4*hf + e; the lanes of the owning half hold it for their query
+    constexpr int RR = D % 32, G_L = RR / 8, HF_L = (RR % 8) / 4, E_L = RR % 4;
+    const float mine = oacc[D / 32][4 * G_L + E_L];
+    const float other = __shfl_xor(mine, 32, 64);
+    l_run = hf == HF_L ? mine : other;
+  }
   const int qi = wave * 32 + fr;
   if (qi < nq) {
     const float inv = 1.0f / l_run;
