@@ -646,6 +646,307 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
   }
 }
 
+// Full attention without rotary (SigLIP): K and V tiles go global -> LDS directly (buffer_load ... lds: no
+// staging registers, no LDS store instructions, no address arithmetic per tile) into a ring of three tile
+// buffers, requested two tiles ahead.  A direct load fixes the LDS side -- the 64 lanes of a wave fill 1 KB of
+// consecutive LDS -- so the padded row layout is produced on the global side: a tile is the flat sequence of
+// 16-byte chunk slots (row, slot), lane l of load j owns slot j*64 + l and fetches chunk `slot % slots_per_row`
+// of row `slot / slots_per_row`; lanes that own padding slots are switched off for the load, which leaves the
+// padding as initialised once per buffer (zeros behind the K rows that the last k-step reads, the ones
+// column of V that yields the softmax denominator).
+typedef __attribute__((address_space(3))) void lds_void_t;
+
+// Transposing LDS reads of the four V^T fragments (keys 16g .. 16g+15, g = 0..3) of dims 32*TT .. 32*TT+31, written in
+// assembly (see the kernel for why); the caller waits for them with an explicit s_waitcnt.
+template <int TT, int G>
+CS_DEVICE void read_vt_pair_asm(i32x2_t& lo, i32x2_t& hi, uint32_t vbase) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(vbase), "n"(G * 16 * V_RS + TT * 64));
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(vbase), "n"(G * 16 * V_RS + TT * 64 + 8 * V_RS));
+}
+template <int TT>
+CS_DEVICE void read_vt_block_asm(i32x2_t (&raw)[8], uint32_t vbase) {
+  read_vt_pair_asm<TT, 0>(raw[0], raw[1], vbase);
+  read_vt_pair_asm<TT, 1>(raw[2], raw[3], vbase);
+  read_vt_pair_asm<TT, 2>(raw[4], raw[5], vbase);
+  read_vt_pair_asm<TT, 3>(raw[6], raw[7], vbase);
+}
+template <bool LAST>
+CS_DEVICE void pv_block(f32x16_t& o, i32x2_t (&raw)[8], const bf16x8_t (&pf)[2][2]) {
+  if constexpr (LAST) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  else asm volatile("s_waitcnt lgkmcnt(8)" ::: "memory");
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    i32x4_t both = {raw[2 * g][0], raw[2 * g][1], raw[2 * g + 1][0], raw[2 * g + 1][1]};
+    asm volatile("" : "+v"(both));  // the registers hold the data only after the wait above
+    o = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, both), pf[g >> 1][g & 1], o, 0, 0, 0);
+  }
+}
+
+template <int D>
+struct AttnDirectShape {
+  static constexpr int KS = (D + 15) / 16, DKC = KS * 2, DC = D / 8;
+  static constexpr int K_SLOTS = DKC | 1, V_SLOTS = V_RS / 16;      // 16-byte slots per tile row
+  static constexpr int RS = K_SLOTS * 16;
+  static constexpr int K_BYTES = BKV * RS, V_BYTES = BKV * V_RS, TILE_BYTES = K_BYTES + V_BYTES;
+  static constexpr int K_LOADS = BKV * K_SLOTS / 64, V_LOADS = BKV * V_SLOTS / 64;   // BKV == 64: one load per slot column
+  static constexpr int LOADS = K_LOADS + V_LOADS, PER_WAVE = (LOADS + 3) / 4;
+  static constexpr int NBUF = 3, LDS = NBUF * TILE_BYTES;
+  static_assert(128 * RS <= 2 * TILE_BYTES, "the Q tile aliases buffers 1 and 2");
+  static_assert(2 * LDS <= 160 * 1024, "two workgroups per CU");
+};
+
+template <int D>
+__global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs a) {
+  constexpr int NT = 256, BQ = 128;
+  using Shape = AttnDirectShape<D>;
+  constexpr int KS = Shape::KS, DT = (D + 31) / 32, DC = Shape::DC, DKC = Shape::DKC;
+  constexpr int RS = Shape::RS, K_SLOTS = Shape::K_SLOTS, V_SLOTS = Shape::V_SLOTS;
+  constexpr int K_BYTES = Shape::K_BYTES, TILE_BYTES = Shape::TILE_BYTES;
+  constexpr int K_LOADS = Shape::K_LOADS, LOADS = Shape::LOADS, PER = Shape::PER_WAVE;
+  static_assert(D % 8 == 0 && D <= 96 && BKV == 64, "head dim / tile");
+  constexpr bool L_FROM_MFMA = (D % 32) != 0;   // see attn_full_kernel
+  extern __shared__ __attribute__((aligned(1024))) char lds[];
+  auto k_buf = [&](int b) -> char* { return lds + b * TILE_BYTES; };
+  auto v_buf = [&](int b) -> char* { return lds + b * TILE_BYTES + K_BYTES; };
+  char* const q_lds = lds + TILE_BYTES;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int fr = lane & 31, hf = lane >> 5;
+  const int xcd = blockIdx.x & 7, j = blockIdx.x >> 3;   // workgroup mapping: see attn_full_kernel
+  const int cid = (j / a.chunk) * 8 + xcd;
+  const int item = (cid % a.n_chunks_x) * a.chunk + j % a.chunk;
+  const int head = cid / a.n_chunks_x;
+  if (item >= a.n_work || head >= a.heads) return;
+  const int seg_start = a.work[item * 4 + 0];
+  const int seg_end = a.work[item * 4 + 1];
+  const int q0 = a.work[item * 4 + 2];
+  const int nq = a.work[item * 4 + 3];
+  const int64_t hoff = (int64_t)head * D;
+  const int seg_len = seg_end - seg_start;
+  const int n_tiles = (seg_len + BKV - 1) / BKV;
+  const bf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  // ---- the wave's direct loads of a tile.  Load u of this wave is load number jl = min(4u + wave, LOADS-1) of the
+  //      tile (the clamp makes a wave without a load of its own repeat the last one: every wave must issue the
+  //      same number, because the waits count loads).  Byte offsets are relative to the segment's first row.
+  const __amdgpu_buffer_rsrc_t rsrc_k =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(a.k + (int64_t)seg_start * a.ld + hoff), 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_v =
+      __builtin_amdgcn_make_buffer_rsrc((void*)(a.v + (int64_t)seg_start * a.ld + hoff), 0, -1, 0x00020000);
+  const uint32_t row_bytes = (uint32_t)a.ld * 2u;
+  int l_row[PER], l_chunk[PER];
+#pragma unroll
+  for (int u = 0; u < PER; ++u) {
+    const int jl = min(4 * u + wave, LOADS - 1);
+    const bool is_k = jl < K_LOADS;
+    const int slot = (is_k ? jl : jl - K_LOADS) * 64 + lane;
+    const int per_row = is_k ? K_SLOTS : V_SLOTS;
+    l_row[u] = slot / per_row;
+    l_chunk[u] = slot - l_row[u] * per_row;   // >= DC: a padding slot, the lane sits the load out
+  }
+  auto issue_k = [&](char* dst, uint32_t off, uint32_t soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (lds_void_t*)dst, 16, off, soff, 0, 0);
+  };
+  auto issue_v = [&](char* dst, uint32_t off, uint32_t soff) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_v, (lds_void_t*)dst, 16, off, soff, 0, 0);
+  };
+  auto issue_tile = [&](int t, int b) {
+    const int nvalid = min(BKV, seg_len - t * BKV);
+    const uint32_t soff = (uint32_t)(t * BKV) * row_bytes;
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+      const int jl = min(4 * u + wave, LOADS - 1);
+      // rows past the segment end repeat the last valid row: as keys they are masked, and P = 0 times a finite V row is 0
+      const uint32_t off = (uint32_t)min(l_row[u], nvalid - 1) * row_bytes + (uint32_t)l_chunk[u] * 16u;
+      if (jl < K_LOADS) {   // uniform
+        char* dst = k_buf(b) + jl * 1024;
+        if (l_chunk[u] < DC) issue_k(dst, off, soff);
+      } else {
+        char* dst = v_buf(b) + (jl - K_LOADS) * 1024;
+        if (l_chunk[u] < DC) issue_v(dst, off, soff);
+      }
+    }
+  };
+  auto init_padding = [&](int b) {
+    if constexpr (DKC > DC) {
+      for (int i = tid; i < BKV * (DKC - DC); i += NT) {
+        const int r = i / (DKC - DC), c = DC + i % (DKC - DC);
+        *(bf16x8_t*)(k_buf(b) + r * RS + c * 16) = zero8;
+      }
+    }
+    if constexpr (L_FROM_MFMA) {
+      bf16x8_t one = zero8;
+      one[0] = f2bf(1.0f);
+      for (int r = tid; r < BKV; r += NT) *(bf16x8_t*)(v_buf(b) + r * V_RS + DC * 16) = one;
+    }
+  };
+  auto wait_loads = [&](auto pending_c) {   // at most `pending` of this wave's direct loads still in flight
+    constexpr int N = decltype(pending_c)::value;
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N) : "memory");
+  };
+  auto barrier = [&]() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+
+  // ---- prologue: tile 0 requested, Q -> LDS -> fragments, then the Q region becomes buffers 1 and 2
+  issue_tile(0, 0);
+  init_padding(0);
+  for (int i = tid; i < BQ * DKC; i += NT) {
+    const int r = i / DKC, c = i - r * DKC;
+    bf16x8_t x = zero8;
+    if (r < nq && c < DC) x = *(const bf16x8_t*)(a.q + (int64_t)(q0 + r) * a.ld + hoff + c * 8);
+    *(bf16x8_t*)(q_lds + r * RS + c * 16) = x;
+  }
+  __syncthreads();
+  bf16x8_t qf[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8_t*)(q_lds + (wave * 32 + fr) * RS + (2 * ks + hf) * 16);
+  __syncthreads();
+  init_padding(1);
+  init_padding(2);
+  if (n_tiles > 1) issue_tile(1, 1);
+
+  f32x16_t oacc[DT];
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) oacc[t][r] = 0.f;
+  float m_run = -INFINITY, l_run = 0.f;
+  const bool wave_active = wave * 32 < nq;
+  const float sl2 = a.scale_log2e;
+
+  int buf = 0, buf2 = 2;   // buffers of tile t and of tile t+2
+  for (int t = 0; t < n_tiles; ++t) {
+    // Tile t has landed when only the loads requested after it (tile t+1's) are in flight; the barrier then also
+    // says that every wave is done with tile t-1, whose buffer the request for tile t+2 reuses.
+    if (t + 1 < n_tiles) wait_loads(std::integral_constant<int, PER>{});
+    else wait_loads(std::integral_constant<int, 0>{});
+    barrier();
+    if (t + 2 < n_tiles) issue_tile(t + 2, buf2);
+    const int nvalid = min(BKV, seg_len - t * BKV);
+    if (wave_active) {
+      const char* kd = k_buf(buf);
+      const char* vd = v_buf(buf);
+      f32x16_t sacc[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sacc[kt][r] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const bf16x8_t kf = *(const bf16x8_t*)(kd + (kt * 32 + fr) * RS + (2 * ks + hf) * 16);
+          sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kt], 0, 0, 0);
+        }
+      }
+      if (nvalid < BKV) {  // only the last tile of a segment can be partial
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+            if (key >= nvalid) sacc[kt][r] = -INFINITY;
+          }
+      }
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      constexpr float LAZY_LOG2 = 6.0f;   // lazily raised reference maximum: see attn_full_kernel
+      float alpha = 1.0f;
+      if (__any((mx - m_run) * sl2 > LAZY_LOG2)) {
+        const float m_new = fmaxf(m_run, mx);
+        alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
+#pragma unroll
+        for (int tt = 0; tt < DT; ++tt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[tt][r] *= alpha;
+        m_run = m_new;
+      }
+      const float mb = m_run * sl2;
+      float psum = 0.f;
+      bf16x8_t pf[2][2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * sl2 - mb);
+          if constexpr (!L_FROM_MFMA) psum += pv;
+          pf[kt][r >> 3][r & 7] = f2bf(pv);
+        }
+      if constexpr (!L_FROM_MFMA) {
+        psum += __shfl_xor(psum, 32, 64);
+        l_run = l_run * alpha + psum;
+      }
+      // V^T fragments (see read_vt_frag for the addressing).  The transposing reads are written in assembly: as
+      // an intrinsic, the compiler takes them for possible readers of the LDS bytes that the direct loads in
+      // flight will write and puts a wait for ALL outstanding loads in front of them -- the tiles requested
+      // ahead included.  The waits on the reads themselves are therefore explicit too: the reads of block
+      // tt+1 are issued before the MFMAs of block tt, which wait until only those 8 are outstanding.
+      {
+        const int sg = lane & 15;
+        const uint32_t vbase = (uint32_t)(uintptr_t)(lds_void_t*)vd + (uint32_t)((4 * hf + (sg >> 2)) * V_RS + (16 * ((lane >> 4) & 1) + 4 * (sg & 3)) * 2);
+        i32x2_t vraw[2][8];   // [block parity][2 * fragment + half]
+        read_vt_block_asm<0>(vraw[0], vbase);
+        read_vt_block_asm<1>(vraw[1], vbase);
+        pv_block<false>(oacc[0], vraw[0], pf);
+        if constexpr (DT == 2) {
+          pv_block<true>(oacc[1], vraw[1], pf);
+        } else {
+          static_assert(DT == 3, "head dims up to 96");
+          read_vt_block_asm<2>(vraw[0], vbase);
+          pv_block<false>(oacc[1], vraw[1], pf);
+          pv_block<true>(oacc[DT - 1], vraw[0], pf);
+        }
+      }
+    }
+    buf2 = buf;   // tile t+3 will reuse this iteration's buffer
+    buf = buf == 2 ? 0 : buf + 1;
+  }
+
+  if constexpr (L_FROM_MFMA) {
+    constexpr int RR = D % 32, G_L = RR / 8, HF_L = (RR % 8) / 4, E_L = RR % 4;
+    const float mine = oacc[D / 32][4 * G_L + E_L];
+    const float other = __shfl_xor(mine, 32, 64);
+    l_run = hf == HF_L ? mine : other;
+  }
+  const int qi = wave * 32 + fr;
+  if (qi < nq) {
+    const float inv = 1.0f / l_run;
+    bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d0 = t * 32 + 8 * g + 4 * hf;
+        if (d0 < D) {
+          bf16x4_t o;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
+          *(bf16x4_t*)(orow + d0) = o;
+        }
+      }
+  }
+}
+
+template <int D>
+int launch_attn_full_direct(const AttnArgs& a, dim3 grid, hipStream_t stream) {
+  constexpr int lds = AttnDirectShape<D>::LDS;
+  static bool attr_set = false;
+  auto kern = attn_full_direct_kernel<D>;
+  if (!attr_set) {
+    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return CS_ERR_LAUNCH;
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, a);
+  return cs_launch_status();
+}
+
 template <int D>
 int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, bool rope, hipStream_t stream) {
   const dim3 grid(n_work, heads);
@@ -673,6 +974,8 @@ int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, 
       if constexpr (D % 16 == 0) hipLaunchKernelGGL((attn_full_kernel<D, true>), grid_full, dim3(256), 0, stream, a);
       else return CS_ERR_UNSUPPORTED;
     } else {
+      // the direct-to-LDS kernel addresses a segment's K/V rows with 32-bit byte offsets
+      if ((int64_t)max_seqlen * a.ld * 2 < (int64_t)1 << 31) return launch_attn_full_direct<D>(a, grid_full, stream);
       hipLaunchKernelGGL((attn_full_kernel<D, false>), grid_full, dim3(256), 0, stream, a);
     }
   }
