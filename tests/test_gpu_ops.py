@@ -418,6 +418,9 @@ def attn_ref(qkv, cu, nh, d, cos_sin=None):
     (72, [0, 500, 1000]),                   # SigLIP head dim (zero padded in LDS)
     (72, [0, 64]),
     (64, [0, 130]),
+    (96, [0, 200, 265]),
+    (72, [0, 4096]),                        # one SigLIP image: 64 key tiles through the three-buffer ring
+    (72, [0, 65, 129, 322]),                # one, two and three key tiles
 ])
 def test_attention(ops, dev, d, cu):
     nh, L = 16, cu[-1]
@@ -426,6 +429,31 @@ def test_attention(ops, dev, d, cu):
     H = nh * d
     got = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], plan, nh, d, d**-0.5)
     close(got, attn_ref(qkv, cu, nh, d), 2**-6, f"attention d={d} cu={cu}")
+
+
+@pytest.mark.parametrize("d,rotary", [(72, False), (80, True), (80, False), (64, False)])
+def test_attention_wide_score_range(ops, dev, d, rotary):
+    """Scores spread over many powers of two, with the largest keys LAST in each segment: the kernels keep a
+    reference maximum that is only raised when a score exceeds it by 2^6, so this walks through both the raised
+    and the not-raised case in every tile position, and through P values well above 1."""
+    nh, cu = 16, [0, 700, 1000]
+    L = cu[-1]
+    g = torch.Generator().manual_seed(3)
+    qkv = torch.randn((L, 3 * nh * d), generator=g)
+    ramp = torch.linspace(0.2, 4.0, L)[:, None]
+    qkv[:, nh * d:2 * nh * d] *= ramp                  # key magnitude grows along the sequence
+    qkv[:, :nh * d] *= 3.0
+    qkv = qkv.bfloat16().to(dev)
+    H = nh * d
+    plan = ops.attn_plan(np.array(cu, np.int32), dev)
+    cs = None
+    ang = None
+    if rotary:
+        ang = torch.rand((L, d // 2), generator=g) * 6.0
+        cs = torch.cat([ang.cos(), ang.sin()], dim=1).float().contiguous().to(dev)
+    got = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], plan, nh, d, d**-0.5, cs)
+    assert torch.isfinite(got.float()).all()
+    close(got, attn_ref(qkv, cu, nh, d, ang), 2**-6, f"wide score range d={d} rotary={rotary}")
 
 
 def test_attention_fused_rotary_and_standalone_rotary(ops, dev):
