@@ -75,6 +75,10 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
   constexpr int RS = (DKC | 1) * 16;   // LDS row stride in bytes, odd chunk count: conflict-free b128 reads
   static_assert(D % 8 == 0 && D <= 96, "head dim");
   static_assert(!ROPE || D % 16 == 0, "rotary needs an even number of chunks per half");
+  // The softmax denominator comes out of the P.V product through a column of ones in the V tile when the head
+  // dim leaves spare rows in the last 32-row block of O^T (see attn_full_kernel; the same arithmetic in every
+  // attention kernel keeps an item's result independent of which of them a batch's longest segment selects).
+  constexpr bool L_FROM_MFMA = (D % 32) != 0;
 
   __shared__ __attribute__((aligned(16))) char q_lds[BQ * RS];
   __shared__ __attribute__((aligned(16))) char k_lds[BKV * RS];
@@ -88,6 +92,11 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
   const int q0 = a.work[blockIdx.x * 4 + 2];
   const int nq = a.work[blockIdx.x * 4 + 3];
   int64_t hoff = (int64_t)head0 * D;  // column offset of the head being processed
+  if constexpr (L_FROM_MFMA) {  // chunk DC of every V row := (1, 0, ..., 0); the staging below never writes there
+    bf16x8_t one = {0, 0, 0, 0, 0, 0, 0, 0};
+    one[0] = f2bf(1.0f);
+    for (int r = tid; r < BKV; r += NT) *(bf16x8_t*)(v_lds + r * V_RS + DC * 16) = one;
+  }
 
   // Stage `nrows` rows starting at global row g0 (valid rows: < g0 + nvalid) of a [*, ld] tensor into an
   // LDS tile with row stride RS, zero-filling invalid rows and pad chunks, optionally rotating.
@@ -111,8 +120,8 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
             const float co = e < 4 ? c0[e] : c1[e - 4];
             const float si = e < 4 ? s0[e] : s1[e - 4];
             const float xa = bf2f(x1[e]), xb = bf2f(x2[e]);
-            o1[e] = f2bf(xa * co - xb * si);
-            o2[e] = f2bf(xa * si + xb * co);
+            o1[e] = f2bf(rot_first(xa, xb, co, si));
+            o2[e] = f2bf(rot_second(xa, xb, co, si));
           }
         }
         *(bf16x8_t*)(dst + r * RS + jc * 16) = o1;
@@ -158,6 +167,12 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
   const bool wave_active = wave * 32 < nq;
   // O^T[d][q] / l -> out[q][head*D + d]; lane owns query wave*32 + fr and 4 consecutive d per group.
   auto write_out = [&]() {
+    if constexpr (L_FROM_MFMA) {
+      constexpr int RR = D % 32, G_L = RR / 8, HF_L = (RR % 8) / 4, E_L = RR % 4;
+      const float mine = oacc[D / 32][4 * G_L + E_L];
+      const float other = __shfl_xor(mine, 32, 64);
+      l_run = hf == HF_L ? mine : other;
+    }
     const int qi = wave * 32 + fr;
     if (qi < nq) {
       const float inv = 1.0f / l_run;
@@ -222,11 +237,13 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * a.scale_log2e - mb);
-        psum += pv;
+        if constexpr (!L_FROM_MFMA) psum += pv;
         pf[kt][r >> 3][r & 7] = f2bf(pv);
       }
-    psum += __shfl_xor(psum, 32, 64);
-    l_run = l_run * alpha + psum;
+    if constexpr (!L_FROM_MFMA) {
+      psum += __shfl_xor(psum, 32, 64);
+      l_run = l_run * alpha + psum;
+    }
     m_run = m_new;
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
@@ -304,11 +321,11 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
             const float co = e < 4 ? c0[it][e] : c1[it][e - 4];
             const float si = e < 4 ? s0[it][e] : s1[it][e - 4];
             const float xa = bf2f(q1[it][e]), xb = bf2f(q2[it][e]);
-            qa[e] = f2bf(xa * co - xb * si);
-            qb[e] = f2bf(xa * si + xb * co);
+            qa[e] = f2bf(rot_first(xa, xb, co, si));
+            qb[e] = f2bf(rot_second(xa, xb, co, si));
             const float ya = bf2f(k1[it][e]), yb = bf2f(k2[it][e]);
-            ka[e] = f2bf(ya * co - yb * si);
-            kb[e] = f2bf(ya * si + yb * co);
+            ka[e] = f2bf(rot_first(ya, yb, co, si));
+            kb[e] = f2bf(rot_second(ya, yb, co, si));
           }
           *(bf16x8_t*)(q_lds + r * RS + jc * 16) = qa;
           *(bf16x8_t*)(q_lds + r * RS + (jc + HC) * 16) = qb;
@@ -451,8 +468,8 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
             const float co = e < 4 ? kc0[u][e] : kc1[u][e - 4];
             const float si = e < 4 ? ks0[u][e] : ks1[u][e - 4];
             const float xa = bf2f(kx1[u][e]), xb = bf2f(kx2[u][e]);
-            o1[e] = f2bf(xa * co - xb * si);
-            o2[e] = f2bf(xa * si + xb * co);
+            o1[e] = f2bf(rot_first(xa, xb, co, si));
+            o2[e] = f2bf(rot_second(xa, xb, co, si));
           }
           *(bf16x8_t*)(kd + r * RS + jc * 16) = o1;
           *(bf16x8_t*)(kd + r * RS + (jc + HC) * 16) = o2;
@@ -506,8 +523,8 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
             const float co = e < 4 ? c0[e] : c1[e - 4];
             const float si = e < 4 ? s0[e] : s1[e - 4];
             const float xa = bf2f(x1[e]), xb = bf2f(x2[e]);
-            o1[e] = f2bf(xa * co - xb * si);
-            o2[e] = f2bf(xa * si + xb * co);
+            o1[e] = f2bf(rot_first(xa, xb, co, si));
+            o2[e] = f2bf(rot_second(xa, xb, co, si));
           }
         }
         *(bf16x8_t*)(q_lds + r * RS + jc * 16) = o1;

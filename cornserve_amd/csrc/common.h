@@ -24,6 +24,20 @@ CS_DEVICE bf16_t f2bf(float x) { return (bf16_t)x; }
 // Round an fp32 value to bf16 precision and return it as fp32 (a "rounding point").
 CS_DEVICE float rbf(float x) { return (float)(bf16_t)x; }
 
+// One rotary pair in fp32 with every product and sum rounded on its own (no fused multiply-add), as the
+// reference's tensor program computes it (x1*cos - x2*sin, x1*sin + x2*cos): every kernel that rotates gives
+// the same bits, whichever of them a launch selects.
+CS_DEVICE float rot_first(float x1, float x2, float co, float si) {
+#pragma clang fp contract(off)
+  const float p = x1 * co, q = x2 * si;
+  return p - q;
+}
+CS_DEVICE float rot_second(float x1, float x2, float co, float si) {
+#pragma clang fp contract(off)
+  const float p = x1 * si, q = x2 * co;
+  return p + q;
+}
+
 CS_DEVICE float wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);

@@ -72,6 +72,53 @@ __global__ __launch_bounds__(256) void vit_index_kernel(const ItemMeta* __restri
   }
 }
 
+// Qwen3-VL learned position embedding, bilinearly interpolated from its side x side table to an item's h x w patch
+// grid (eric/models/qwen3_vl.py:364-420), written in patch order (2x2-block-major rows, repeated per frame).  The
+// arithmetic follows the reference's tensor program step by step: fp32 linspace positions (torch's two-sided
+// formula), fp32 corner weights, weights and table rows in bf16, each product rounded to bf16, the four products
+// summed in fp32 and rounded once.  One thread per 8 channels of one patch.
+__global__ __launch_bounds__(256) void pos_embed_interp_kernel(const bf16_t* __restrict__ table, int side, int E,
+                                                               const ItemMeta* __restrict__ meta, int merge,
+                                                               bf16_t* __restrict__ out, int64_t ldo) {
+  const ItemMeta it = meta[blockIdx.y];
+  const int chunks = E >> 3;
+  const int mm = merge * merge;
+  const int h = it.gh * merge, w = it.gw * merge;
+  const int64_t n = (int64_t)it.t * h * w * chunks;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= n) return;
+  const int c = (int)(idx % chunks);
+  const int pl = (int)(idx / chunks);         // patch within the item, in patch (block-major) order
+  const int ul = pl / mm, s = pl - ul * mm;
+  const int rem = ul % (it.gh * it.gw);
+  const int y = (rem / it.gw) * merge + s / merge, x = (rem % it.gw) * merge + s % merge;
+  auto position = [&](int i, int steps) -> float {   // torch.linspace(0, side - 1, steps)[i] in fp32
+    if (steps == 1) return 0.f;
+    const float end = (float)(side - 1);
+    const float step = end / (float)(steps - 1);
+    return i < steps / 2 ? step * (float)i : __fmaf_rn(-step, (float)(steps - i - 1), end);
+  };
+  const float hy = position(y, h), wx = position(x, w);
+  const int y0 = (int)hy, x0 = (int)wx;
+  const int y1 = min(y0 + 1, side - 1), x1 = min(x0 + 1, side - 1);
+  const float dh = hy - (float)y0, dw = wx - (float)x0;
+  const float w11 = dh * dw, w10 = dh - w11, w01 = dw - w11, w00 = 1.f - dh - dw + w11;
+  const float wq[4] = {rbf(w00), rbf(w01), rbf(w10), rbf(w11)};
+  const bf16_t* rows[4] = {table + (int64_t)(y0 * side + x0) * E, table + (int64_t)(y0 * side + x1) * E,
+                           table + (int64_t)(y1 * side + x0) * E, table + (int64_t)(y1 * side + x1) * E};
+  float acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const bf16x8_t e = *(const bf16x8_t*)(rows[k] + c * 8);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) acc[q] += rbf(bf2f(e[q]) * wq[k]);
+  }
+  bf16x8_t o;
+#pragma unroll
+  for (int q = 0; q < 8; ++q) o[q] = f2bf(acc[q]);
+  *(bf16x8_t*)(out + (int64_t)(it.patch_base + pl) * ldo + c * 8) = o;
+}
+
 template <typename V>
 __global__ __launch_bounds__(256) void row_gather_kernel(const char* __restrict__ in, int64_t in_stride,
                                                          const int32_t* __restrict__ rows,
@@ -86,12 +133,14 @@ __global__ __launch_bounds__(256) void row_gather_kernel(const char* __restrict_
 }
 
 // In-place rotary on the q and k column blocks of a packed [L, 3*heads*d] buffer.  One thread owns
-// 8 consecutive j of one (row, q|k, head): it reads x[j..j+8) and x[d/2+j..), rotates in fp32 and
+// VEC (8, or 4 when d/2 is not a multiple of 8) consecutive j of one (row, q|k, head): it reads x[j..j+VEC) and x[d/2+j..), rotates in fp32 and
 // writes both halves back with a single bf16 rounding.
+template <int VEC>
 __global__ __launch_bounds__(256) void rope_qk_kernel(bf16_t* __restrict__ qkv, int64_t ld,
                                                       const float* __restrict__ cos_sin, int L, int heads, int d) {
+  typedef __attribute__((__vector_size__(VEC * sizeof(__bf16)))) __bf16 vec_t;
   const int half = d >> 1;
-  const int cpr = half >> 3;  // chunks per (row, head, tensor)
+  const int cpr = half / VEC;  // chunks per (row, head, tensor)
   const int64_t total = (int64_t)L * 2 * heads * cpr;
   int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
@@ -101,23 +150,29 @@ __global__ __launch_bounds__(256) void rope_qk_kernel(bf16_t* __restrict__ qkv, 
   idx /= heads;
   const int which = idx % 2;
   const int64_t l = idx / 2;
-  bf16_t* base = qkv + l * ld + (int64_t)which * heads * d + h * d + jc * 8;
-  const float* cs = cos_sin + l * d + jc * 8;
-  const bf16x8_t x1 = *(const bf16x8_t*)base;
-  const bf16x8_t x2 = *(const bf16x8_t*)(base + half);
-  const f32x4_t c0 = *(const f32x4_t*)cs, c1 = *(const f32x4_t*)(cs + 4);
-  const f32x4_t s0 = *(const f32x4_t*)(cs + half), s1 = *(const f32x4_t*)(cs + half + 4);
-  bf16x8_t o1, o2;
+  bf16_t* base = qkv + l * ld + (int64_t)which * heads * d + h * d + jc * VEC;
+  const float* cs = cos_sin + l * d + jc * VEC;
+  const vec_t x1 = *(const vec_t*)base;
+  const vec_t x2 = *(const vec_t*)(base + half);
+  float co[VEC], si[VEC];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const float co = e < 4 ? c0[e] : c1[e - 4];
-    const float si = e < 4 ? s0[e] : s1[e - 4];
-    const float a = bf2f(x1[e]), b = bf2f(x2[e]);
-    o1[e] = f2bf(a * co - b * si);
-    o2[e] = f2bf(a * si + b * co);
+  for (int e = 0; e < VEC; e += 4) {
+    const f32x4_t c = *(const f32x4_t*)(cs + e), s = *(const f32x4_t*)(cs + half + e);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      co[e + q] = c[q];
+      si[e + q] = s[q];
+    }
   }
-  *(bf16x8_t*)base = o1;
-  *(bf16x8_t*)(base + half) = o2;
+  vec_t o1, o2;
+#pragma unroll
+  for (int e = 0; e < VEC; ++e) {
+    const float a = bf2f(x1[e]), b = bf2f(x2[e]);
+    o1[e] = f2bf(rot_first(a, b, co[e], si[e]));
+    o2[e] = f2bf(rot_second(a, b, co[e], si[e]));
+  }
+  *(vec_t*)base = o1;
+  *(vec_t*)(base + half) = o2;
 }
 
 }  // namespace
@@ -195,6 +250,22 @@ extern "C" int cs_vit_index(const int32_t* item_meta, int32_t n_items, int32_t m
   return cs_launch_status();
 }
 
+extern "C" int cs_pos_embed_interp(const void* table, int32_t side, int32_t E, const int32_t* item_meta, int32_t n_items,
+                                   int32_t max_units_per_item, int32_t merge, void* out, int64_t ldo, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (!table || !item_meta || !out || side <= 0 || E <= 0 || E % 8 || n_items < 0 || max_units_per_item < 0 || merge <= 0 ||
+      ldo < E || ldo % 8 || (((uintptr_t)table | (uintptr_t)out) & 15))
+    return CS_ERR_INVALID_ARG;
+  if (n_items == 0 || max_units_per_item == 0) return CS_OK;
+  if (n_items > 65535) return CS_ERR_TOO_LARGE;
+  const int64_t work = (int64_t)max_units_per_item * merge * merge * (E / 8);
+  if ((work + 255) / 256 > 0x7fffffff) return CS_ERR_TOO_LARGE;
+  const dim3 grid((unsigned)((work + 255) / 256), n_items), block(256);
+  hipLaunchKernelGGL(pos_embed_interp_kernel, grid, block, 0, stream, (const bf16_t*)table, side, E,
+                     (const ItemMeta*)item_meta, merge, (bf16_t*)out, ldo);
+  return cs_launch_status();
+}
+
 extern "C" int cs_row_gather(const void* in, int64_t in_stride_bytes, const int32_t* rows, void* out,
                              int64_t out_stride_bytes, int32_t n_rows, int32_t row_bytes, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
@@ -217,12 +288,18 @@ extern "C" int cs_row_gather(const void* in, int64_t in_stride_bytes, const int3
 extern "C" int cs_rope_qk(void* qkv, int64_t ld, const float* cos_sin, int32_t L, int32_t heads, int32_t head_dim,
                           void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
-  if (!qkv || !cos_sin || L < 0 || heads <= 0 || head_dim <= 0 || head_dim % 16 || ld % 8 ||
+  if (!qkv || !cos_sin || L < 0 || heads <= 0 || head_dim <= 0 || head_dim % 8 || ld % 8 ||
       ld < (int64_t)3 * heads * head_dim || (((uintptr_t)qkv | (uintptr_t)cos_sin) & 15))
     return CS_ERR_INVALID_ARG;
   if (L == 0) return CS_OK;
-  const int64_t total = (int64_t)L * 2 * heads * (head_dim / 16);
-  hipLaunchKernelGGL(rope_qk_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (bf16_t*)qkv, ld,
-                     cos_sin, L, heads, head_dim);
+  if (head_dim % 16 == 0) {
+    const int64_t total = (int64_t)L * 2 * heads * (head_dim / 16);
+    hipLaunchKernelGGL(rope_qk_kernel<8>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (bf16_t*)qkv, ld,
+                       cos_sin, L, heads, head_dim);
+  } else {  // d/2 is a multiple of 4 only (head dim 72): 8-byte vectors
+    const int64_t total = (int64_t)L * 2 * heads * (head_dim / 8);
+    hipLaunchKernelGGL(rope_qk_kernel<4>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (bf16_t*)qkv, ld,
+                       cos_sin, L, heads, head_dim);
+  }
   return cs_launch_status();
 }

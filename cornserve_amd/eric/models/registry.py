@@ -63,6 +63,22 @@ MODEL_REGISTRY: dict[str, RegistryEntry] = {
         weight=WeightInfo(required_prefixes=["visual."], strip_prefixes=True),
         modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
     ),
+    "qwen3_vl": RegistryEntry(
+        module="qwen3_vl",
+        class_name="Qwen3_VisionTransformer",
+        adapter_attr=None,
+        vit_resolution_type=ViTResolutionType.DYNAMIC,
+        weight=WeightInfo(required_prefixes=["model.visual."], strip_prefixes=True),
+        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
+    ),
+    "qwen3_vl_moe": RegistryEntry(
+        module="qwen3_vl",
+        class_name="Qwen3_VisionTransformer",
+        adapter_attr=None,
+        vit_resolution_type=ViTResolutionType.DYNAMIC,
+        weight=WeightInfo(required_prefixes=["model.visual."], strip_prefixes=True),
+        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
+    ),
     "gemma3": RegistryEntry(
         module="gemma3",
         class_name="Gemma3VisionEncoder",

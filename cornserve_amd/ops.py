@@ -255,6 +255,24 @@ def vit_index(item_meta: torch.Tensor, total_patches: int, max_units_per_item: i
     return VitIndex(window_index, reverse_index, src_rows, pos_ids, cos_sin)
 
 
+def pos_embed_interp(table: torch.Tensor, item_meta: torch.Tensor, total_patches: int, max_units_per_item: int,
+                     merge: int) -> torch.Tensor:
+    """Qwen3-VL position rows [total_patches, E] (bf16, patch order) interpolated from the learned side x side table."""
+    lib = _l.load()
+    _req(table, torch.bfloat16, "table")
+    _req(item_meta, torch.int32, "item_meta")
+    side = int(round(table.shape[0] ** 0.5))
+    if table.dim() != 2 or side * side != table.shape[0] or not table.is_contiguous():
+        raise ValueError("table must be a contiguous [side*side, E] tensor")
+    out = torch.empty((total_patches, table.shape[1]), dtype=torch.bfloat16, device=table.device)
+    _l.check(
+        lib.cs_pos_embed_interp(table.data_ptr(), side, table.shape[1], item_meta.data_ptr(), item_meta.shape[0],
+                                max_units_per_item, merge, out.data_ptr(), out.stride(0), _stream()),
+        "cs_pos_embed_interp",
+    )
+    return out
+
+
 def row_gather(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
     """out[i] = x[rows[i]] for a 2-D tensor with contiguous rows."""
     lib = _l.load()

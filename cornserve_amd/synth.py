@@ -152,6 +152,58 @@ def qwen2_linear_weight_keys(config) -> list[str]:
     return keys + ["merger.mlp.0.weight", "merger.mlp.2.weight"]
 
 
+# ------------------------------------------------------------------------------------------ Qwen3-VL
+def qwen3_vision_config(depth: int = 27, deepstack_visual_indexes=(8, 16, 24), out_hidden_size: int = 4096) -> SimpleNamespace:
+    """The Qwen3-VL-8B vision tower's hyper-parameters (only `vision_config` is read)."""
+    vc = SimpleNamespace(depth=depth, hidden_size=1152, intermediate_size=4304, num_heads=16, in_channels=3,
+                         patch_size=16, temporal_patch_size=2, spatial_merge_size=2, out_hidden_size=out_hidden_size,
+                         num_position_embeddings=2304, deepstack_visual_indexes=list(deepstack_visual_indexes),
+                         hidden_act="gelu_pytorch_tanh")
+    return SimpleNamespace(vision_config=vc, model_type="qwen3_vl")
+
+
+def qwen3_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
+    """fp32 state dict with the Qwen3-VL checkpoint's names (after `visual.` is stripped; Conv3d-shaped patch weight)."""
+    vc = config.vision_config
+    E, I, O = vc.hidden_size, vc.intermediate_size, vc.out_hidden_size
+    M = E * vc.spatial_merge_size**2
+    sd: dict[str, torch.Tensor] = {}
+
+    def mat(name, *shape):
+        sd[name] = normal(seed, name, shape, 0.02)
+
+    def ln(prefix, n):
+        sd[prefix + ".weight"] = normal(seed, prefix + ".weight", (n,), 0.02, 1.0)
+        sd[prefix + ".bias"] = normal(seed, prefix + ".bias", (n,), 0.02)
+
+    mat("patch_embed.proj.weight", E, vc.in_channels, vc.temporal_patch_size, vc.patch_size, vc.patch_size)
+    mat("patch_embed.proj.bias", E)
+    mat("pos_embed.weight", vc.num_position_embeddings, E)
+    for i in range(vc.depth):
+        p = f"blocks.{i}."
+        ln(p + "norm1", E)
+        ln(p + "norm2", E)
+        for name, n, k in (("attn.qkv", 3 * E, E), ("attn.proj", E, E), ("mlp.linear_fc1", I, E), ("mlp.linear_fc2", E, I)):
+            mat(p + name + ".weight", n, k)
+            mat(p + name + ".bias", n)
+    for prefix, width in [("merger.", E)] + [(f"deepstack_merger_list.{j}.", M) for j in range(len(vc.deepstack_visual_indexes))]:
+        ln(prefix + "norm", width)
+        mat(prefix + "linear_fc1.weight", M, M)
+        mat(prefix + "linear_fc1.bias", M)
+        mat(prefix + "linear_fc2.weight", O, M)
+        mat(prefix + "linear_fc2.bias", O)
+    return sd
+
+
+def qwen3_inputs(grids, seed: int = 0) -> tuple[list[torch.Tensor], list[torch.Tensor]]:
+    """One [t*h*w, 1536] fp32 N(0,1) tensor (patch 16) and one [1,3] int64 grid per item."""
+    px, gr = [], []
+    for i, (t, h, w) in enumerate(grids):
+        px.append(normal(seed, f"pixel_values.{i}", (t * h * w, 3 * 2 * 16 * 16)))
+        gr.append(torch.tensor([[t, h, w]], dtype=torch.int64))
+    return px, gr
+
+
 # --------------------------------------------------------------------------------------- Gemma-3 / SigLIP
 def gemma3_config(num_hidden_layers: int = 27, image_size: int = 896, text_hidden: int = 2560,
                   mm_tokens_per_image: int = 256) -> SimpleNamespace:

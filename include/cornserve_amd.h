@@ -154,8 +154,18 @@ int cs_row_gather(const void* in, int64_t in_stride_bytes, const int32_t* rows, 
  *   o[j] = x[j]*cos[l,j] - x[j+d/2]*sin[l,j];  o[j+d/2] = x[j]*sin[l,j] + x[j+d/2]*cos[l,j]
  * fp32 math, one bf16 rounding.  In place on the q and k column blocks of a packed [L, 3*heads*d]
  * QKV buffer.  cos_sin is the [L, d] table written by cs_vit_index (cos | sin, d/2 each).        */
+/* head_dim must be a multiple of 8 (72 for Qwen3-VL, qwen3_vl.py:218-219, takes an 8-byte-vector path).       */
 int cs_rope_qk(void* qkv, int64_t ld, const float* cos_sin, int32_t L, int32_t heads, int32_t head_dim,
                void* stream);
+
+/* Qwen3-VL learned position embedding, fast_pos_embed_interpolate at qwen3_vl.py:364-420: the side x side table
+ * (bf16 [side*side, E]) bilinearly interpolated at linspace(0, side-1, h) x linspace(0, side-1, w) for every item
+ * of item_meta (the records of cs_vit_seqlens_host: t, h/merge, w/merge, ..., first patch row), rows written in patch
+ * order (merge x merge blocks, repeated per frame) to out (bf16 [L, ldo]).  Same operation order and rounding points
+ * as the reference's tensor program (fp32 positions and weights, bf16 weights, bf16 products, one rounding of the
+ * sum).                                                                                               */
+int cs_pos_embed_interp(const void* table, int32_t side, int32_t E, const int32_t* item_meta, int32_t n_items,
+                        int32_t max_units_per_item, int32_t merge, void* out, int64_t ldo, void* stream);
 
 /* ------------------------------------------------------------------------------------------------
  * Variable-length non-causal attention: replaces flash_attn_varlen_func (qwen2_5_vl.py:110-120)

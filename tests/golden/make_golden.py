@@ -15,6 +15,8 @@ of cornserve_amd.synth, fp32, CPU, eager/sdpa attention.  Outputs:
                              output, per-row L2 norms, sum and abs-sum
     qwen2_vl_small.npz       2-block Qwen2-VL tower (width 1280), an image (1,16,16) and a video (2,8,12): every 8th
                              column of the [112,3584] output, per-row L2 norms, sum
+    qwen3_vl_small.npz       3-block Qwen3-VL tower (width 1152, deepstack after blocks 0 and 2, output width 1024), an
+                             image (1,12,20) and a video (2,8,8): every 4th column of the [92,3072] output, row norms, sum
     gemma3_small.npz         2-layer SigLIP (224x224, 256 tokens) + projector to 16 tokens x 640: full output
 """
 
@@ -136,6 +138,44 @@ def make_qwen2_vl_small() -> None:
     print("qwen2_vl_small.npz", out.shape, float(np.abs(out).mean()))
 
 
+def _hf_qwen3(cfg):
+    from transformers.models.qwen3_vl.configuration_qwen3_vl import Qwen3VLVisionConfig
+    from transformers.models.qwen3_vl.modeling_qwen3_vl import Qwen3VLVisionModel
+
+    vc = cfg.vision_config
+    hf_cfg = Qwen3VLVisionConfig(depth=vc.depth, hidden_size=vc.hidden_size, hidden_act=vc.hidden_act,
+                                 intermediate_size=vc.intermediate_size, num_heads=vc.num_heads, in_channels=vc.in_channels,
+                                 patch_size=vc.patch_size, spatial_merge_size=vc.spatial_merge_size,
+                                 temporal_patch_size=vc.temporal_patch_size, out_hidden_size=vc.out_hidden_size,
+                                 num_position_embeddings=vc.num_position_embeddings,
+                                 deepstack_visual_indexes=list(vc.deepstack_visual_indexes))
+    hf_cfg._attn_implementation = "sdpa"
+    return Qwen3VLVisionModel(hf_cfg).float().eval()
+
+
+def hf_qwen3_forward(cfg, sd, px, grid) -> torch.Tensor:
+    """[L/4, out * (1 + n_deepstack)]: the main output with the deepstack features behind it, as the reference
+    concatenates them (eric/models/qwen3_vl.py:300-311)."""
+    model = _hf_qwen3(cfg)
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys, inc
+    with torch.no_grad():
+        out = model(torch.cat(px), grid_thw=torch.cat(grid))
+    return torch.cat([out.pooler_output, *out.deepstack_features], dim=1).float()
+
+
+def make_qwen3_vl_small() -> None:
+    cfg = synth.qwen3_vision_config(depth=3, deepstack_visual_indexes=(0, 2), out_hidden_size=1024)
+    sd = synth.qwen3_state_dict(cfg, seed=6)
+    px, grid = synth.qwen3_inputs([(1, 12, 20), (2, 8, 8)], seed=6)
+    out = hf_qwen3_forward(cfg, sd, px, grid).numpy()
+    assert out.shape == ((240 + 128) // 4, 3 * 1024), out.shape
+    np.savez_compressed(HERE / "qwen3_vl_small.npz", sample=out[:, ::4].astype(np.float32),
+                        row_l2=np.linalg.norm(out.astype(np.float64), axis=1).astype(np.float32),
+                        total=np.float64(out.astype(np.float64).sum()), seed=np.int64(6))
+    print("qwen3_vl_small.npz", out.shape, float(np.abs(out).mean()))
+
+
 def make_gemma3_small() -> None:
     from transformers.models.gemma3.configuration_gemma3 import Gemma3Config, Gemma3TextConfig
     from transformers.models.gemma3.modeling_gemma3 import Gemma3MultiModalProjector
@@ -177,4 +217,5 @@ if __name__ == "__main__":
     make_index()
     make_qwen_cfg1()
     make_qwen2_vl_small()
+    make_qwen3_vl_small()
     make_gemma3_small()

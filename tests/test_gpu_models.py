@@ -222,6 +222,61 @@ def test_qwen2_vl_ragged_frames_and_fp8(dev):
     check(out[0], o2.forward(sd_dq, ocfg8, px, grid, dtype=torch.float32)[0], REL_FP8, "qwen2-vl fp8 vs de-quantised fp32 oracle")
 
 
+# ------------------------------------------------------------------------------------------ Qwen3-VL
+def build_qwen3(dev, depth, deepstack, out, seed, weight_format="bf16"):
+    from cornserve_amd.eric.models.qwen3_vl import Qwen3_VisionTransformer
+    from oracle import qwen3_vl as o3
+
+    cfg = synth.qwen3_vision_config(depth=depth, deepstack_visual_indexes=deepstack, out_hidden_size=out)
+    sd = synth.qwen3_state_dict(cfg, seed=seed)
+    model = Qwen3_VisionTransformer(cfg, weight_format=weight_format)
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys
+    ocfg = o3.Qwen3VisionConfig(depth=depth, deepstack_visual_indexes=list(deepstack), out_hidden_size=out)
+    return model.to(device=dev, dtype=torch.bfloat16).eval(), sd, ocfg, cfg
+
+
+def test_qwen3_vl_against_oracle_and_golden(dev, golden_dir):
+    from oracle import qwen3_vl as o3
+
+    model, sd, ocfg, _ = build_qwen3(dev, 3, (0, 2), 1024, seed=6)
+    px, grid = synth.qwen3_inputs([(1, 12, 20), (2, 8, 8)], seed=6)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    assert [tuple(o.shape) for o in out] == [(60, 3072), (32, 3072)] and out[0].dtype == torch.bfloat16
+    vid = model(Modality.VIDEO, "", {"pixel_values_videos": px[1:], "video_grid_thw": grid[1:]})
+    assert torch.equal(vid[0], out[1])                                   # items are independent
+    ref16 = o3.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
+    ref32 = o3.forward(sd, ocfg, px, grid, dtype=torch.float32)
+    for i in range(2):
+        check(out[i], ref16[i], REL_BF16, f"qwen3-vl item {i} vs bf16 oracle")
+        check(out[i], ref32[i], REL_BF16, f"qwen3-vl item {i} vs fp32 oracle")
+        for j in range(3):                                               # main output and each deepstack block
+            check(out[i][:, j * 1024:(j + 1) * 1024], ref32[i][:, j * 1024:(j + 1) * 1024], REL_BF16, f"item {i} block {j}")
+    gold = np.load(golden_dir / "qwen3_vl_small.npz")                    # Hugging Face fp32 output, every 4th column
+    check(torch.cat(out)[:, ::4], torch.from_numpy(gold["sample"]), REL_BF16, "qwen3-vl vs committed golden sample")
+
+
+def test_qwen3_vl_ragged_consecutive_deepstack_and_fp8(dev):
+    from oracle import qwen3_vl as o3
+    from oracle import qwen2_5_vl as oq5
+
+    # deepstack after consecutive blocks (each kept state must survive the next block's in-place updates) and none after the last
+    model, sd, ocfg, _ = build_qwen3(dev, 4, (0, 1, 2), 512, seed=7)
+    grids = [(1, 18, 14), (1, 2, 2), (1, 6, 34), (3, 4, 8)]
+    px, grid = synth.qwen3_inputs(grids, seed=7)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    ref = o3.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
+    assert [tuple(o.shape) for o in out] == [tuple(r.shape) for r in ref]
+    for i, (o, r) in enumerate(zip(out, ref)):
+        check(o, r, REL_BF16, f"qwen3-vl ragged item {i} {grids[i]}")
+    model8, sd8, ocfg8, cfg8 = build_qwen3(dev, 2, (0,), 512, seed=8, weight_format="fp8_e4m3")
+    keys = [k for k in sd8 if k.endswith(".weight") and sd8[k].dim() == 2 and not k.startswith(("pos_embed", "patch_embed"))]
+    sd_dq = oq5.dequantized_state_dict(sd8, keys)
+    px, grid = synth.qwen3_inputs([(2, 12, 20)], seed=8)
+    out = model8(Modality.VIDEO, "", {"pixel_values_videos": px, "video_grid_thw": grid})
+    check(out[0], o3.forward(sd_dq, ocfg8, px, grid, dtype=torch.float32)[0], REL_FP8, "qwen3-vl fp8 vs de-quantised fp32 oracle")
+
+
 def build_gemma(dev, layers, image_size, text_hidden, tokens, seed):
     from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
 

@@ -456,6 +456,57 @@ def test_attention_wide_score_range(ops, dev, d, rotary):
     close(got, attn_ref(qkv, cu, nh, d, ang), 2**-6, f"wide score range d={d} rotary={rotary}")
 
 
+@pytest.mark.parametrize("d,rotary", [(72, False), (80, True), (80, False), (64, False)])
+def test_attention_short_segment_same_bits_in_either_kernel(ops, dev, d, rotary):
+    """A segment of at most 64 rows takes the 64-row kernel when it is the batch's longest and the 128-row kernels
+    when a longer segment is in the batch: the result must not depend on that."""
+    nh = 16
+    cu_short, cu_both = [0, 40, 104], [0, 40, 104, 404]
+    L = cu_both[-1]
+    g = torch.Generator().manual_seed(5)
+    qkv = torch.randn((L, 3 * nh * d), generator=g).bfloat16().to(dev)
+    cs = None
+    if rotary:
+        ang = torch.rand((L, d // 2), generator=g) * 6.0
+        cs = torch.cat([ang.cos(), ang.sin()], dim=1).float().contiguous().to(dev)
+    H = nh * d
+    both = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], ops.attn_plan(np.array(cu_both, np.int32), dev), nh, d, d**-0.5, cs)
+    short = ops.attn_varlen(qkv[:104, :H], qkv[:104, H:2 * H], qkv[:104, 2 * H:], ops.attn_plan(np.array(cu_short, np.int32), dev),
+                            nh, d, d**-0.5, None if cs is None else cs[:104].contiguous())
+    assert torch.equal(both[:104], short)
+
+
+def test_rotary_head_dim_72(ops, dev):
+    """Qwen3-VL: head dim 72, rotary halves of 36 (the 8-byte-vector path of the in-place kernel)."""
+    nh, d, L = 16, 72, 333
+    qkv = rnd((L, 3 * nh * d), 1.0, 61, dev)
+    ang = torch.rand((L, d // 2), generator=torch.Generator().manual_seed(62)) * 6.0
+    cs = torch.cat([ang.cos(), ang.sin()], dim=1).float().contiguous().to(dev)
+    H = nh * d
+    out = ops.rope_qk_(qkv.clone(), cs, nh, d)
+    close(out[:, :H], oq.apply_rotary(qkv[:, :H].cpu().reshape(L, nh, d), ang).reshape(L, H), 2**-8, "rope q d=72")
+    close(out[:, H:2 * H], oq.apply_rotary(qkv[:, H:2 * H].cpu().reshape(L, nh, d), ang).reshape(L, H), 2**-8, "rope k d=72")
+    assert torch.equal(out[:, 2 * H:], qkv[:, 2 * H:])
+
+
+@pytest.mark.parametrize("grids", [[(1, 12, 20)], [(2, 8, 8), (1, 48, 48), (1, 2, 2), (3, 6, 90)]])
+def test_pos_embed_interp(ops, dev, grids):
+    from oracle import qwen3_vl as o3
+
+    side, E = 48, 1152
+    table = rnd((side * side, E), 0.02, 63)
+    g = np.array(grids, np.int64)
+    ref = o3.pos_embed_interpolate(table, g, 2)                   # bf16 table: the reference's rounding points
+    sl = ops.vit_seqlens_host(g, 2, 1 << 20)
+    meta = torch.from_numpy(sl.item_meta).to(dev)
+    got = ops.pos_embed_interp(table.to(dev), meta, sl.total_patches, sl.max_units_per_item, 2)
+    assert got.shape == ref.shape and got.dtype == torch.bfloat16
+    # identical operation order; a last-bit difference of an fp32 linspace position can move a bf16 weight
+    diff = (got.float().cpu() - ref.float()).abs()
+    assert diff.max().item() <= 2**-7 * ref.float().abs().max().item()
+    assert (diff > 0).float().mean().item() < 0.02
+
+
 def test_attention_fused_rotary_and_standalone_rotary(ops, dev):
     nh, d, cu = 16, 80, [0, 64, 128, 1024 + 128, 1024 + 128 + 37]
     L = cu[-1]

@@ -133,3 +133,27 @@ def test_qwen2_vl_class_surface():
         model._ensure_packed()
     with pytest.raises(ValueError):
         Qwen2VisionTransformer(cfg, weight_format="int4")
+
+
+def test_qwen3_vl_class_surface():
+    from cornserve_amd import synth
+    from cornserve_amd.eric.models.qwen3_vl import Qwen3_VisionTransformer
+    from cornserve_amd.eric.models.registry import MODEL_REGISTRY
+
+    cfg = synth.qwen3_vision_config(depth=2, deepstack_visual_indexes=(0,))
+    model = Qwen3_VisionTransformer(cfg)
+    sd = synth.qwen3_state_dict(cfg, seed=0)          # Conv3d-shaped patch weight, as in the checkpoint
+    inc = model.load_state_dict(sd, strict=False)
+    assert not inc.missing_keys and not inc.unexpected_keys
+    assert model.patch_embed.proj.weight.shape == (1152, 1536)
+    assert model.chunk_shape == (1, 4096 * 2)
+    for key in ("qwen3_vl", "qwen3_vl_moe"):
+        entry = MODEL_REGISTRY[key]
+        assert entry.module == "qwen3_vl" and entry.class_name == "Qwen3_VisionTransformer"
+        assert entry.weight.required_prefixes == ["model.visual."]
+    with pytest.raises(RuntimeError):
+        model._ensure_packed()
+    bad = synth.qwen3_vision_config(depth=1)
+    bad.vision_config.hidden_act = "relu6"
+    with pytest.raises(NotImplementedError):
+        Qwen3_VisionTransformer(bad)

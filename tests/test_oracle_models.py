@@ -176,3 +176,60 @@ def test_qwen2_vl_pieces():
     px2[0][16:] += 1.0                                                           # change the second frame group only
     pert = o2.forward(sd, ocfg, px2, grid)
     assert torch.equal(pert[0][:4], both[0][:4]) and not torch.allclose(pert[0][4:], both[0][4:])
+
+
+# ------------------------------------------------------------------------------------------ Qwen3-VL
+def _qwen3_small(depth=3, deepstack=(0, 2), out=1024, seed=6):
+    from oracle import qwen3_vl as o3
+
+    cfg = synth.qwen3_vision_config(depth=depth, deepstack_visual_indexes=deepstack, out_hidden_size=out)
+    ocfg = o3.Qwen3VisionConfig(depth=depth, deepstack_visual_indexes=list(deepstack), out_hidden_size=out)
+    return o3, cfg, ocfg, synth.qwen3_state_dict(cfg, seed=seed)
+
+
+def test_qwen3_vl_against_golden(golden_dir):
+    gold = np.load(golden_dir / "qwen3_vl_small.npz")
+    o3, cfg, ocfg, sd = _qwen3_small(seed=int(gold["seed"]))
+    px, grid = synth.qwen3_inputs([(1, 12, 20), (2, 8, 8)], seed=int(gold["seed"]))
+    out = o3.forward(sd, ocfg, px, grid, dtype=torch.float32)
+    assert [tuple(o.shape) for o in out] == [(60, 3072), (32, 3072)]      # main + two deepstack blocks of 1024
+    o = torch.cat(out).numpy()
+    assert np.abs(o[:, ::4] - gold["sample"]).max() <= 2e-4 * np.abs(gold["sample"]).max()
+    assert np.allclose(np.linalg.norm(o.astype(np.float64), axis=1), gold["row_l2"], rtol=1e-4)
+
+
+def test_qwen3_vl_live_against_hugging_face():
+    pytest.importorskip("transformers.models.qwen3_vl.modeling_qwen3_vl")
+    import sys
+    from pathlib import Path
+    sys.path.insert(0, str(Path(__file__).parent / "golden"))
+    import make_golden
+
+    o3, cfg, ocfg, sd = _qwen3_small(depth=2, deepstack=(1,), out=512, seed=10)
+    px, grid = synth.qwen3_inputs([(1, 6, 10), (3, 4, 4)], seed=10)
+    ref = make_golden.hf_qwen3_forward(cfg, sd, px, grid)
+    got = torch.cat(o3.forward(sd, ocfg, px, grid, dtype=torch.float32))
+    assert got.shape == ref.shape == ((60 + 48) // 4, 1024)
+    assert (got - ref).abs().max().item() <= 2e-4 * ref.abs().max().item()
+
+
+def test_qwen3_vl_position_interpolation_closed_forms():
+    from oracle import qwen3_vl as o3
+
+    side, E = 6, 8
+    table = torch.arange(side * side * E, dtype=torch.float32).reshape(side * side, E)
+    # a grid of the table's own size samples it exactly; rows come out in 2x2-block-major order
+    got = o3.pos_embed_interpolate(table, np.array([[1, side, side]]), merge=2)
+    order = [(by * 2 + my) * side + bx * 2 + mx for by in range(3) for bx in range(3) for my in range(2) for mx in range(2)]
+    assert torch.equal(got, table[order])
+    # two points per side: the four corners
+    got = o3.pos_embed_interpolate(table, np.array([[1, 2, 2]]), merge=2)
+    assert torch.equal(got, table[[0, side - 1, side * (side - 1), side * side - 1]])
+    # a linear table is reproduced by bilinear interpolation at any resolution
+    yy, xx = torch.meshgrid(torch.arange(side, dtype=torch.float32), torch.arange(side, dtype=torch.float32), indexing="ij")
+    lin = (3.0 * yy + 0.5 * xx).reshape(-1, 1).repeat(1, E)
+    got = o3.pos_embed_interpolate(lin, np.array([[2, 4, 10]]), merge=2)
+    hs, ws = torch.linspace(0, side - 1, 4), torch.linspace(0, side - 1, 10)
+    want = [3.0 * hs[by * 2 + my] + 0.5 * ws[bx * 2 + mx] for by in range(2) for bx in range(5) for my in range(2) for mx in range(2)]
+    assert got.shape == (80, E) and torch.allclose(got[:40, 0], torch.stack(want), atol=1e-5)
+    assert torch.equal(got[:40], got[40:])                       # repeated per frame
