@@ -116,6 +116,11 @@ class QwenVisionBase(EricModel):
     `forward_device`, `chunk_shape` and the attributes patch_size, temporal_patch_size, spatial_merge_size,
     in_channels, weight_format and patch_embed."""
 
+    # what the checkpoint's image processor normalises with (preprocessor_config.json): CLIP statistics for
+    # Qwen2-VL and Qwen2.5-VL; subclasses override
+    image_mean: tuple = frame_ops.CLIP_MEAN
+    image_std: tuple = frame_ops.CLIP_STD
+
     def __init__(self) -> None:
         super().__init__()
         self._packed: dict | None = None
@@ -167,10 +172,10 @@ class QwenVisionBase(EricModel):
         the Hugging Face processor the reference runs (:488-512) produces from the same frames, with rescale,
         normalise and the patch layout done on the GPU."""
         p, m, tps, dev = self.patch_size, self.spatial_merge_size, self.temporal_patch_size, self.device
-        key = ("byte_table", arithmetic)
+        key = ("byte_table", arithmetic)   # (a model's mean / std are fixed)
         pk = self._ensure_packed()
         if key not in pk:
-            pk[key] = frame_ops.byte_table(arithmetic=arithmetic).to(dev)
+            pk[key] = frame_ops.byte_table(self.image_mean, self.image_std, arithmetic=arithmetic).to(dev)
         items, grids = [], []
         for f in frames:
             f = torch.as_tensor(f)
@@ -418,12 +423,14 @@ class FrameModalityProcessor(BaseModalityProcessor):
     PIL bicubic resampling) and emits `pixel_frames` / `pixel_frames_videos`; rescale, normalise and the patch
     layout run on the GPU inside the model's forward.  Needs no model files."""
 
-    def __init__(self, model_id: str, min_pixels: int = 56 * 56, max_pixels: int = 14 * 14 * 4 * 1280) -> None:
+    def __init__(self, model_id: str, min_pixels: int = 56 * 56, max_pixels: int = 14 * 14 * 4 * 1280,
+                 factor: int = 28) -> None:
+        """`factor` = patch size x merge size of the encoder (28 for Qwen2-VL / Qwen2.5-VL, 32 for Qwen3-VL)."""
         super().__init__(model_id=model_id)
-        self.min_pixels, self.max_pixels = min_pixels, max_pixels
+        self.min_pixels, self.max_pixels, self.factor = min_pixels, max_pixels, factor
 
     def _resized(self, frames) -> torch.Tensor:
-        return torch.from_numpy(frame_ops.resize_frames(frames, 28, self.min_pixels, self.max_pixels))
+        return torch.from_numpy(frame_ops.resize_frames(frames, self.factor, self.min_pixels, self.max_pixels))
 
     def get_image_processor(self) -> Callable | None:
         return lambda image: {"pixel_frames": self._resized(image)}

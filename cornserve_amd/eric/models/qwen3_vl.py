@@ -88,6 +88,9 @@ class _Merger(nn.Module):
 
 
 class Qwen3_VisionTransformer(QwenVisionBase):
+    image_mean = (0.5, 0.5, 0.5)   # the Qwen3-VL checkpoints' preprocessor_config.json
+    image_std = (0.5, 0.5, 0.5)
+
     def __init__(self, config: Any, weight_format: str = "bf16") -> None:
         super().__init__()
         vc = config.vision_config if hasattr(config, "vision_config") else config

@@ -269,6 +269,15 @@ def test_qwen3_vl_ragged_consecutive_deepstack_and_fp8(dev):
     assert [tuple(o.shape) for o in out] == [tuple(r.shape) for r in ref]
     for i, (o, r) in enumerate(zip(out, ref)):
         check(o, r, REL_BF16, f"qwen3-vl ragged item {i} {grids[i]}")
+    # uint8 frames: patch 16, the checkpoints' mean = std = 0.5
+    from oracle import qwen_preprocess as qp
+    frames = np.random.default_rng(7).integers(0, 256, (3, 64, 96, 3), dtype=np.uint8)
+    table = qp.normalization_table((0.5, 0.5, 0.5), (0.5, 0.5, 0.5), arithmetic="fused")
+    fpx, fgrid = qp.patchify_frames(frames, table, patch=16)
+    assert fgrid == (2, 4, 6) and fpx.shape == (48, 1536)
+    a = model(Modality.VIDEO, "", {"pixel_values_videos": [torch.from_numpy(fpx)], "video_grid_thw": [torch.tensor([fgrid])]})
+    b = model(Modality.VIDEO, "", {"pixel_frames_videos": [torch.from_numpy(frames)]})
+    assert torch.equal(a[0], b[0])
     model8, sd8, ocfg8, cfg8 = build_qwen3(dev, 2, (0,), 512, seed=8, weight_format="fp8_e4m3")
     keys = [k for k in sd8 if k.endswith(".weight") and sd8[k].dim() == 2 and not k.startswith(("pos_embed", "patch_embed"))]
     sd_dq = oq5.dequantized_state_dict(sd8, keys)
