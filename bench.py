@@ -18,6 +18,8 @@ with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
                         the instrumented pass applied to the timed step
   host_inputs           the same step with the batch handed over as fp32 host tensors (PCIe-inclusive)
   host_inputs_uint8_frames  the same step from resized uint8 frames on the host (PCIe-inclusive; GPU patch layout)
+  (--workload cfg3 | cfg4 | cfg5 | qwen2_vl | qwen3_vl prints a shorter line -- throughput only -- for the other
+  configurations; the default, cfg2, is the headline benchmark)
   cpu_baseline          the CPU oracle (a port of the reference's algorithm, plain PyTorch) timed on this
                         host's cores on a bounded sample of the same workload
 """
@@ -119,6 +121,76 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0) -> dict:
     }
 
 
+OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl")
+
+
+def other_workload(name: str, steps: int, warmup: int, dev) -> dict:
+    """Whole-forward throughput of one of the other configurations (inputs resident in HBM as bf16, synthetic
+    weights): configs[2] (SigLIP / Gemma-3, 4 x 896x896), configs[3] (16 ragged images), configs[4] (fp8 weights,
+    two 8-frame videos), and the sibling encoders Qwen2-VL / Qwen3-VL on 8 images of 32 x 32 patches."""
+    import numpy as np
+    import torch
+
+    from cornserve_amd import synth
+
+    def qwen_like(model_cls, cfg, sd, grids, in_dim, **kw):
+        model = model_cls(cfg, **kw)
+        model.load_state_dict(sd, strict=False)
+        model = model.to(device=dev, dtype=torch.bfloat16).eval()
+        L = sum(t * h * w for t, h, w in grids)
+        px = synth.normal(0, "bench.pixel_values", (L, in_dim)).to(device=dev, dtype=torch.bfloat16)
+        g = np.array(grids, np.int64)
+        return (lambda: model.forward_device(px, g)), L, len(grids)
+
+    if name == "cfg3":
+        from cornserve_amd.eric.api import Modality
+        from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
+
+        cfg = synth.gemma3_config()
+        model = Gemma3VisionEncoder(cfg).to(device=dev, dtype=torch.bfloat16).eval()
+        synth.load_gemma3(model, synth.gemma3_state_dict(cfg, seed=0), "a")
+        px, crops = synth.gemma3_inputs(4, 896, seed=0)
+        batch = {"pixel_values": [p.to(device=dev, dtype=torch.bfloat16) for p in px], "num_crops": crops}
+        run, L, items = (lambda: model.forward(Modality.IMAGE, "a", batch)), 4 * 4096, 4
+        what = "configs[2]: SigLIP-so400m tower (27 layers) + Gemma-3 projector, 4 x 896x896 images = 16384 patches"
+    elif name in ("cfg4", "cfg5"):
+        from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
+
+        cfg = synth.qwen_vision_config()
+        sd = synth.qwen_state_dict(cfg, seed=0)
+        if name == "cfg4":
+            run, L, items = qwen_like(Qwen2_5_VisionTransformer, cfg, sd, synth.ragged_grids(16, seed=4), 1176)
+            what = f"configs[3]: Qwen2.5-VL-7B ViT, 16 images with sides drawn from 224..1344 = {L} patches"
+        else:
+            run, L, items = qwen_like(Qwen2_5_VisionTransformer, cfg, sd, [(8, 24, 42)] * 2, 1176, weight_format="fp8_e4m3")
+            what = "configs[4]: Qwen2.5-VL-7B ViT with fp8-e4m3 weights, 2 videos of 8 frame pairs x 24 x 42 = 16128 patches"
+    elif name == "qwen2_vl":
+        from cornserve_amd.eric.models.qwen2_vl import Qwen2VisionTransformer
+
+        cfg = synth.qwen2_vision_config()
+        run, L, items = qwen_like(Qwen2VisionTransformer, cfg, synth.qwen2_state_dict(cfg, seed=0), [(1, 32, 32)] * 8, 1176)
+        what = "Qwen2-VL-7B ViT (32 blocks, full attention per frame), 8 x 448x448 images = 8192 patches"
+    else:
+        from cornserve_amd.eric.models.qwen3_vl import Qwen3_VisionTransformer
+
+        cfg = synth.qwen3_vision_config()
+        run, L, items = qwen_like(Qwen3_VisionTransformer, cfg, synth.qwen3_state_dict(cfg, seed=0), [(1, 32, 32)] * 8, 1536)
+        what = "Qwen3-VL-8B ViT (27 blocks, 3 deepstack mergers), 8 x 512x512 images = 8192 patches"
+    with torch.inference_mode():
+        for _ in range(warmup):
+            run()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            run()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+    return {"metric": "encoder patches/sec on 1 MI355X", "value": L * steps / dt, "unit": "patches/s", "n_gpus": 1,
+            "steps": steps, "warmup": warmup, "ms_per_step": dt / steps * 1e3, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic (seeded inputs and random-init weights)",
+            "config": {"workload": what, "patches": L, "items": items}}
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -128,6 +200,9 @@ def main() -> None:
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (counter calibration for rocprofv3 --pmc runs)")
     ap.add_argument("--cpu-sample-images", type=int, default=8)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg2", *OTHER_WORKLOADS],
+                    help="cfg2 (default) is the headline benchmark; the others print a shorter line for one of the "
+                         "other configurations / encoders built on the same kernels")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (every image is independent; more GPUs would each "
@@ -142,6 +217,9 @@ def main() -> None:
 
     lib.load()
     dev = torch.device("cuda:0")
+    if args.workload != "cfg2":
+        print(json.dumps(other_workload(args.workload, args.steps, args.warmup, dev)))
+        return
     cfg = synth.qwen_vision_config()
     sd = synth.qwen_state_dict(cfg, seed=0)
     model = Qwen2_5_VisionTransformer(cfg)
