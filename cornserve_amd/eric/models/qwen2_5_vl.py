@@ -314,7 +314,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         win = self.window_size // merge // self.patch_size
         dev = self.device
         sl = ops.vit_seqlens_host(grid_thw, merge, win)
-        meta = torch.from_numpy(sl.item_meta).to(dev, non_blocking=True)
+        meta = ops.host_to_device(sl.item_meta, dev)
         ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, merge, win, self._ensure_packed()["inv_freq"])
         return ix, ops.attn_plan(sl.cu_window, dev), ops.attn_plan(sl.cu_full, dev), sl.total_patches
 

@@ -130,7 +130,7 @@ class Qwen2VisionTransformer(QwenVisionBase):
         merge = self.spatial_merge_size
         no_window = 1 << 20
         sl = ops.vit_seqlens_host(grid_thw, merge, no_window)
-        meta = torch.from_numpy(sl.item_meta).to(dev, non_blocking=True)
+        meta = ops.host_to_device(sl.item_meta, dev)
         ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, merge, no_window, pk["inv_freq"])
         plan = ops.attn_plan(sl.cu_full, dev)
         L = sl.total_patches

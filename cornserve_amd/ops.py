@@ -28,6 +28,17 @@ def _stream() -> int:
     return torch.cuda.current_stream().cuda_stream
 
 
+def host_to_device(a: np.ndarray, device: torch.device) -> torch.Tensor:
+    """Small host array -> device tensor through pinned memory, so that the copy is asynchronous and the host
+    can keep enqueueing work (a copy from pageable memory waits for the stream)."""
+    a = np.ascontiguousarray(a)
+    if a.size == 0:
+        return torch.from_numpy(a.copy()).to(device)
+    staged = torch.empty(a.shape, dtype=torch.from_numpy(a[:0].reshape(-1)).dtype, pin_memory=True)
+    staged.numpy()[...] = a
+    return staged.to(device, non_blocking=True)
+
+
 def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
@@ -327,8 +338,7 @@ def attn_plan(cu_seqlens_host: np.ndarray, device: torch.device) -> AttnPlan:
     n_work = ctypes.c_int32(0)
     _l.check(lib.cs_attn_work_host(cu.ctypes.data, n_seg, bq, work.ctypes.data, cap, ctypes.byref(n_work)),
              "cs_attn_work_host")
-    w = torch.from_numpy(work[: n_work.value].copy()).to(device, non_blocking=True)
-    return AttnPlan(w, n_work.value, max_seqlen)
+    return AttnPlan(host_to_device(work[: n_work.value], device), n_work.value, max_seqlen)
 
 
 def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan, heads: int, head_dim: int,
