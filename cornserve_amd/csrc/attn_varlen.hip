@@ -64,8 +64,107 @@ struct AttnArgs {
   int n_work, heads, chunk, n_chunks_x;
 };
 
+// ---- pieces shared by the attention kernels.  A wave owns 32 query rows (lane % 32 = query, lane / 32 = which
+//      half of the 8-row groups of a 32x32 MFMA result it holds) and works on tiles of BKV = 64 keys.
+
+// S^T = K.Q^T for one key tile in LDS (row stride RS bytes), keys past `nvalid` masked to -inf.
+template <int KS, int RS>
+CS_DEVICE void score_tile(f32x16_t (&sacc)[2], const char* k_tile, const bf16x8_t (&qf)[KS], int nvalid, int fr, int hf) {
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) sacc[kt][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const bf16x8_t kf = *(const bf16x8_t*)(k_tile + (kt * 32 + fr) * RS + (2 * ks + hf) * 16);
+      sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kt], 0, 0, 0);
+    }
+  }
+  if (nvalid < BKV) {  // uniform: only the last tile of a segment can be partial
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
+        if (key >= nvalid) sacc[kt][r] = -INFINITY;
+      }
+  }
+}
+
+// Online softmax of one tile's scores -> P (bf16 fragments for the P.V product).
+// Lazy reference maximum: P = exp2((s - m_run) * scale) with an m_run that is only raised when some query of the
+// wave sees a score more than LAZY_LOG2 (in log2 units) above it.  P then ranges up to 2^LAZY_LOG2 instead of 1,
+// which fp32 accumulation and bf16's exponent range do not care about, the final division by the denominator
+// (built from the same P) cancels the reference, and the rescale of O -- DT*16 multiplies and an exponential per
+// tile -- runs only in the first tiles of a segment.  m_run starts at -inf, so the first tile always sets it to
+// its own maximum.  With L_FROM_MFMA the denominator is not summed here (see attn_full_kernel).
+// FIRST_TILE: the caller knows that nothing has been accumulated yet (O = 0, m_run = -inf): no rescale to consider.
+template <int DT, bool L_FROM_MFMA, bool FIRST_TILE = false>
+CS_DEVICE void softmax_tile(const f32x16_t (&sacc)[2], bf16x8_t (&pf)[2][2], f32x16_t (&oacc)[DT], float& m_run,
+                            float& l_run, float sl2) {
+  float mx = -INFINITY;
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  constexpr float LAZY_LOG2 = 6.0f;
+  float alpha = 1.0f;
+  if constexpr (FIRST_TILE) {
+    m_run = mx;
+  } else if (__any((mx - m_run) * sl2 > LAZY_LOG2)) {
+    const float m_new = fmaxf(m_run, mx);
+    alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
+#pragma unroll
+    for (int t = 0; t < DT; ++t)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
+    m_run = m_new;
+  }
+  const float mb = m_run * sl2;
+  float psum = 0.f;
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * sl2 - mb);
+      if constexpr (!L_FROM_MFMA) psum += pv;
+      pf[kt][r >> 3][r & 7] = f2bf(pv);
+    }
+  if constexpr (!L_FROM_MFMA) {
+    psum += __shfl_xor(psum, 32, 64);
+    l_run = l_run * alpha + psum;
+  }
+}
+
+// O^T[d][q] / l -> out[q][d0 ...]: a lane owns query `qi` and 4 consecutive d per 8-row group.  With L_FROM_MFMA the
+// denominator is row D of O^T (block D/32, row D%32 = 8g + 4*half + e), held by the lanes of one half.
+template <int D, int DT, bool L_FROM_MFMA>
+CS_DEVICE void write_output(const f32x16_t (&oacc)[DT], float l_run, bf16_t* orow, bool valid, int hf) {
+  if constexpr (L_FROM_MFMA) {
+    constexpr int RR = D % 32, G_L = RR / 8, HF_L = (RR % 8) / 4, E_L = RR % 4;
+    const float mine = oacc[D / 32][4 * G_L + E_L];
+    const float other = __shfl_xor(mine, 32, 64);
+    l_run = hf == HF_L ? mine : other;
+  }
+  if (!valid) return;
+  const float inv = 1.0f / l_run;
+#pragma unroll
+  for (int t = 0; t < DT; ++t)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int d0 = t * 32 + 8 * g + 4 * hf;
+      if (d0 < D) {
+        bf16x4_t o;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
+        *(bf16x4_t*)(orow + d0) = o;
+      }
+    }
+}
+
 template <int D, int NWAVES, bool ROPE, int HPW>
-__global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(NWAVES * 64, 2) void attn_kernel(const AttnArgs a) {
   constexpr int NT = NWAVES * 64;
   constexpr int BQ = NWAVES * 32;
   constexpr int KS = (D + 15) / 16;    // MFMA k-steps over the head dim
@@ -165,31 +264,9 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
     l_run = 0.f;
   };
   const bool wave_active = wave * 32 < nq;
-  // O^T[d][q] / l -> out[q][head*D + d]; lane owns query wave*32 + fr and 4 consecutive d per group.
   auto write_out = [&]() {
-    if constexpr (L_FROM_MFMA) {
-      constexpr int RR = D % 32, G_L = RR / 8, HF_L = (RR % 8) / 4, E_L = RR % 4;
-      const float mine = oacc[D / 32][4 * G_L + E_L];
-      const float other = __shfl_xor(mine, 32, 64);
-      l_run = hf == HF_L ? mine : other;
-    }
     const int qi = wave * 32 + fr;
-    if (qi < nq) {
-      const float inv = 1.0f / l_run;
-      bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
-#pragma unroll
-      for (int t = 0; t < DT; ++t)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const int d0 = t * 32 + 8 * g + 4 * hf;
-          if (d0 < D) {
-            bf16x4_t o;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
-            *(bf16x4_t*)(orow + d0) = o;
-          }
-        }
-    }
+    write_output<D, DT, L_FROM_MFMA>(oacc, l_run, a.out + (int64_t)(q0 + min(qi, nq - 1)) * a.ldo + hoff, qi < nq, hf);
   };
   bf16x8_t qf[KS];
   auto load_q_frags = [&]() {
@@ -199,58 +276,12 @@ __global__ __launch_bounds__(NWAVES * 64) void attn_kernel(const AttnArgs a) {
 
   // One K/V tile in LDS (nvalid keys): S^T = K Q^T, online softmax, O^T += V^T P^T.
   auto compute_tile = [&](int nvalid, auto first_c) {
-    constexpr bool FIRST_TILE = decltype(first_c)::value;  // nothing accumulated yet: no rescale of O
     f32x16_t sacc[2];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) sacc[kt][r] = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const bf16x8_t kf = *(const bf16x8_t*)(k_lds + (kt * 32 + fr) * RS + (2 * ks + hf) * 16);
-        sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kt], 0, 0, 0);
-      }
-    }
-    // mask keys past the segment end, running max
-    float mx = -INFINITY;
-    if (nvalid < BKV) {  // uniform: only a segment's last tile can be partial
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-          if (key >= nvalid) sacc[kt][r] = -INFINITY;
-        }
-    }
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m_run, mx);
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * a.scale_log2e);
-    const float mb = m_new * a.scale_log2e;
-    float psum = 0.f;
     bf16x8_t pf[2][2];
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * a.scale_log2e - mb);
-        if constexpr (!L_FROM_MFMA) psum += pv;
-        pf[kt][r >> 3][r & 7] = f2bf(pv);
-      }
-    if constexpr (!L_FROM_MFMA) {
-      psum += __shfl_xor(psum, 32, 64);
-      l_run = l_run * alpha + psum;
-    }
-    m_run = m_new;
+    score_tile<KS, RS>(sacc, k_lds, qf, nvalid, fr, hf);
+    softmax_tile<DT, L_FROM_MFMA, decltype(first_c)::value>(sacc, pf, oacc, m_run, l_run, a.scale_log2e);
 #pragma unroll
     for (int t = 0; t < DT; ++t) {
-      if (!FIRST_TILE) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
-      }
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
@@ -566,62 +597,9 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
       const char* kd = k_buf(buf);
       const char* vd = v_buf(buf);
       f32x16_t sacc[2];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[kt][r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8_t kf = *(const bf16x8_t*)(kd + (kt * 32 + fr) * RS + (2 * ks + hf) * 16);
-          sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kt], 0, 0, 0);
-        }
-      }
-      if (nvalid < BKV) {  // only the last tile of a segment can be partial
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-            if (key >= nvalid) sacc[kt][r] = -INFINITY;
-          }
-      }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      // Lazy reference maximum: P = exp2((s - m_run) * scale) with an m_run that is only raised when some
-      // query of the wave sees a score more than LAZY_LOG2 (in log2 units) above it.  P then ranges up to
-      // 2^LAZY_LOG2 instead of 1, which fp32 accumulation and bf16's exponent range do not care about, the
-      // final division by the denominator (built from the same P) cancels the reference, and the rescale of
-      // O -- DT*16 multiplies and an exponential per tile -- runs only in the first tiles of a segment.
-      constexpr float LAZY_LOG2 = 6.0f;
-      float alpha = 1.0f;
-      if (__any((mx - m_run) * sl2 > LAZY_LOG2)) {  // m_run starts at -inf: always taken for the first tile
-        const float m_new = fmaxf(m_run, mx);
-        alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
-#pragma unroll
-        for (int t = 0; t < DT; ++t)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[t][r] *= alpha;
-        m_run = m_new;
-      }
-      const float mb = m_run * sl2;
-      float psum = 0.f;
       bf16x8_t pf[2][2];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * sl2 - mb);
-          if constexpr (!L_FROM_MFMA) psum += pv;
-          pf[kt][r >> 3][r & 7] = f2bf(pv);
-        }
-      if constexpr (!L_FROM_MFMA) {
-        psum += __shfl_xor(psum, 32, 64);
-        l_run = l_run * alpha + psum;
-      }
+      score_tile<KS, RS>(sacc, kd, qf, nvalid, fr, hf);
+      softmax_tile<DT, L_FROM_MFMA>(sacc, pf, oacc, m_run, l_run, sl2);
 #pragma unroll
       for (int t = 0; t < DT; ++t) {
 #pragma unroll
@@ -637,30 +615,8 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
     __syncthreads();
   }
 
-  if constexpr (L_FROM_MFMA) {
-    // row D of O^T: block D/32, row D%32 = 8g + 4*hf + e; the lanes of the owning half hold it for their query
-    constexpr int RR = D % 32, G_L = RR / 8, HF_L = (RR % 8) / 4, E_L = RR % 4;
-    const float mine = oacc[D / 32][4 * G_L + E_L];
-    const float other = __shfl_xor(mine, 32, 64);
-    l_run = hf == HF_L ? mine : other;
-  }
   const int qi = wave * 32 + fr;
-  if (qi < nq) {
-    const float inv = 1.0f / l_run;
-    bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
-#pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int d0 = t * 32 + 8 * g + 4 * hf;
-        if (d0 < D) {
-          bf16x4_t o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
-          *(bf16x4_t*)(orow + d0) = o;
-        }
-      }
-  }
+  write_output<D, DT, L_FROM_MFMA>(oacc, l_run, a.out + (int64_t)(q0 + min(qi, nq - 1)) * a.ldo + hoff, qi < nq, hf);
 }
 
 // Full attention without rotary (SigLIP): K and V tiles go global -> LDS directly (buffer_load ... lds: no
@@ -848,57 +804,9 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
       const char* kd = k_buf(buf);
       const char* vd = v_buf(buf);
       f32x16_t sacc[2];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[kt][r] = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const bf16x8_t kf = *(const bf16x8_t*)(kd + (kt * 32 + fr) * RS + (2 * ks + hf) * 16);
-          sacc[kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, qf[ks], sacc[kt], 0, 0, 0);
-        }
-      }
-      if (nvalid < BKV) {  // only the last tile of a segment can be partial
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = kt * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-            if (key >= nvalid) sacc[kt][r] = -INFINITY;
-          }
-      }
-      float mx = -INFINITY;
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sacc[kt][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      constexpr float LAZY_LOG2 = 6.0f;   // lazily raised reference maximum: see attn_full_kernel
-      float alpha = 1.0f;
-      if (__any((mx - m_run) * sl2 > LAZY_LOG2)) {
-        const float m_new = fmaxf(m_run, mx);
-        alpha = __builtin_amdgcn_exp2f((m_run - m_new) * sl2);
-#pragma unroll
-        for (int tt = 0; tt < DT; ++tt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) oacc[tt][r] *= alpha;
-        m_run = m_new;
-      }
-      const float mb = m_run * sl2;
-      float psum = 0.f;
       bf16x8_t pf[2][2];
-#pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float pv = __builtin_amdgcn_exp2f(sacc[kt][r] * sl2 - mb);
-          if constexpr (!L_FROM_MFMA) psum += pv;
-          pf[kt][r >> 3][r & 7] = f2bf(pv);
-        }
-      if constexpr (!L_FROM_MFMA) {
-        psum += __shfl_xor(psum, 32, 64);
-        l_run = l_run * alpha + psum;
-      }
+      score_tile<KS, RS>(sacc, kd, qf, nvalid, fr, hf);
+      softmax_tile<DT, L_FROM_MFMA>(sacc, pf, oacc, m_run, l_run, sl2);
       // V^T fragments (see read_vt_frag for the addressing).  The transposing reads are written in assembly: as
       // an intrinsic, the compiler takes them for possible readers of the LDS bytes that the direct loads in
       // flight will write and puts a wait for ALL outstanding loads in front of them -- the tiles requested
@@ -925,30 +833,10 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
     buf = buf == 2 ? 0 : buf + 1;
   }
 
-  if constexpr (L_FROM_MFMA) {
-    constexpr int RR = D % 32, G_L = RR / 8, HF_L = (RR % 8) / 4, E_L = RR % 4;
-    const float mine = oacc[D / 32][4 * G_L + E_L];
-    const float other = __shfl_xor(mine, 32, 64);
-    l_run = hf == HF_L ? mine : other;
-  }
   const int qi = wave * 32 + fr;
-  if (qi < nq) {
-    const float inv = 1.0f / l_run;
-    bf16_t* orow = a.out + (int64_t)(q0 + qi) * a.ldo + hoff;
-#pragma unroll
-    for (int t = 0; t < DT; ++t)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const int d0 = t * 32 + 8 * g + 4 * hf;
-        if (d0 < D) {
-          bf16x4_t o;
-#pragma unroll
-          for (int e = 0; e < 4; ++e) o[e] = f2bf(oacc[t][4 * g + e] * inv);
-          *(bf16x4_t*)(orow + d0) = o;
-        }
-      }
-  }
+  write_output<D, DT, L_FROM_MFMA>(oacc, l_run, a.out + (int64_t)(q0 + min(qi, nq - 1)) * a.ldo + hoff, qi < nq, hf);
 }
+
 
 template <int D>
 int launch_attn_full_direct(const AttnArgs& a, dim3 grid, hipStream_t stream) {
