@@ -22,6 +22,7 @@ rotates while staging, so rotary runs as its own in-place kernel and attention t
 from __future__ import annotations
 
 import math
+from collections.abc import Callable
 from typing import Any
 
 import numpy as np
@@ -29,7 +30,8 @@ import torch
 import torch.nn as nn
 
 from cornserve_amd import ops
-from cornserve_amd.eric.models.qwen2_5_vl import QwenVisionBase, _Attn, _Linear, _no_mark
+from cornserve_amd.eric.models.base import BaseModalityProcessor
+from cornserve_amd.eric.models.qwen2_5_vl import FrameModalityProcessor, QwenVisionBase, _Attn, _Linear, _no_mark  # noqa: F401
 from cornserve_amd.eric.models.qwen2_vl import _LayerNorm
 
 _ACTIVATIONS = {"gelu_pytorch_tanh": ops.EPI_GELU_TANH, "gelu": ops.EPI_GELU_ERF, "quick_gelu": ops.EPI_QUICK_GELU}
@@ -235,3 +237,35 @@ class Qwen3_VisionTransformer(QwenVisionBase):
         g = grid_thw.reshape(-1, 3)
         seqlens = (g[:, 0] * g[:, 1] * g[:, 2]) // unit
         return list(out.split([int(s) for s in seqlens], dim=0))
+
+
+class ModalityProcessor(BaseModalityProcessor):
+    """Qwen3-VL modality processor (reference: :428-461): wraps the Hugging Face processor's image and video
+    processors, which have to be available locally; preprocessing is outside the accelerated path.
+
+    The reference's video processor passes the metadata (fps, duration, frame indices) that its own video loader
+    recorded for the clip; a caller that has such a record sets `video_metadata_provider` to a callable returning
+    it (a `transformers.video_utils.VideoMetadata`), otherwise the clip is processed without metadata."""
+
+    def __init__(self, model_id: str) -> None:
+        super().__init__(model_id=model_id)
+        from transformers import AutoProcessor  # deferred: needs the model files
+
+        self.hf_processor = AutoProcessor.from_pretrained(model_id, trust_remote_code=True)
+        self.video_metadata_provider: Callable | None = None
+
+    def get_image_processor(self) -> Callable | None:
+        def processor(image) -> dict[str, torch.Tensor]:
+            return self.hf_processor.image_processor(images=[image], videos=None, return_tensors="pt").data
+
+        return processor
+
+    def get_video_processor(self) -> Callable | None:
+        def processor(video) -> dict[str, torch.Tensor]:
+            kwargs = {}
+            if self.video_metadata_provider is not None:
+                kwargs["video_metadata"] = [self.video_metadata_provider()]
+            return self.hf_processor.video_processor(videos=[video], do_sample_frames=False, return_tensors="pt",
+                                                     **kwargs).data
+
+        return processor
