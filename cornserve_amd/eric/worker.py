@@ -1,0 +1,100 @@
+"""The step after the forward pass: handing a batch's embeddings to the sidecar.
+
+Mirrors what the reference's worker does around the model call (eric/executor/worker.py:279-344, without the
+tracing spans): run `model(modality, adapter_name, data)`, then for every item whose `receiver_ranks` entry is not
+None call `sidecar.send(data=embedding, id=data_id, chunk_id=..., num_chunks=..., dst_sidecar_ranks=...)`.  The
+embeddings this build's encoders return are contiguous device tensors (row slices of one output buffer), which is
+what the reference's sender needs to export them by IPC handle (sidecar/api.py:236-243).
+
+`MockSidecar` implements the reference client's file-based test mode (sidecar/api.py:41-59,176-188): with
+CORNSERVE_MOCK_SIDECAR=1 and CORNSERVE_MOCK_SIDECAR_MAPPING='{"<id>-<chunk>": "<path>", ...}' every tensor is
+saved with torch.save to the mapped path (other values as JSON), so the encoders can be exercised by the
+reference's executor test harness without a running sidecar.
+"""
+
+from __future__ import annotations
+
+import json
+import os
+from dataclasses import dataclass, field
+from pathlib import Path
+from typing import Any
+
+import torch
+
+from cornserve_amd.eric.api import Modality
+
+
+@dataclass
+class WorkerBatch:
+    """Same fields as the reference's WorkerBatch (eric/schema.py:101-137), minus the tracing carriers."""
+
+    modality: Modality
+    adapter_name: str
+    request_ids: list[str] = field(default_factory=list)
+    data_ids: list[str] = field(default_factory=list)
+    chunk_ids: list[int] = field(default_factory=list)
+    num_chunks: list[int] = field(default_factory=list)
+    receiver_ranks: list[list[list[int]] | None] = field(default_factory=list)
+    data: dict[str, list[torch.Tensor]] = field(default_factory=dict)
+    _dump_prefix: str | None = None
+
+    def __len__(self) -> int:
+        return len(self.data_ids)
+
+
+def mock_sidecar_enabled() -> bool:
+    return os.environ.get("CORNSERVE_MOCK_SIDECAR", "0").lower() in ("1", "true")
+
+
+class MockSidecar:
+    """The reference client's mocking branch of `Sidecar.send` as a stand-alone object."""
+
+    def __init__(self, mapping: dict[str, str | Path] | None = None) -> None:
+        if mapping is None:
+            raw = os.environ.get("CORNSERVE_MOCK_SIDECAR_MAPPING", "")
+            mapping = json.loads(raw) if raw else {}
+        self.mapping = {k: Path(v) for k, v in mapping.items()}
+
+    def send(self, data: Any, id: str, dst_sidecar_ranks: list[list[int]], chunk_id: int = 0, num_chunks: int = 1,
+             stream: bool = False) -> None:
+        key = f"{id}-{chunk_id}"
+        if key not in self.mapping:
+            raise ValueError(f"Mocking sidecar but key {key} not in mapping")
+        path = self.mapping[key]
+        if isinstance(data, torch.Tensor):
+            torch.save(data, path)
+        else:
+            path.write_text(json.dumps(data))
+
+
+class Worker:
+    """Runs batches through one encoder and forwards the embeddings (reference: Worker.execute_model)."""
+
+    def __init__(self, model, sender_sidecar_client=None) -> None:
+        self.model = model
+        if sender_sidecar_client is None and mock_sidecar_enabled():
+            sender_sidecar_client = MockSidecar()
+        self.sender_sidecar_client = sender_sidecar_client
+
+    @torch.inference_mode()
+    def execute_model(self, batch: WorkerBatch) -> list[torch.Tensor]:
+        n = len(batch)
+        if not (len(batch.chunk_ids) == len(batch.num_chunks) == len(batch.receiver_ranks) == n):
+            raise ValueError("data_ids, chunk_ids, num_chunks and receiver_ranks must have one entry per item")
+        output = self.model(modality=batch.modality, adapter_name=batch.adapter_name, batch=batch.data)
+        if len(output) != n:
+            raise RuntimeError(f"the model returned {len(output)} embeddings for {n} items")
+        if self.sender_sidecar_client is not None:
+            for i in range(n):
+                dst = batch.receiver_ranks[i]
+                if dst is None:
+                    continue
+                emb = output[i]
+                if not emb.is_contiguous():   # the reference's sender would copy: keep that cost visible here
+                    raise RuntimeError("embeddings handed to the sidecar must be contiguous")
+                self.sender_sidecar_client.send(data=emb, id=batch.data_ids[i], chunk_id=batch.chunk_ids[i],
+                                                num_chunks=batch.num_chunks[i], dst_sidecar_ranks=dst)
+        if batch._dump_prefix is not None:
+            torch.save([o.cpu() for o in output], batch._dump_prefix + "-tp1.pt")
+        return output

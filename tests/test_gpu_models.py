@@ -151,6 +151,26 @@ def test_qwen_fp8_weights(dev):
     check(out[0], ref[0], REL_FP8, "fp8 weights vs de-quantised fp32 oracle")
 
 
+def test_worker_hand_off_of_real_embeddings(dev, tmp_path):
+    """Embeddings of a real forward pass through the worker's hand-off to the mock sidecar: contiguous device
+    tensors (what the reference's sender exports by IPC handle), saved and reloaded bit-exactly."""
+    from cornserve_amd.eric.worker import MockSidecar, Worker, WorkerBatch
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=9)
+    px, grid = synth.qwen_inputs([(1, 8, 12), (2, 4, 4)], seed=9)
+    direct = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    mapping = {"img0-0": tmp_path / "0.pt", "img1-0": tmp_path / "1.pt"}
+    worker = Worker(model, MockSidecar(mapping))
+    out = worker.execute_model(WorkerBatch(modality=Modality.IMAGE, adapter_name="", request_ids=["r0", "r1"],
+                                           data_ids=["img0", "img1"], chunk_ids=[0, 0], num_chunks=[1, 1],
+                                           receiver_ranks=[[[0]], [[0]]],
+                                           data={"pixel_values": px, "image_grid_thw": grid}))
+    for i in range(2):
+        assert out[i].is_cuda and out[i].is_contiguous() and torch.equal(out[i], direct[i])
+        saved = torch.load(mapping[f"img{i}-0"], weights_only=True)
+        assert torch.equal(saved.to(dev), direct[i])
+
+
 def test_qwen_errors_on_gpu(dev):
     model, _, _ = build_qwen(dev, 1, (0,), seed=6)
     px, grid = synth.qwen_inputs([(1, 4, 4)], seed=6)

@@ -157,3 +157,36 @@ def test_qwen3_vl_class_surface():
     bad.vision_config.hidden_act = "relu6"
     with pytest.raises(NotImplementedError):
         Qwen3_VisionTransformer(bad)
+
+
+def test_worker_hands_embeddings_to_the_mock_sidecar(tmp_path, monkeypatch):
+    """Host logic of the hand-off (the reference's Worker.execute_model + the sidecar client's mock mode)."""
+    from cornserve_amd.eric.api import Modality
+    from cornserve_amd.eric.worker import MockSidecar, Worker, WorkerBatch
+
+    class FakeModel:
+        def __call__(self, modality, adapter_name, batch):
+            return [x.float() * 2 for x in batch["pixel_values"]]
+
+    mapping = {"a-0": str(tmp_path / "a.pt"), "b-1": str(tmp_path / "b.pt")}
+    monkeypatch.setenv("CORNSERVE_MOCK_SIDECAR", "1")
+    monkeypatch.setenv("CORNSERVE_MOCK_SIDECAR_MAPPING", __import__("json").dumps(mapping))
+    worker = Worker(FakeModel())
+    assert isinstance(worker.sender_sidecar_client, MockSidecar)
+    xs = [torch.arange(6.0).reshape(2, 3), torch.ones(1, 3), torch.zeros(4, 3)]
+    batch = WorkerBatch(modality=Modality.IMAGE, adapter_name="", request_ids=["r", "r", "s"], data_ids=["a", "b", "c"],
+                        chunk_ids=[0, 1, 0], num_chunks=[1, 2, 1], receiver_ranks=[[[1]], [[2, 3]], None],
+                        data={"pixel_values": xs})
+    out = worker.execute_model(batch)
+    assert len(out) == 3
+    assert torch.equal(torch.load(tmp_path / "a.pt", weights_only=True), xs[0] * 2)
+    assert torch.equal(torch.load(tmp_path / "b.pt", weights_only=True), xs[1] * 2)
+    assert not (tmp_path / "c.pt").exists()                          # no receiver: nothing sent
+    batch.data_ids[0] = "zzz"
+    with pytest.raises(ValueError):                                  # key not in the mapping
+        worker.execute_model(batch)
+    batch.chunk_ids = [0]
+    with pytest.raises(ValueError):
+        worker.execute_model(batch)
+    MockSidecar({"j-0": tmp_path / "j.json"}).send({"k": 1}, "j", [[0]])
+    assert (tmp_path / "j.json").read_text() == '{"k": 1}'
