@@ -171,6 +171,33 @@ def test_worker_hand_off_of_real_embeddings(dev, tmp_path):
         assert torch.equal(saved.to(dev), direct[i])
 
 
+def test_load_model_from_checkpoint_directory_runs(dev, tmp_path):
+    """A checkpoint directory (config.json + safetensors shards with `visual.` names among other weights) loaded by
+    the loader gives the same embeddings as the model built from the same tensors directly."""
+    import json
+    from types import SimpleNamespace
+    from safetensors.torch import save_file
+    from cornserve_amd.eric.loader import load_model
+
+    def to_dict(o):
+        return {k: to_dict(v) for k, v in vars(o).items()} if isinstance(o, SimpleNamespace) else o
+
+    model, sd, _ = build_qwen(dev, 2, (1,), seed=11)
+    cfg = synth.qwen_vision_config(depth=2, fullatt_block_indexes=(1,))
+    d = tmp_path / "ckpt"
+    d.mkdir()
+    (d / "config.json").write_text(json.dumps({**to_dict(cfg), "dtype": "bfloat16"}))
+    tensors = {"visual." + k: v.bfloat16().contiguous() for k, v in sd.items()}
+    tensors["lm_head.weight"] = torch.zeros(2, 2)
+    save_file(tensors, str(d / "model.safetensors"))
+    loaded = load_model(d, torch_device=dev)
+    assert loaded.dtype == torch.bfloat16 and loaded.device.type == "cuda"
+    px, grid = synth.qwen_inputs([(1, 8, 12), (1, 4, 4)], seed=11)
+    a = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    b = loaded(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+
+
 def test_qwen_errors_on_gpu(dev):
     model, _, _ = build_qwen(dev, 1, (0,), seed=6)
     px, grid = synth.qwen_inputs([(1, 4, 4)], seed=6)

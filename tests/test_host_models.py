@@ -190,3 +190,83 @@ def test_worker_hands_embeddings_to_the_mock_sidecar(tmp_path, monkeypatch):
         worker.execute_model(batch)
     MockSidecar({"j-0": tmp_path / "j.json"}).send({"k": 1}, "j", [[0]])
     assert (tmp_path / "j.json").read_text() == '{"k": 1}'
+
+
+# ------------------------------------------------------------------ loading from a local checkpoint directory
+def _ns_to_dict(o):
+    from types import SimpleNamespace
+    if isinstance(o, SimpleNamespace):
+        return {k: _ns_to_dict(v) for k, v in vars(o).items()}
+    return o
+
+
+def _write_checkpoint(directory, config, tensors: dict, shards: int = 2, with_index: bool = True):
+    import json
+    from safetensors.torch import save_file
+
+    directory.mkdir(parents=True, exist_ok=True)
+    cfg = _ns_to_dict(config)
+    cfg.setdefault("dtype", "float32")
+    (directory / "config.json").write_text(json.dumps(cfg))
+    names = sorted(tensors)
+    weight_map = {}
+    for s in range(shards):
+        part = {n: tensors[n].contiguous() for n in names[s::shards]}
+        fname = f"model-{s + 1:05d}-of-{shards:05d}.safetensors"
+        save_file(part, str(directory / fname))
+        weight_map.update({n: fname for n in part})
+    if with_index:
+        (directory / "model.safetensors.index.json").write_text(json.dumps({"weight_map": weight_map}))
+
+
+def test_load_model_from_local_checkpoint(tmp_path):
+    from cornserve_amd import synth
+    from cornserve_amd.eric.loader import load_model
+    from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
+    from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
+
+    cpu = torch.device("cpu")
+    # Qwen2.5-VL: `visual.` weights among language-model weights, two shards with an index
+    cfg = synth.qwen_vision_config(depth=2, fullatt_block_indexes=(1,))
+    sd = synth.qwen_state_dict(cfg, seed=3)
+    ckpt = {"visual." + k: v for k, v in sd.items()}
+    ckpt.update({"model.layers.0.mlp.up_proj.weight": torch.zeros(4, 4), "lm_head.weight": torch.ones(2, 2)})
+    _write_checkpoint(tmp_path / "qwen", cfg, ckpt)
+    model = load_model(tmp_path / "qwen", torch_device=cpu)
+    assert isinstance(model, Qwen2_5_VisionTransformer) and not model.training and model.dtype == torch.float32
+    assert torch.equal(model.blocks[1].attn.qkv.weight, sd["blocks.1.attn.qkv.weight"])
+    assert load_model(tmp_path / "qwen", torch_device=cpu, torch_dtype=torch.bfloat16).dtype == torch.bfloat16
+    assert load_model(tmp_path / "qwen", torch_device=cpu, weight_format="fp8_e4m3").weight_format == "fp8_e4m3"
+    # a missing weight and an unexpected one are errors, as in the reference
+    bad = dict(ckpt)
+    del bad["visual.merger.ln_q.weight"]
+    _write_checkpoint(tmp_path / "qwen_missing", cfg, bad, shards=1, with_index=False)
+    with pytest.raises(ValueError, match="Missing weights"):
+        load_model(tmp_path / "qwen_missing", torch_device=cpu)
+    bad = dict(ckpt)
+    bad["visual.extra.weight"] = torch.zeros(1)
+    _write_checkpoint(tmp_path / "qwen_extra", cfg, bad, shards=1, with_index=False)
+    with pytest.raises(ValueError, match="Unexpected weights"):
+        load_model(tmp_path / "qwen_extra", torch_device=cpu)
+    with pytest.raises(FileNotFoundError):
+        load_model(tmp_path / "nowhere", torch_device=cpu)
+    unknown = synth.qwen_vision_config(depth=1)
+    unknown.model_type = "no_such_model"
+    _write_checkpoint(tmp_path / "unknown", unknown, {"visual.x": torch.zeros(1)}, shards=1)
+    with pytest.raises(KeyError):
+        load_model(tmp_path / "unknown", torch_device=cpu)
+
+    # Gemma-3: tower weights into the model (post_layernorm ignored), projector weights into an adapter per directory
+    gcfg = synth.gemma3_config(num_hidden_layers=1, image_size=56, text_hidden=64, mm_tokens_per_image=4)
+    gsd = synth.gemma3_state_dict(gcfg, seed=4)
+    gsd["language_model.embed.weight"] = torch.zeros(3, 3)
+    _write_checkpoint(tmp_path / "gemma", gcfg, gsd)
+    other = {k: v + 1 for k, v in gsd.items() if k.startswith("multi_modal_projector.")}
+    _write_checkpoint(tmp_path / "gemma_ft", gcfg, other, shards=1, with_index=False)
+    g = load_model(tmp_path / "gemma", adapter_model_dirs=[tmp_path / "gemma_ft"], torch_device=cpu)
+    assert isinstance(g, Gemma3VisionEncoder)
+    adapters = g.multi_modal_projector.adapters
+    assert list(adapters) == [str(tmp_path / "gemma"), str(tmp_path / "gemma_ft")]
+    w0 = adapters[str(tmp_path / "gemma")].mm_input_projection_weight
+    w1 = adapters[str(tmp_path / "gemma_ft")].mm_input_projection_weight
+    assert torch.equal(w0, gsd["multi_modal_projector.mm_input_projection_weight"]) and torch.equal(w1, w0 + 1)
