@@ -128,6 +128,22 @@ def test_qwen_multi_image_ragged_and_video(dev):
         check(o, r, REL_BF16, f"video {i} {vgrids[i]}")
 
 
+def test_qwen_largest_image_and_many_tiny_items(dev):
+    """The largest image the processor emits (1344 x 1344 = 96 x 96 patches: 144 key tiles per full-attention
+    segment, 144 windows) and a batch of 40 one-block items (every segment shorter than a tile)."""
+    model, sd, ocfg = build_qwen(dev, 2, (1,), seed=12)
+    px, grid = synth.qwen_inputs([(1, 96, 96)], seed=12)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    assert out[0].shape == (2304, 3584)
+    check(out[0], oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)[0], REL_BF16, "96x96 grid")
+    tiny = [(1, 2, 2)] * 40
+    px, grid = synth.qwen_inputs(tiny, seed=13)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    ref = oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
+    assert len(out) == 40 and all(o.shape == (1, 3584) for o in out)
+    check(torch.cat(out), torch.cat(ref), REL_BF16, "40 one-block items")
+
+
 def test_qwen_batch_items_are_independent(dev):
     """An item's embedding does not depend on what else is in the batch (bit-identical)."""
     model, _, _ = build_qwen(dev, 2, (1,), seed=4)
