@@ -244,7 +244,9 @@ extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
   if (((uintptr_t)a.A | (uintptr_t)a.W) & 15) return CS_ERR_INVALID_ARG;
   if (((uintptr_t)a.C | (uintptr_t)a.bias | (uintptr_t)a.residual | (uintptr_t)a.pos) & 7) return CS_ERR_INVALID_ARG;
   if ((uintptr_t)a.w_scale & 15) return CS_ERR_INVALID_ARG;
-  if (((uintptr_t)a.a_row_sumsq | (uintptr_t)a.c_row_sumsq) & 15) return CS_ERR_INVALID_ARG;
+  if (((uintptr_t)a.a_row_sumsq | (uintptr_t)a.c_row_sumsq | (uintptr_t)a.a_row_sum | (uintptr_t)a.c_row_sum |
+       (uintptr_t)a.w_col_sum) & 15)
+    return CS_ERR_INVALID_ARG;
 
   // Fast path (direct-to-LDS pipeline) when the shape allows it; otherwise the general kernel below.
   {
@@ -252,7 +254,7 @@ extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
     const int st = cs_gemm_fast(a, stream, &handled);
     if (handled) return st;
   }
-  if (a.a_row_sumsq || a.c_row_sumsq) return CS_ERR_UNSUPPORTED;  // the folded norm exists in the fast kernel only
+  if (a.a_row_sumsq || a.c_row_sumsq || a.a_row_sum || a.c_row_sum) return CS_ERR_UNSUPPORTED;  // the folded norms exist in the fast kernel only
   // Tile choice: 256x256 when that fills the chip's 256 CUs reasonably, else smaller tiles for more workgroups.
   const int64_t t256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
   const bool small = t256 < 192;

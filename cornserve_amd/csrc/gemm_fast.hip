@@ -125,7 +125,10 @@ struct RingShape {
 // by rsqrt(sum of squares of the A row / K + eps) before the bias (the norm's weight is folded into W by the
 // caller); FUSE_SUMSQ_C = besides C, the sum of squares of every output row over this tile's columns goes to
 // c_row_sumsq (what the next FUSE_NORM_A launch reads).
-constexpr int FUSE_NORM_A = 1, FUSE_SUMSQ_C = 2;
+// FUSE_LN_A / FUSE_STATS_C: the same for LayerNorm -- the producer also emits the row sums, the consumer computes
+// rstd * (acc - mean * w_col_sum[n]) + bias[n] with mean and rstd from the two sets of parts (the norm's weight is
+// folded into W, its bias into the GEMM bias, and w_col_sum[n] = sum_k W'[n,k] carries the mean term).
+constexpr int FUSE_NORM_A = 1, FUSE_SUMSQ_C = 2, FUSE_LN_A = 3, FUSE_STATS_C = 4;
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE>
 __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -457,7 +460,23 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         const int mc = min(mrow[i], p.M - 1);
         crow[i] = p.c_rows ? p.c_rows[mc] : mc;
       }
-      float rstd[FUSE == FUSE_NORM_A ? MT : 1];
+      constexpr bool NORM_A = FUSE == FUSE_NORM_A || FUSE == FUSE_LN_A;
+      float rstd[NORM_A ? MT : 1];
+      float nmean_rstd[FUSE == FUSE_LN_A ? MT : 1];   // -mean * rstd
+      if constexpr (FUSE == FUSE_LN_A) {
+        auto total = [](const float* parts) {
+          const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
+          return ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
+        };
+#pragma unroll
+        for (int i = 0; i < MT; ++i) {
+          const int64_t row = (int64_t)min(mrow[i], p.M - 1) * CS_SUMSQ_PARTS;
+          const float mean = total(p.a_row_sum + row) / (float)p.K;
+          const float var = fmaxf(total(p.a_row_sumsq + row) / (float)p.K - mean * mean, 0.f);
+          rstd[i] = rsqrtf(var + p.norm_eps);
+          nmean_rstd[i] = -mean * rstd[i];
+        }
+      }
       if constexpr (FUSE == FUSE_NORM_A) {
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
@@ -466,6 +485,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
           rstd[i] = rsqrtf(ss / (float)p.K + p.norm_eps);
         }
+      }
+      f32x4_t csum_v[FUSE == FUSE_LN_A ? NT : 1];
+      if constexpr (FUSE == FUSE_LN_A) {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) csum_v[j] = *(const f32x4_t*)(p.w_col_sum + min(n_lane + piece_col(j), p.N - 4));
       }
       bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
 #pragma unroll
@@ -515,7 +539,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           for (int r = 0; r < 4; ++r) {
             float t = racc[j][r];
             if constexpr (W_FP8) t *= scale_v[W_FP8 ? j : 0][r];
-            if constexpr (FUSE == FUSE_NORM_A) t *= rstd[FUSE == FUSE_NORM_A ? i : 0];
+            if constexpr (NORM_A) t *= rstd[NORM_A ? i : 0];
+            if constexpr (FUSE == FUSE_LN_A) t += nmean_rstd[FUSE == FUSE_LN_A ? i : 0] * csum_v[FUSE == FUSE_LN_A ? j : 0][r];
             v[r] = t + bf2f(bias_v[j][r]);
           }
           if (EPI == CS_EPI_SWIGLU) {
@@ -543,23 +568,29 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
             for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
           }
         }
-        if constexpr (FUSE == FUSE_SUMSQ_C) {
+        if constexpr (FUSE == FUSE_SUMSQ_C || FUSE == FUSE_STATS_C) {
           // Sum of squares of the row's ROUNDED outputs over this wave's columns: lane-local over the lane's
           // pieces, then over the four lanes of the row (fixed order: the result does not depend on timing).
           static_assert(WAVES_N == 1 && EPI != CS_EPI_SWIGLU, "one wave spans the tile's columns: one part per tile");
-          float ss = 0.f;
+          float ss = 0.f, sm = 0.f;
 #pragma unroll
           for (int j = 0; j < NT; ++j) {
             const bool nok = n_lane + piece_col(j) < p.N;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-              const float o = bf2f(out[j][r]);
-              ss += nok ? o * o : 0.f;
+              const float o = nok ? bf2f(out[j][r]) : 0.f;
+              ss += o * o;
+              if constexpr (FUSE == FUSE_STATS_C) sm += o;
             }
           }
           ss += __shfl_xor(ss, 16);
           ss += __shfl_xor(ss, 32);
           if (mok && kq == 0) p.c_row_sumsq[(int64_t)crow[i] * CS_SUMSQ_PARTS + n0 / BN] = ss;
+          if constexpr (FUSE == FUSE_STATS_C) {
+            sm += __shfl_xor(sm, 16);
+            sm += __shfl_xor(sm, 32);
+            if (mok && kq == 0) p.c_row_sum[(int64_t)crow[i] * CS_SUMSQ_PARTS + n0 / BN] = sm;
+          }
         }
         // With G == 2 the pieces of fragments 2g and 2g+1 are adjacent: one 16-byte store per lane, and the
         // four lanes of an output row write 64 consecutive bytes (32 with the halved SwiGLU output).
@@ -634,6 +665,26 @@ template <int BM, int BN, int WAVES_M, int WAVES_N, bool W_FP8>
 int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
   if constexpr (!W_FP8) {
     // the fused-norm forms exist for the epilogues an encoder block pairs them with
+    if (a.a_row_sum) {   // LayerNorm in front of this GEMM
+      if (!a.a_row_sumsq || !a.w_col_sum || a.pos || a.c_row_sumsq || a.c_row_sum) return CS_ERR_UNSUPPORTED;
+      // (the per-column sums take 4 registers per piece on top of the bias: with the 64 pieces of a 256x256 tile's
+      // wave the epilogue no longer fits the architectural registers, so that tile is not built; cs_gemm_fast
+      // sends these launches to the 256x160 tile)
+      if constexpr (BM == 256 && BN == 256) return CS_ERR_UNSUPPORTED;
+      else switch (a.epilogue) {
+        case CS_EPI_BIAS: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_LN_A>(a, s);
+        case CS_EPI_GELU_TANH: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_TANH, false, FUSE_LN_A>(a, s);
+        case CS_EPI_QUICK_GELU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_QUICK_GELU, false, FUSE_LN_A>(a, s);
+        default: return CS_ERR_UNSUPPORTED;
+      }
+    }
+    if (a.c_row_sum) {   // ... and behind it: sums and sums of squares of the output rows
+      if (!a.c_row_sumsq || a.pos) return CS_ERR_UNSUPPORTED;
+      if constexpr (BN == 160 && WAVES_N == 1) {
+        if (a.epilogue == CS_EPI_RESIDUAL) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_STATS_C>(a, s);
+      }
+      return CS_ERR_UNSUPPORTED;
+    }
     if (a.a_row_sumsq) {
       if (a.pos || a.c_row_sumsq) return CS_ERR_UNSUPPORTED;
       if (a.epilogue == CS_EPI_BIAS) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_NORM_A>(a, s);
@@ -648,7 +699,7 @@ int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
       return CS_ERR_UNSUPPORTED;
     }
   } else {
-    if (a.a_row_sumsq || a.c_row_sumsq) return CS_ERR_UNSUPPORTED;
+    if (a.a_row_sumsq || a.c_row_sumsq || a.a_row_sum || a.c_row_sum) return CS_ERR_UNSUPPORTED;
   }
   switch (a.epilogue) {
     case CS_EPI_BIAS:
@@ -707,6 +758,7 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
     if (a.N > CS_SUMSQ_PARTS * 160 || a.w_fp8) return CS_ERR_UNSUPPORTED;
     return dispatch_epi<256, 160, 4, 1>(a, stream);
   }
+  if (a.a_row_sum) return dispatch_epi<256, 160, 4, 1>(a, stream);   // see dispatch_epi_w
   if (fits160 && (force ? force[0] == '1' : c160 < c256)) return dispatch_epi<256, 160, 4, 1>(a, stream);
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller

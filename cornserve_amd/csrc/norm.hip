@@ -113,8 +113,9 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const bf16_t* __restrict
 
 // Sums of squares of a row in parts of 160 columns (20 chunks): the variance term of RMSNorm in the form
 // that a GEMM with CsGemmArgs.a_row_sumsq consumes.  out is [rows][CS_SUMSQ_PARTS].
+template <bool WITH_SUM>
 __global__ __launch_bounds__(256) void row_sumsq_kernel(const bf16_t* __restrict__ x, int64_t ldx, int rows, int H,
-                                                        float* __restrict__ out) {
+                                                        float* __restrict__ out, float* __restrict__ sum_out) {
   constexpr int NC = (160 * CS_SUMSQ_PARTS / 8 + 63) / 64;
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
@@ -122,24 +123,41 @@ __global__ __launch_bounds__(256) void row_sumsq_kernel(const bf16_t* __restrict
   const int nchunks = H >> 3;
   float v[NC][8];
   load_row<NC>(x + (int64_t)row * ldx, nchunks, lane, v);
-  float part[CS_SUMSQ_PARTS];
+  float part[CS_SUMSQ_PARTS], spart[WITH_SUM ? CS_SUMSQ_PARTS : 1];
 #pragma unroll
-  for (int q = 0; q < CS_SUMSQ_PARTS; ++q) part[q] = 0.f;
-#pragma unroll
-  for (int j = 0; j < NC; ++j) {
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) ss += v[j][e] * v[j][e];
-    const int q_of_chunk = (lane + 64 * j) / 20;
-#pragma unroll
-    for (int q = 0; q < CS_SUMSQ_PARTS; ++q) part[q] += (q == q_of_chunk) ? ss : 0.f;
+  for (int q = 0; q < CS_SUMSQ_PARTS; ++q) {
+    part[q] = 0.f;
+    if (WITH_SUM) spart[WITH_SUM ? q : 0] = 0.f;
   }
 #pragma unroll
-  for (int q = 0; q < CS_SUMSQ_PARTS; ++q) part[q] = wave_sum(part[q]);
+  for (int j = 0; j < NC; ++j) {
+    float ss = 0.f, sm = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      ss += v[j][e] * v[j][e];
+      sm += v[j][e];
+    }
+    const int q_of_chunk = (lane + 64 * j) / 20;
+#pragma unroll
+    for (int q = 0; q < CS_SUMSQ_PARTS; ++q) {
+      part[q] += (q == q_of_chunk) ? ss : 0.f;
+      if (WITH_SUM) spart[WITH_SUM ? q : 0] += (q == q_of_chunk) ? sm : 0.f;
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < CS_SUMSQ_PARTS; ++q) {
+    part[q] = wave_sum(part[q]);
+    if (WITH_SUM) spart[WITH_SUM ? q : 0] = wave_sum(spart[WITH_SUM ? q : 0]);
+  }
   if (lane == 0) {
     float* o = out + (int64_t)row * CS_SUMSQ_PARTS;
 #pragma unroll
     for (int q = 0; q < CS_SUMSQ_PARTS; q += 4) *(f32x4_t*)(o + q) = f32x4_t{part[q], part[q + 1], part[q + 2], part[q + 3]};
+    if constexpr (WITH_SUM) {
+      float* so = sum_out + (int64_t)row * CS_SUMSQ_PARTS;
+#pragma unroll
+      for (int q = 0; q < CS_SUMSQ_PARTS; q += 4) *(f32x4_t*)(so + q) = f32x4_t{spart[q], spart[q + 1], spart[q + 2], spart[q + 3]};
+    }
   }
 }
 
@@ -254,15 +272,23 @@ extern "C" int cs_rmsnorm(const void* x, int64_t ldx, const void* w, void* y, in
   return cs_launch_status();
 }
 
-extern "C" int cs_row_sumsq(const void* x, int64_t ldx, int32_t rows, int32_t H, float* out, void* stream_) {
+extern "C" int cs_row_stats(const void* x, int64_t ldx, int32_t rows, int32_t H, float* out, float* sum_out, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
-  if (!x || !out || rows < 0 || H <= 0 || H % 8 || ldx % 8 || ldx < H || (((uintptr_t)x | (uintptr_t)out) & 15))
+  if (!x || !out || rows < 0 || H <= 0 || H % 8 || ldx % 8 || ldx < H ||
+      (((uintptr_t)x | (uintptr_t)out | (uintptr_t)sum_out) & 15))
     return CS_ERR_INVALID_ARG;
   if (H > 160 * CS_SUMSQ_PARTS) return CS_ERR_UNSUPPORTED;
   if (rows == 0) return CS_OK;
   const dim3 grid((rows + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK), block(256);
-  hipLaunchKernelGGL(row_sumsq_kernel, grid, block, 0, stream, (const bf16_t*)x, ldx, rows, H, out);
+  if (sum_out)
+    hipLaunchKernelGGL(row_sumsq_kernel<true>, grid, block, 0, stream, (const bf16_t*)x, ldx, rows, H, out, sum_out);
+  else
+    hipLaunchKernelGGL(row_sumsq_kernel<false>, grid, block, 0, stream, (const bf16_t*)x, ldx, rows, H, out, sum_out);
   return cs_launch_status();
+}
+
+extern "C" int cs_row_sumsq(const void* x, int64_t ldx, int32_t rows, int32_t H, float* out, void* stream_) {
+  return cs_row_stats(x, ldx, rows, H, out, nullptr, stream_);
 }
 
 extern "C" int cs_layernorm(const void* x, int64_t ldx, const void* w, const void* b, void* y, int64_t ldy,

@@ -96,3 +96,15 @@ class BaseModalityProcessor:
         if processor is None:
             raise ValueError(f"{getter[1]} processor not available.")
         return processor(data)
+
+
+@torch.no_grad()
+def fold_layernorm(w: torch.Tensor, b: torch.Tensor | None, ln_w: torch.Tensor, ln_b: torch.Tensor):
+    """A LayerNorm's affine part folded into the linear layer behind it, for the GEMM that applies the
+    normalisation itself (CsGemmArgs.a_row_sum):  LN(x) . W^T + b  ==  rstd * (x . W'^T - mean * colsum) + b'.
+    Returns (W' = W * ln_w along the columns, b' = b + W . ln_b, colsum = row sums of the rounded W' in fp32)."""
+    wf = (w.float() * ln_w.float()[None, :]).to(w.dtype)
+    bf = w.float() @ ln_b.float()
+    if b is not None:
+        bf = bf + b.float()
+    return wf.contiguous(), bf.to(w.dtype).contiguous(), wf.float().sum(dim=1).contiguous()

@@ -30,7 +30,7 @@ import torch
 import torch.nn as nn
 
 from cornserve_amd import ops
-from cornserve_amd.eric.models.base import BaseModalityProcessor
+from cornserve_amd.eric.models.base import BaseModalityProcessor, fold_layernorm
 from cornserve_amd.eric.models.qwen2_5_vl import FrameModalityProcessor, QwenVisionBase, _Attn, _Linear, _no_mark  # noqa: F401
 from cornserve_amd.eric.models.qwen2_vl import _LayerNorm
 
@@ -93,12 +93,18 @@ class Qwen3_VisionTransformer(QwenVisionBase):
     image_mean = (0.5, 0.5, 0.5)   # the Qwen3-VL checkpoints' preprocessor_config.json
     image_std = (0.5, 0.5, 0.5)
 
-    def __init__(self, config: Any, weight_format: str = "bf16") -> None:
+    def __init__(self, config: Any, weight_format: str = "bf16", fold_norm: bool = True) -> None:
+        """`fold_norm`: norm1 / norm2 of every block are applied inside the GEMM that follows them (see
+        Qwen2_5_VisionTransformer; here the norms are LayerNorms: the residual GEMMs also emit the row sums).  On by
+        default (measured: 10.09 against 10.17 ms per 8192 patches)."""
         super().__init__()
         vc = config.vision_config if hasattr(config, "vision_config") else config
         if weight_format not in ("bf16", "fp8_e4m3"):
             raise ValueError(f"Unknown weight_format: {weight_format}")
         self.weight_format = weight_format
+        E = vc.hidden_size
+        self.fold_norm = (bool(fold_norm) and weight_format == "bf16" and E % 64 == 0 and 192 <= E <= 160 * ops.SUMSQ_PARTS
+                          and vc.hidden_act in ("gelu_pytorch_tanh", "quick_gelu"))
         self.in_channels = vc.in_channels
         self.embed_dim = vc.hidden_size
         self.num_heads = vc.num_heads
@@ -151,14 +157,23 @@ class Qwen3_VisionTransformer(QwenVisionBase):
         # (the patch embedding stays bf16 also with fp8 weights, like the other Qwen encoders')
         pk: dict = {"pe": {"w": self.patch_embed.proj.weight.contiguous(), "s": None, "b": self.patch_embed.proj.bias},
                     "pos": self.pos_embed.weight.contiguous()}
+        def folded(w: torch.Tensor, b: torch.Tensor, norm: _LayerNorm, padded: bool) -> dict:
+            w, b, colsum = fold_layernorm(w, b, norm.weight, norm.bias)
+            if padded:   # pad AFTER folding: the pad rows stay exactly zero (weight, bias and column sum)
+                w, b, colsum = pad_rows(w), pad_rows(b), pad_rows(colsum)
+            return {"w": w.contiguous(), "s": None, "b": b.contiguous(), "colsum": colsum.contiguous()}
+
+        fold = self.fold_norm
         pk["blocks"] = [
             {
                 "n1": (b.norm1.weight, b.norm1.bias),
                 "n2": (b.norm2.weight, b.norm2.bias),
-                "qkv": self._lin(b.attn.qkv.weight, b.attn.qkv.bias),
+                "qkv": folded(b.attn.qkv.weight, b.attn.qkv.bias, b.norm1, False) if fold
+                else self._lin(b.attn.qkv.weight, b.attn.qkv.bias),
                 "proj": self._lin(b.attn.proj.weight, b.attn.proj.bias),
                 # gelu(0) = 0 and the padded fc2 columns are zero: the padding contributes exactly nothing
-                "fc1": self._lin(pad_rows(b.mlp.linear_fc1.weight), pad_rows(b.mlp.linear_fc1.bias)),
+                "fc1": folded(b.mlp.linear_fc1.weight, b.mlp.linear_fc1.bias, b.norm2, True) if fold
+                else self._lin(pad_rows(b.mlp.linear_fc1.weight), pad_rows(b.mlp.linear_fc1.bias)),
                 "fc2": self._lin(pad_cols(b.mlp.linear_fc2.weight), b.mlp.linear_fc2.bias),
             }
             for b in self.blocks
@@ -201,11 +216,28 @@ class Qwen3_VisionTransformer(QwenVisionBase):
         out = torch.empty((L // unit, O * n_out), dtype=torch.bfloat16, device=dev)
         scale = d**-0.5
         kept: list[torch.Tensor] = []
-        for i, b in enumerate(pk["blocks"]):
+        fold = self.fold_norm
+        if fold:
+            if L * max(3 * E, self.intermediate_size + self.mlp_pad) * 2 >= 2**32:
+                raise ValueError(f"{L} patches in one forward exceed what the folded-norm GEMMs address; split the batch "
+                                 "or construct the model with fold_norm=False")
             mark("norm")
-            ops.layernorm(x, *b["n1"], eps, out=n)
-            mark("gemm_qkv")
-            self._g(n, b["qkv"], out=qkv)
+            ss = torch.zeros((L, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev)
+            sm = torch.zeros_like(ss)
+            ops.row_stats(x, ss, sm)
+            stats_in = lambda lin: {"a_row_sumsq": ss, "a_row_sum": sm, "w_col_sum": lin["colsum"], "norm_eps": eps}  # noqa: E731
+            stats_out = {"c_row_sumsq": ss, "c_row_sum": sm}
+        else:
+            stats_out = {}
+        for i, b in enumerate(pk["blocks"]):
+            if fold:
+                mark("gemm_qkv")
+                ops.gemm(x, b["qkv"]["w"], b["qkv"]["b"], out=qkv, **stats_in(b["qkv"]))
+            else:
+                mark("norm")
+                ops.layernorm(x, *b["n1"], eps, out=n)
+                mark("gemm_qkv")
+                self._g(n, b["qkv"], out=qkv)
             mark("rope")
             ops.rope_qk_(qkv, ix.cos_sin, nh, d)
             mark("attn_full")
@@ -213,14 +245,18 @@ class Qwen3_VisionTransformer(QwenVisionBase):
             mark("gemm_proj")
             # a hidden state kept for a deepstack merger must survive: the next update goes to a new buffer
             x_next = torch.empty_like(x) if kept and kept[-1] is x else x
-            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x_next)
+            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x_next, **stats_out)
             x = x_next
-            mark("norm")
-            ops.layernorm(x, *b["n2"], eps, out=n)
-            mark("gemm_fc1")
-            self._g(n, b["fc1"], epilogue=self.act_epilogue, out=hmid)
+            if fold:
+                mark("gemm_fc1")
+                ops.gemm(x, b["fc1"]["w"], b["fc1"]["b"], epilogue=self.act_epilogue, out=hmid, **stats_in(b["fc1"]))
+            else:
+                mark("norm")
+                ops.layernorm(x, *b["n2"], eps, out=n)
+                mark("gemm_fc1")
+                self._g(n, b["fc1"], epilogue=self.act_epilogue, out=hmid)
             mark("gemm_fc2")
-            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
+            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **stats_out)
             if i in self.deepstack_visual_indexes:
                 kept.append(x)
 

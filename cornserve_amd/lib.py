@@ -17,7 +17,7 @@ CS_ERR_INVALID_ARG = 1
 CS_ERR_UNSUPPORTED = 2
 CS_ERR_LAUNCH = 3
 CS_ERR_TOO_LARGE = 4
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH, EPI_QUICK_GELU = range(6)
 
@@ -51,6 +51,9 @@ class CsGemmArgs(ctypes.Structure):
         ("a_row_sumsq", c_void_p),
         ("c_row_sumsq", c_void_p),
         ("norm_eps", ctypes.c_float),
+        ("a_row_sum", c_void_p),
+        ("c_row_sum", c_void_p),
+        ("w_col_sum", c_void_p),
     ]
 
 
@@ -59,6 +62,7 @@ _SIGNATURES: dict[str, list] = {
     "cs_abi_version": [],
     "cs_gemm": [POINTER(CsGemmArgs), c_void_p],
     "cs_row_sumsq": [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p],
+    "cs_row_stats": [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
     "cs_rmsnorm": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_float, c_int32, c_void_p],
     "cs_layernorm": [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_float, c_void_p],
     "cs_vit_seqlens_host": [

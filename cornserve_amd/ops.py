@@ -69,12 +69,17 @@ def gemm(
     a_row_sumsq: torch.Tensor | None = None,
     c_row_sumsq: torch.Tensor | None = None,
     norm_eps: float = 0.0,
+    a_row_sum: torch.Tensor | None = None,
+    c_row_sum: torch.Tensor | None = None,
+    w_col_sum: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`.
 
     `a_row_sumsq` (fp32 [M, SUMSQ_PARTS]) scales row m of the product by rsqrt(sum(parts)/K + norm_eps): an
     RMSNorm of `a` whose weight the caller has folded into the columns of `w`.  `c_row_sumsq` (same layout,
-    indexed by output row) receives the sums of squares of the output rows."""
+    indexed by output row) receives the sums of squares of the output rows.  With `a_row_sum` (and `w_col_sum`,
+    fp32 [N], the row sums of the folded weight) the fold is a LayerNorm's: rstd * (acc - mean * w_col_sum) + bias;
+    `c_row_sum` receives the plain sums of the output rows."""
     lib = _l.load()
     _req(a, torch.bfloat16, "a")
     if a.dim() != 2 or w.dim() != 2:
@@ -108,7 +113,8 @@ def gemm(
     args.M, args.N, args.K = M, N, K
     args.epilogue = epilogue
     args.w_fp8 = 1 if fp8 else 0
-    for name, t in (("a_row_sumsq", a_row_sumsq), ("c_row_sumsq", c_row_sumsq)):
+    for name, t in (("a_row_sumsq", a_row_sumsq), ("c_row_sumsq", c_row_sumsq), ("a_row_sum", a_row_sum),
+                    ("c_row_sum", c_row_sum)):
         if t is not None:
             _req(t, torch.float32, name)
             if t.dim() != 2 or t.shape[1] != SUMSQ_PARTS or not t.is_contiguous() or t.shape[0] < M:
@@ -116,12 +122,31 @@ def gemm(
     args.a_row_sumsq = _ptr(a_row_sumsq)
     args.c_row_sumsq = _ptr(c_row_sumsq)
     args.norm_eps = norm_eps
+    if w_col_sum is not None:
+        _req(w_col_sum, torch.float32, "w_col_sum")
+        if tuple(w_col_sum.shape) != (N,) or not w_col_sum.is_contiguous():
+            raise ValueError(f"w_col_sum must be a contiguous fp32 [{N}] tensor")
+    args.a_row_sum = _ptr(a_row_sum)
+    args.c_row_sum = _ptr(c_row_sum)
+    args.w_col_sum = _ptr(w_col_sum)
     _l.check(lib.cs_gemm(ctypes.byref(args), _stream()), "cs_gemm")
     return out
 
 
 # -------------------------------------------------------------------------------------------- norms
 SUMSQ_PARTS = 8  # CS_SUMSQ_PARTS
+
+
+def row_stats(x: torch.Tensor, sumsq_out: torch.Tensor, sum_out: torch.Tensor) -> None:
+    """Sums of squares and sums of the rows of `x`, each fp32 [rows, SUMSQ_PARTS] in parts of 160 columns."""
+    lib = _l.load()
+    _req(x, torch.bfloat16, "x")
+    _req(sumsq_out, torch.float32, "sumsq_out")
+    _req(sum_out, torch.float32, "sum_out")
+    if x.dim() != 2 or tuple(sumsq_out.shape) != (x.shape[0], SUMSQ_PARTS) or tuple(sum_out.shape) != (x.shape[0], SUMSQ_PARTS):
+        raise ValueError("row_stats takes a 2-D tensor and two [rows, SUMSQ_PARTS] outputs")
+    _l.check(lib.cs_row_stats(x.data_ptr(), x.stride(0), x.shape[0], x.shape[1], sumsq_out.data_ptr(), sum_out.data_ptr(),
+                              _stream()), "cs_row_stats")
 
 
 def row_sumsq(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:

@@ -36,7 +36,7 @@ extern "C" {
 #define CS_ERR_TOO_LARGE 4
 
 /* ABI version of this header; cs_abi_version() returns the value the library was built with. */
-#define CS_ABI_VERSION 2
+#define CS_ABI_VERSION 3
 int cs_abi_version(void);
 
 /* ------------------------------------------------------------------------------------------------
@@ -90,6 +90,17 @@ typedef struct CsGemmArgs {
   const float* a_row_sumsq;
   float* c_row_sumsq;
   float norm_eps;
+  /* LayerNorm folded the same way (nn.LayerNorm in front of qkv / fc1: siglip.py:333-345, qwen2_vl.py:277-291,
+   * qwen3_vl.py:139-153).  With mean = sum/K, var = sumsq/K - mean^2, rstd = rsqrt(var + norm_eps):
+   *   LN(x) . W^T + b  ==  rstd * (x . W'^T - mean * w_col_sum) + b'   with W' = W * w_ln (columns), b' = b + W . b_ln,
+   *   w_col_sum[n] = sum_k W'[n,k]; the caller passes W', b' and w_col_sum.
+   * a_row_sum:  optional fp32 [M][CS_SUMSQ_PARTS], parts of sum_k A[m,k]; needs a_row_sumsq and w_col_sum (fp32 [N]).
+   *   CS_EPI_BIAS, CS_EPI_GELU_TANH, CS_EPI_QUICK_GELU, bf16 W.
+   * c_row_sum:  optional, the sums of the rounded output rows in the layout of c_row_sumsq (which it needs);
+   *   CS_EPI_RESIDUAL, bf16 W, N <= 160 * CS_SUMSQ_PARTS.                                           */
+  const float* a_row_sum;
+  float* c_row_sum;
+  const float* w_col_sum;
 } CsGemmArgs;
 #define CS_SUMSQ_PARTS 8
 
@@ -107,6 +118,9 @@ int cs_rmsnorm(const void* x, int64_t ldx, const void* w, void* y, int64_t ldy, 
  * CsGemmArgs.c_row_sumsq: out[m][p] = sum of x[m, 160p .. 160p+159]^2, parts beyond H are written as 0.
  * The variance term of RMSNorm (norm.py:35-70) for a GEMM launched with a_row_sumsq.               */
 int cs_row_sumsq(const void* x, int64_t ldx, int32_t rows, int32_t H, float* out, void* stream);
+/* The same with the plain row sums next to them (sum_out in the same layout): the statistics of LayerNorm for a
+ * GEMM launched with a_row_sum.                                                                     */
+int cs_row_stats(const void* x, int64_t ldx, int32_t rows, int32_t H, float* sumsq_out, float* sum_out, void* stream);
 /* nn.LayerNorm with affine, siglip.py:173-175,333.                                                */
 int cs_layernorm(const void* x, int64_t ldx, const void* w, const void* b, void* y, int64_t ldy,
                  int32_t rows, int32_t H, float eps, void* stream);

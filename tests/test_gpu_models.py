@@ -226,13 +226,13 @@ def test_qwen_errors_on_gpu(dev):
 
 
 # ------------------------------------------------------------------------------------------ Qwen2-VL
-def build_qwen2(dev, depth, seed, weight_format="bf16"):
+def build_qwen2(dev, depth, seed, weight_format="bf16", fold_norm=False):
     from cornserve_amd.eric.models.qwen2_vl import Qwen2VisionTransformer
     from oracle import qwen2_vl as o2
 
     cfg = synth.qwen2_vision_config(depth=depth)
     sd = synth.qwen2_state_dict(cfg, seed=seed)
-    model = Qwen2VisionTransformer(cfg, weight_format=weight_format)
+    model = Qwen2VisionTransformer(cfg, weight_format=weight_format, fold_norm=fold_norm)
     inc = model.load_state_dict(sd, strict=False)
     assert not inc.missing_keys and not inc.unexpected_keys
     return model.to(device=dev, dtype=torch.bfloat16).eval(), sd, o2.Qwen2VisionConfig(depth=depth), cfg
@@ -286,13 +286,13 @@ def test_qwen2_vl_ragged_frames_and_fp8(dev):
 
 
 # ------------------------------------------------------------------------------------------ Qwen3-VL
-def build_qwen3(dev, depth, deepstack, out, seed, weight_format="bf16"):
+def build_qwen3(dev, depth, deepstack, out, seed, weight_format="bf16", fold_norm=True):
     from cornserve_amd.eric.models.qwen3_vl import Qwen3_VisionTransformer
     from oracle import qwen3_vl as o3
 
     cfg = synth.qwen3_vision_config(depth=depth, deepstack_visual_indexes=deepstack, out_hidden_size=out)
     sd = synth.qwen3_state_dict(cfg, seed=seed)
-    model = Qwen3_VisionTransformer(cfg, weight_format=weight_format)
+    model = Qwen3_VisionTransformer(cfg, weight_format=weight_format, fold_norm=fold_norm)
     inc = model.load_state_dict(sd, strict=False)
     assert not inc.missing_keys and not inc.unexpected_keys
     ocfg = o3.Qwen3VisionConfig(depth=depth, deepstack_visual_indexes=list(deepstack), out_hidden_size=out)
@@ -349,12 +349,12 @@ def test_qwen3_vl_ragged_consecutive_deepstack_and_fp8(dev):
     check(out[0], o3.forward(sd_dq, ocfg8, px, grid, dtype=torch.float32)[0], REL_FP8, "qwen3-vl fp8 vs de-quantised fp32 oracle")
 
 
-def build_gemma(dev, layers, image_size, text_hidden, tokens, seed):
+def build_gemma(dev, layers, image_size, text_hidden, tokens, seed, fold_norm=False):
     from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
 
     cfg = synth.gemma3_config(layers, image_size, text_hidden, tokens)
     sd = synth.gemma3_state_dict(cfg, seed=seed)
-    model = Gemma3VisionEncoder(cfg).to(device=dev, dtype=torch.bfloat16).eval()
+    model = Gemma3VisionEncoder(cfg, fold_norm=fold_norm).to(device=dev, dtype=torch.bfloat16).eval()
     synth.load_gemma3(model, sd, adapter_name="a")
     ocfg = og.SiglipConfig(num_hidden_layers=layers, image_size=image_size, mm_tokens_per_image=tokens,
                            text_hidden_size=text_hidden)
@@ -385,3 +385,40 @@ def test_gemma3_real_resolution_and_crops(dev):
         check(out[i], ref[i], REL_BF16, f"gemma3 896 item {i}")
     with pytest.raises(ValueError, match="not found"):
         model(Modality.IMAGE, "missing", {"pixel_values": px, "num_crops": crops})
+
+
+def test_layernorm_encoders_without_folded_norms(dev):
+    """Qwen2-VL, Qwen3-VL and SigLIP with every LayerNorm as its own kernel (the reference's rounding points exactly)
+    against the oracles, and the distance between the folded and the unfolded forms."""
+    from oracle import qwen2_vl as o2
+    from oracle import qwen3_vl as o3
+
+    m_f, sd, ocfg, _ = build_qwen2(dev, 2, seed=21, fold_norm=True)
+    m_u, _, _, _ = build_qwen2(dev, 2, seed=21, fold_norm=False)
+    assert m_f.fold_norm and not m_u.fold_norm
+    px, grid = synth.qwen_inputs([(1, 16, 12), (2, 4, 6)], seed=21)
+    batch = {"pixel_values": px, "image_grid_thw": grid}
+    a, b = torch.cat(m_f(Modality.IMAGE, "", batch)), torch.cat(m_u(Modality.IMAGE, "", batch))
+    ref = torch.cat(o2.forward(sd, ocfg, px, grid, dtype=torch.bfloat16))
+    check(b, ref, REL_BF16, "qwen2-vl unfolded vs bf16 oracle")
+    check(a, b, REL_BF16, "qwen2-vl folded vs unfolded")
+
+    m_f, sd, ocfg, _ = build_qwen3(dev, 2, (0,), 512, seed=22)
+    m_u, _, _, _ = build_qwen3(dev, 2, (0,), 512, seed=22, fold_norm=False)
+    assert m_f.fold_norm and not m_u.fold_norm
+    px, grid = synth.qwen3_inputs([(1, 16, 12), (2, 4, 6)], seed=22)
+    batch = {"pixel_values": px, "image_grid_thw": grid}
+    a, b = torch.cat(m_f(Modality.IMAGE, "", batch)), torch.cat(m_u(Modality.IMAGE, "", batch))
+    ref = torch.cat(o3.forward(sd, ocfg, px, grid, dtype=torch.bfloat16))
+    check(b, ref, REL_BF16, "qwen3-vl unfolded vs bf16 oracle")
+    check(a, b, REL_BF16, "qwen3-vl folded vs unfolded")
+
+    m_f, sd, ocfg = build_gemma(dev, 2, 224, 640, 16, seed=23, fold_norm=True)
+    m_u, _, _ = build_gemma(dev, 2, 224, 640, 16, seed=23, fold_norm=False)
+    assert m_f.fold_norm and not m_u.fold_norm
+    px, crops = synth.gemma3_inputs(2, 224, seed=23)
+    a = torch.stack(m_f(Modality.IMAGE, "a", {"pixel_values": px, "num_crops": crops}))
+    b = torch.stack(m_u(Modality.IMAGE, "a", {"pixel_values": px, "num_crops": crops}))
+    ref = torch.stack(og.forward(sd, ocfg, px, crops, dtype=torch.bfloat16))
+    check(b.flatten(0, 1), ref.flatten(0, 1), REL_BF16, "siglip unfolded vs bf16 oracle")
+    check(a.flatten(0, 1), b.flatten(0, 1), REL_BF16, "siglip folded vs unfolded")

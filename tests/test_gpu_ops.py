@@ -349,6 +349,45 @@ def test_gemm_with_folded_rmsnorm(ops, dev, M, N, K):
         ops.gemm(a[:, :72].contiguous(), wf[:, :72].contiguous(), b, a_row_sumsq=ss, norm_eps=eps)   # K the fast kernel does not take
 
 
+@pytest.mark.parametrize("M,N,K", [(8192, 3456, 1152), (1000, 1280, 320), (300, 520, 448)])
+def test_gemm_with_folded_layernorm(ops, dev, M, N, K):
+    eps = 1e-6
+    a = (rnd((M, K), 2.0, 71).float() + 0.7).bfloat16().to(dev)          # rows with a non-zero mean
+    w, b = rnd((N, K), 0.05, 72, dev), rnd((N,), 0.02, 73, dev)
+    g, beta = (1.0 + rnd((K,), 0.1, 74)).bfloat16(), rnd((K,), 0.1, 75)
+    wf = (w.float().cpu() * g.float()[None, :]).bfloat16()                # norm weight folded into W's columns
+    bf = (b.float().cpu() + w.float().cpu() @ beta.float()).bfloat16()    # norm bias folded into the GEMM bias
+    csum = wf.float().sum(dim=1).contiguous()
+    ss = torch.empty((M, 8), dtype=torch.float32, device=dev)
+    sm = torch.empty_like(ss)
+    ops.row_stats(a, ss, sm)
+    torch.testing.assert_close(sm.cpu().sum(1), a.float().cpu().sum(1), rtol=1e-5, atol=1e-3)
+    rows = torch.cat([torch.arange(0, M, max(1, M // 257)), torch.tensor([M - 1])])
+    af = a[rows].float().cpu()
+    n_ref = F.layer_norm(af, (K,), g.float(), beta.float(), eps).bfloat16()     # the unfused reference sequence
+    base = lin_ref(n_ref, w, b).bfloat16().float()
+    for epi in (ops.EPI_BIAS, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU):
+        got = ops.gemm(a, wf.to(dev), bf.to(dev), epilogue=epi, a_row_sumsq=ss, a_row_sum=sm, w_col_sum=csum.to(dev), norm_eps=eps)
+        close(got[rows], _epilogue_ref(ops, epi, base, None), 2**-6, f"folded LayerNorm {M}x{N}x{K} epilogue {epi}")
+    unfused = ops.gemm(ops.layernorm(a, g.to(dev), beta.bfloat16().to(dev), eps), w, b)
+    fused = ops.gemm(a, wf.to(dev), bf.to(dev), a_row_sumsq=ss, a_row_sum=sm, w_col_sum=csum.to(dev), norm_eps=eps)
+    close(fused, unfused.float().cpu(), 2**-6, "folded vs layernorm + gemm")
+    with pytest.raises(RuntimeError):      # the mean term needs the column sums
+        ops.gemm(a, wf.to(dev), bf.to(dev), a_row_sumsq=ss, a_row_sum=sm, norm_eps=eps)
+    # producer side: a residual GEMM that also emits the sums of its output rows
+    if N <= 1280:
+        res = rnd((M, N), 1.0, 76, dev)
+        a2 = rnd((M, K), 1.0, 77, dev)
+        plain = ops.gemm(a2, w, b, epilogue=ops.EPI_RESIDUAL, residual=res)
+        s2, m2 = torch.zeros((M, 8), dtype=torch.float32, device=dev), torch.zeros((M, 8), dtype=torch.float32, device=dev)
+        got = ops.gemm(a2, w, b, epilogue=ops.EPI_RESIDUAL, residual=res, c_row_sumsq=s2, c_row_sum=m2)
+        assert torch.equal(got, plain)
+        torch.testing.assert_close(s2.cpu(), _sumsq_parts_ref(plain), rtol=1e-5, atol=1e-6)
+        pad = torch.zeros((M, 1280))
+        pad[:, :N] = plain.float().cpu()
+        torch.testing.assert_close(m2.cpu(), pad.view(M, 8, 160).sum(-1), rtol=1e-5, atol=1e-4)
+
+
 def test_gemm_row_maps(ops, dev):
     M, N, K = 400, 512, 256
     a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
