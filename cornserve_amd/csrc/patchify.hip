@@ -115,8 +115,8 @@ extern "C" int cs_qwen_patchify_u8(const void* frames, int32_t T, int32_t H, int
 extern "C" int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_t H, int32_t W, int32_t patch,
                                 void* out, int64_t ldo, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
-  if (!pixels || !out || B < 0 || C <= 0 || H <= 0 || W <= 0 || patch <= 0 || patch % 2 || H % patch ||
-      W % patch || ldo < (int64_t)C * patch * patch || ldo % 2 || (((uintptr_t)pixels | (uintptr_t)out) & 3))
+  if (!pixels || !out || B < 0 || C <= 0 || H <= 0 || W <= 0 || patch <= 0 || patch % 2 || H < patch ||
+      W < patch || W % 2 || ldo < (int64_t)C * patch * patch || ldo % 2 || (((uintptr_t)pixels | (uintptr_t)out) & 3))
     return CS_ERR_INVALID_ARG;
   if (B == 0) return CS_OK;
   const int64_t total = (int64_t)B * (H / patch) * C * patch * (W / patch);

@@ -119,6 +119,52 @@ __global__ __launch_bounds__(256) void pos_embed_interp_kernel(const bf16_t* __r
   *(bf16x8_t*)(out + (int64_t)(it.patch_base + pl) * ldo + c * 8) = o;
 }
 
+// Rows mixed from up to four source rows: LLaVA-OneVision's merge of per-tile features into one sequence
+// (eric/models/llava_onevision.py:78-153: tiles laid out as one grid, the padding cropped, large grids shrunk with
+// torch.nn.functional.interpolate(mode="bilinear"), a newline row behind every grid row) and its 2x pooling of video
+// frames (:169-183).  The caller turns that tensor program into, per output row, four source rows (y0x0, y0x1, y1x0,
+// y1x1) and the two fractions (ly, lx) of the interpolation; the value is
+//   (1-ly) * ((1-lx)*a00 + lx*a01) + ly * ((1-lx)*a10 + lx*a11)
+// in fp32 with no contraction, rounded once to bf16 (the form of torch's bilinear kernel on a GPU, which accumulates
+// bf16 inputs in fp32).  ly == lx == 0 copies row y0x0 bit for bit (crop, reorder, newline).  A tap outside
+// [0, n_src) gives a zero row instead of a stray read.  One thread per 8 channels of one output row.
+__global__ __launch_bounds__(256) void rows_bilinear_kernel(const bf16_t* __restrict__ src, int64_t lds, int n_src,
+                                                            const int32_t* __restrict__ taps,
+                                                            const float* __restrict__ frac, int n_rows, int E,
+                                                            bf16_t* __restrict__ out, int64_t ldo) {
+#pragma clang fp contract(off)
+  const int chunks = E >> 3;
+  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (int64_t)n_rows * chunks) return;
+  const int r = (int)(idx / chunks), c = (int)(idx - (int64_t)r * chunks);
+  const i32x4_t t = *(const i32x4_t*)(taps + 4 * (int64_t)r);
+  const float ly = frac[2 * (int64_t)r], lx = frac[2 * (int64_t)r + 1];
+  bf16_t* dst = out + (int64_t)r * ldo + c * 8;
+  bool ok = true;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) ok = ok && t[k] >= 0 && t[k] < n_src;
+  bf16x8_t o;
+  if (!ok) {
+#pragma unroll
+    for (int q = 0; q < 8; ++q) o[q] = f2bf(0.f);
+  } else if (ly == 0.f && lx == 0.f) {
+    o = *(const bf16x8_t*)(src + (int64_t)t[0] * lds + c * 8);
+  } else {
+    const bf16x8_t a00 = *(const bf16x8_t*)(src + (int64_t)t[0] * lds + c * 8);
+    const bf16x8_t a01 = *(const bf16x8_t*)(src + (int64_t)t[1] * lds + c * 8);
+    const bf16x8_t a10 = *(const bf16x8_t*)(src + (int64_t)t[2] * lds + c * 8);
+    const bf16x8_t a11 = *(const bf16x8_t*)(src + (int64_t)t[3] * lds + c * 8);
+    const float hy = 1.f - ly, hx = 1.f - lx;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const float top = hx * bf2f(a00[q]) + lx * bf2f(a01[q]);
+      const float bot = hx * bf2f(a10[q]) + lx * bf2f(a11[q]);
+      o[q] = f2bf(hy * top + ly * bot);
+    }
+  }
+  *(bf16x8_t*)dst = o;
+}
+
 template <typename V>
 __global__ __launch_bounds__(256) void row_gather_kernel(const char* __restrict__ in, int64_t in_stride,
                                                          const int32_t* __restrict__ rows,
@@ -263,6 +309,20 @@ extern "C" int cs_pos_embed_interp(const void* table, int32_t side, int32_t E, c
   const dim3 grid((unsigned)((work + 255) / 256), n_items), block(256);
   hipLaunchKernelGGL(pos_embed_interp_kernel, grid, block, 0, stream, (const bf16_t*)table, side, E,
                      (const ItemMeta*)item_meta, merge, (bf16_t*)out, ldo);
+  return cs_launch_status();
+}
+
+extern "C" int cs_rows_bilinear(const void* src, int64_t lds, int32_t n_src_rows, const int32_t* taps, const float* frac,
+                                int32_t n_rows, int32_t E, void* out, int64_t ldo, void* stream_) {
+  hipStream_t stream = (hipStream_t)stream_;
+  if (n_rows < 0 || n_src_rows < 0 || E <= 0 || E % 8 || lds < E || lds % 8 || ldo < E || ldo % 8) return CS_ERR_INVALID_ARG;
+  if (n_rows == 0) return CS_OK;
+  if (!src || !taps || !frac || !out || (((uintptr_t)src | (uintptr_t)out | (uintptr_t)taps) & 15) || ((uintptr_t)frac & 3))
+    return CS_ERR_INVALID_ARG;
+  const int64_t work = (int64_t)n_rows * (E / 8);
+  if ((work + 255) / 256 > 0x7fffffff) return CS_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(rows_bilinear_kernel, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, stream, (const bf16_t*)src,
+                     lds, n_src_rows, taps, frac, n_rows, E, (bf16_t*)out, ldo);
   return cs_launch_status();
 }
 

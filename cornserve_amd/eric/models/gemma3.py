@@ -82,25 +82,34 @@ class _EncoderLayer(nn.Module):
 
 
 class _Encoder(nn.Module):
-    def __init__(self, cfg: Any) -> None:
+    def __init__(self, cfg: Any, num_layers: int) -> None:
         super().__init__()
-        self.layers = nn.ModuleList(
-            [_EncoderLayer(cfg.hidden_size, cfg.intermediate_size) for _ in range(cfg.num_hidden_layers)]
-        )
+        self.layers = nn.ModuleList([_EncoderLayer(cfg.hidden_size, cfg.intermediate_size) for _ in range(num_layers)])
 
 
 class SiglipVisionTransformer(nn.Module):
-    def __init__(self, cfg: Any) -> None:
+    """The tower, optionally built only up to a feature layer and then without its final LayerNorm (reference:
+    siglip.py:301-335)."""
+
+    def __init__(self, cfg: Any, num_hidden_layers_override: int | None = None,
+                 require_post_norm: bool | None = None) -> None:
         super().__init__()
+        num_layers = cfg.num_hidden_layers if num_hidden_layers_override is None else num_hidden_layers_override
+        if num_layers > cfg.num_hidden_layers:
+            raise ValueError(f"The original encoder only has {cfg.num_hidden_layers} layers, "
+                             f"but you requested {num_layers} layers.")
         self.embeddings = _Embeddings(cfg)
-        self.encoder = _Encoder(cfg)
-        self.post_layernorm = _LN(cfg.hidden_size)
+        self.encoder = _Encoder(cfg, num_layers)
+        if require_post_norm is None:
+            require_post_norm = num_layers == cfg.num_hidden_layers
+        self.post_layernorm = _LN(cfg.hidden_size) if require_post_norm else None
 
 
 class SiglipVisionModel(nn.Module):
-    def __init__(self, cfg: Any) -> None:
+    def __init__(self, cfg: Any, num_hidden_layers_override: int | None = None,
+                 require_post_norm: bool | None = None) -> None:
         super().__init__()
-        self.vision_model = SiglipVisionTransformer(cfg)
+        self.vision_model = SiglipVisionTransformer(cfg, num_hidden_layers_override, require_post_norm)
 
 
 class Gemma3MultiModalProjector(nn.Module):
@@ -141,22 +150,15 @@ class Gemma3MultiModalProjectorAdapter(BaseAdapterModule):
         super().__init__(adapter_cls=Gemma3MultiModalProjector)
 
 
-class Gemma3VisionEncoder(EricModel):
-    def __init__(self, config: Any, fold_norm: bool = False) -> None:
-        """`fold_norm`: layer_norm1 / layer_norm2 of every SigLIP layer are applied inside the GEMM that follows them
-        (the norm's weight and bias are folded into that GEMM's weight and bias at pack time, mean and variance come
-        from row sums that the residual GEMMs emit): the normalised activations are not rounded to bf16 on their
-        own, unlike the reference (siglip.py:333-345), so results stay inside the parity tolerance but are not
-        bit-identical to fold_norm=False.  Off by default: the folded LayerNorm GEMM exists for the 256x160 tile only,
-        which costs the wide QKV and fc1 projections more than the norm kernels take (measured on 4 x 896x896 images:
-        25.6 against 24.8 ms)."""
-        super().__init__()
-        self.config = config
-        vc = config.vision_config
+class SiglipEncoderBase(EricModel):
+    """What the encoders built on the SigLIP tower share: the packed weights and the tower's launch sequence.
+    A subclass sets `self.config` (with `.vision_config`), `self.vision_tower` (a SiglipVisionModel) and calls
+    `_init_tower(fold_norm)`."""
+
+    def _init_tower(self, fold_norm: bool) -> None:
+        vc = self.config.vision_config
         self.fold_norm = (bool(fold_norm) and vc.hidden_size % 64 == 0 and 192 <= vc.hidden_size <= 160 * ops.SUMSQ_PARTS
                           and getattr(vc, "hidden_act", "gelu_pytorch_tanh") == "gelu_pytorch_tanh")
-        self.vision_tower = SiglipVisionModel(config.vision_config)
-        self.multi_modal_projector = Gemma3MultiModalProjectorAdapter()
         self._packed: dict | None = None
         self.register_load_state_dict_post_hook(lambda module, incompatible: setattr(module, "_packed", None))
 
@@ -168,17 +170,9 @@ class Gemma3VisionEncoder(EricModel):
     def device(self) -> torch.device:
         return self.vision_tower.vision_model.embeddings.patch_embedding.weight.device
 
-    @property
-    def chunk_shape(self) -> tuple[int, ...]:
-        # Same fixed chunking as the reference (gemma3.py:76-88): 256 divides 2560, 3840 and 5376.
-        return (1, self.config.mm_tokens_per_image, 256)
-
     def _apply(self, fn, recurse=True):
         self._packed = None
-        out = super()._apply(fn, recurse)
-        for adapter in self.multi_modal_projector.adapters.values():  # adapters sit outside _modules
-            adapter._apply(fn)
-        return out
+        return super()._apply(fn, recurse)
 
     @torch.no_grad()
     def _pack(self) -> dict:
@@ -226,7 +220,7 @@ class Gemma3VisionEncoder(EricModel):
             layers.append(entry)
         return {"pe_w": pe_w, "pe_b": vm.embeddings.patch_embedding.bias, "kp": kp, "ip": ip,
                 "pos": vm.embeddings.position_embedding.weight, "layers": layers,
-                "post": (vm.post_layernorm.weight, vm.post_layernorm.bias)}
+                "post": None if vm.post_layernorm is None else (vm.post_layernorm.weight, vm.post_layernorm.bias)}
 
     def _ensure_packed(self) -> dict:
         if self._packed is None:
@@ -239,7 +233,7 @@ class Gemma3VisionEncoder(EricModel):
         return self._packed
 
     def vision_tower_forward(self, pixel_values: torch.Tensor) -> torch.Tensor:
-        """pixel_values: bf16 [B,3,S,S] on the device -> [B, tokens, H] after post-layernorm."""
+        """pixel_values: bf16 [B,3,S,S] on the device -> [B, tokens, H] (after the post-layernorm if the tower has one)."""
         pk = self._ensure_packed()
         vc = self.config.vision_config
         H, nh = vc.hidden_size, vc.num_attention_heads
@@ -288,8 +282,37 @@ class Gemma3VisionEncoder(EricModel):
                 ops.layernorm(x, *lyr["ln2"], eps, out=n)
                 ops.gemm(n, *lyr["fc1"], epilogue=epi, out=hmid)
             ops.gemm(hmid, *lyr["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **stats_out)
+        if pk["post"] is None:
+            return x.view(B, tokens, H)
         ops.layernorm(x, *pk["post"], eps, out=n)
         return n.view(B, tokens, H)
+
+
+class Gemma3VisionEncoder(SiglipEncoderBase):
+    def __init__(self, config: Any, fold_norm: bool = False) -> None:
+        """`fold_norm`: layer_norm1 / layer_norm2 of every SigLIP layer are applied inside the GEMM that follows them
+        (the norm's weight and bias are folded into that GEMM's weight and bias at pack time, mean and variance come
+        from row sums that the residual GEMMs emit): the normalised activations are not rounded to bf16 on their
+        own, unlike the reference (siglip.py:333-345), so results stay inside the parity tolerance but are not
+        bit-identical to fold_norm=False.  Off by default: the folded LayerNorm GEMM exists for the 256x160 tile only,
+        which costs the wide QKV and fc1 projections more than the norm kernels take (measured on 4 x 896x896 images:
+        25.6 against 24.8 ms)."""
+        super().__init__()
+        self.config = config
+        self.vision_tower = SiglipVisionModel(config.vision_config)
+        self.multi_modal_projector = Gemma3MultiModalProjectorAdapter()
+        self._init_tower(fold_norm)
+
+    @property
+    def chunk_shape(self) -> tuple[int, ...]:
+        # Same fixed chunking as the reference (gemma3.py:76-88): 256 divides 2560, 3840 and 5376.
+        return (1, self.config.mm_tokens_per_image, 256)
+
+    def _apply(self, fn, recurse=True):
+        out = super()._apply(fn, recurse)
+        for adapter in self.multi_modal_projector.adapters.values():  # adapters sit outside _modules
+            adapter._apply(fn)
+        return out
 
     @torch.inference_mode()
     def forward(self, modality: Modality, adapter_name: str, batch: dict[str, list[torch.Tensor]]) -> list[torch.Tensor]:

@@ -79,6 +79,18 @@ MODEL_REGISTRY: dict[str, RegistryEntry] = {
         weight=WeightInfo(required_prefixes=["model.visual."], strip_prefixes=True),
         modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
     ),
+    "llava_onevision": RegistryEntry(
+        module="llava_onevision",
+        class_name="LlavaOneVisionEncoder",
+        adapter_attr=None,
+        vit_resolution_type=ViTResolutionType.FIXED,
+        weight=WeightInfo(
+            required_prefixes=["vision_tower.", "multi_modal_projector.", "image_newline"],
+            ignored_prefixes=["vision_tower.vision_model.post_layernorm"],
+            strip_prefixes=False,
+        ),
+        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
+    ),
     "gemma3": RegistryEntry(
         module="gemma3",
         class_name="Gemma3VisionEncoder",

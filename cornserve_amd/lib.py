@@ -77,6 +77,7 @@ _SIGNATURES: dict[str, list] = {
     ],
     "cs_row_gather": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p],
     "cs_pos_embed_interp": [c_void_p, c_int32, c_int32, c_void_p, c_int32, c_int32, c_int32, c_void_p, c_int64, c_void_p],
+    "cs_rows_bilinear": [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_int64, c_void_p],
     "cs_rope_qk": [c_void_p, c_int64, c_void_p, c_int32, c_int32, c_int32, c_void_p],
     "cs_attn_varlen": [
         c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,

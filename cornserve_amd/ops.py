@@ -309,6 +309,33 @@ def pos_embed_interp(table: torch.Tensor, item_meta: torch.Tensor, total_patches
     return out
 
 
+def rows_bilinear(src: torch.Tensor, taps: torch.Tensor, frac: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[r] = bilinear mix of the four rows taps[r] of src with the fractions frac[r] = (ly, lx); (0, 0) copies
+    row taps[r, 0].  src: bf16 [n, E] with contiguous rows, taps: int32 [R, 4], frac: fp32 [R, 2] (device tensors)."""
+    lib = _l.load()
+    _req(src, torch.bfloat16, "src")
+    _req(taps, torch.int32, "taps")
+    _req(frac, torch.float32, "frac")
+    if src.dim() != 2 or src.stride(1) != 1:
+        raise ValueError("src must be 2-D with contiguous rows")
+    R = taps.shape[0]
+    if taps.shape != (R, 4) or frac.shape != (R, 2) or not taps.is_contiguous() or not frac.is_contiguous():
+        raise ValueError("taps must be contiguous [R, 4] and frac contiguous [R, 2]")
+    E = src.shape[1]
+    if out is None:
+        out = torch.empty((R, E), dtype=torch.bfloat16, device=src.device)
+    else:
+        _req(out, torch.bfloat16, "out")
+        if out.shape != (R, E) or out.stride(1) != 1:
+            raise ValueError("out must be [R, E] with contiguous rows")
+    _l.check(
+        lib.cs_rows_bilinear(src.data_ptr(), src.stride(0), src.shape[0], taps.data_ptr(), frac.data_ptr(), R, E,
+                             out.data_ptr(), out.stride(0), _stream()),
+        "cs_rows_bilinear",
+    )
+    return out
+
+
 def row_gather(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
     """out[i] = x[rows[i]] for a 2-D tensor with contiguous rows."""
     lib = _l.load()
@@ -418,7 +445,8 @@ def qwen_patchify_u8(frames: torch.Tensor, table: torch.Tensor, patch: int, merg
 
 
 def patchify_nchw(pixels: torch.Tensor, patch: int, ldo: int) -> torch.Tensor:
-    """[B,C,H,W] bf16 -> [B*(H/p)*(W/p), ldo] rows of (c,ky,kx)-ordered patch values, zero padded."""
+    """[B,C,H,W] bf16 -> [B*(H//p)*(W//p), ldo] rows of (c,ky,kx)-ordered patch values, zero padded.  Pixels past the
+    last whole patch are dropped, as a convolution with stride = kernel and no padding drops them."""
     lib = _l.load()
     _req(pixels, torch.bfloat16, "pixels")
     if pixels.dim() != 4 or not pixels.is_contiguous():

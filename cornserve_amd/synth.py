@@ -216,9 +216,7 @@ def gemma3_config(num_hidden_layers: int = 27, image_size: int = 896, text_hidde
                            mm_tokens_per_image=mm_tokens_per_image, model_type="gemma3")
 
 
-def gemma3_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
-    """fp32 state dict with the checkpoint's names: `vision_tower.*` and `multi_modal_projector.*`."""
-    vc = config.vision_config
+def _siglip_tower_state_dict(vc, seed: int, post_norm: bool = True) -> dict[str, torch.Tensor]:
     H, I = vc.hidden_size, vc.intermediate_size
     VT = "vision_tower.vision_model."
     sd: dict[str, torch.Tensor] = {}
@@ -244,9 +242,19 @@ def gemma3_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
         mat(p + "mlp.fc1.bias", I)
         mat(p + "mlp.fc2.weight", H, I)
         mat(p + "mlp.fc2.bias", H)
-    ln(VT + "post_layernorm")
-    mat("multi_modal_projector.mm_input_projection_weight", H, config.text_config.hidden_size)
-    mat("multi_modal_projector.mm_soft_emb_norm.weight", H)
+    if post_norm:
+        ln(VT + "post_layernorm")
+    return sd
+
+
+def gemma3_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
+    """fp32 state dict with the checkpoint's names: `vision_tower.*` and `multi_modal_projector.*`."""
+    vc = config.vision_config
+    sd = _siglip_tower_state_dict(vc, seed)
+    sd["multi_modal_projector.mm_input_projection_weight"] = normal(
+        seed, "multi_modal_projector.mm_input_projection_weight", (vc.hidden_size, config.text_config.hidden_size), 0.02)
+    sd["multi_modal_projector.mm_soft_emb_norm.weight"] = normal(
+        seed, "multi_modal_projector.mm_soft_emb_norm.weight", (vc.hidden_size,), 0.02)
     return sd
 
 
@@ -271,3 +279,53 @@ def load_gemma3(model, sd: dict[str, torch.Tensor], adapter_name: str = "default
     inc = adapter.load_state_dict(ad, strict=False)
     if inc.missing_keys or inc.unexpected_keys:
         raise ValueError(f"Adapter weights mismatch: {inc}")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# LLaVA-OneVision (SigLIP tower without its last norm + two-layer projector + anyres merge)
+# ---------------------------------------------------------------------------------------------------------
+def llava_ov_config(num_hidden_layers: int = 26, image_size: int = 384, text_hidden: int = 3584,
+                    max_grid: int = 6) -> SimpleNamespace:
+    """llava-onevision-qwen2-7b-ov-hf: SigLIP-so400m at 384 px (27 x 27 patches a tile), 26 layers, every token kept."""
+    vc = SimpleNamespace(
+        hidden_size=1152, intermediate_size=4304, num_hidden_layers=num_hidden_layers, num_attention_heads=16,
+        num_channels=3, image_size=image_size, patch_size=14, layer_norm_eps=1e-6,
+        hidden_act="gelu_pytorch_tanh", attention_dropout=0.0, vision_use_head=False,
+    )
+    pinpoints = [[image_size * i, image_size * j] for i in range(1, max_grid + 1) for j in range(1, max_grid + 1)]
+    return SimpleNamespace(vision_config=vc, text_config=SimpleNamespace(hidden_size=text_hidden),
+                           vision_feature_layer=-1, vision_feature_select_strategy="full", projector_hidden_act="gelu",
+                           multimodal_projector_bias=True, image_grid_pinpoints=pinpoints,
+                           vision_aspect_ratio="anyres_max_9", model_type="llava_onevision")
+
+
+def llava_ov_state_dict(config, seed: int = 0) -> dict[str, torch.Tensor]:
+    """fp32 state dict with the checkpoint's names: `vision_tower.*`, `multi_modal_projector.*`, `image_newline`."""
+    vc = config.vision_config
+    T = config.text_config.hidden_size
+    sd = _siglip_tower_state_dict(vc, seed, post_norm=False)
+    for name, shape in (("linear_1.weight", (T, vc.hidden_size)), ("linear_1.bias", (T,)),
+                        ("linear_2.weight", (T, T)), ("linear_2.bias", (T,))):
+        sd["multi_modal_projector." + name] = normal(seed, "multi_modal_projector." + name, shape, 0.02)
+    sd["image_newline"] = normal(seed, "image_newline", (T,), 0.02)
+    return sd
+
+
+def llava_ov_image_inputs(config, sizes: list[tuple[int, int]], seed: int = 0) -> tuple[list[torch.Tensor], list[torch.Tensor]]:
+    """One entry per original image size (height, width): the base tile plus the tiles of the best-fitting grid, as
+    the Hugging Face image processor emits them (random pixels: only the shapes matter here)."""
+    from cornserve_amd.eric.models.llava_onevision import anyres_grid_shape
+
+    S = config.vision_config.image_size
+    px, szs = [], []
+    for i, (h, w) in enumerate(sizes):
+        th, tw = anyres_grid_shape((h, w), config.image_grid_pinpoints, S)
+        n = 1 + th * tw
+        px.append(uniform(seed, f"pixel_values.{i}", (n, 3, S, S), -1.0, 1.0))
+        szs.append(torch.tensor([h, w], dtype=torch.int64))
+    return px, szs
+
+
+def llava_ov_video_inputs(config, frames: list[int], seed: int = 0) -> list[torch.Tensor]:
+    S = config.vision_config.image_size
+    return [uniform(seed, f"pixel_values_videos.{i}", (n, 3, S, S), -1.0, 1.0) for i, n in enumerate(frames)]

@@ -181,6 +181,17 @@ int cs_rope_qk(void* qkv, int64_t ld, const float* cos_sin, int32_t L, int32_t h
 int cs_pos_embed_interp(const void* table, int32_t side, int32_t E, const int32_t* item_meta, int32_t n_items,
                         int32_t max_units_per_item, int32_t merge, void* out, int64_t ldo, void* stream);
 
+/* LLaVA-OneVision feature merge, llava_onevision.py:78-153 (`_merge_image_patch_embeddings`, strategy
+ * "spatial_unpad": tiles arranged as one grid, padding cropped, grids above the token budget shrunk with
+ * torch.nn.functional.interpolate(mode="bilinear"), one newline row behind every grid row) and :169-183
+ * (`apply_pooling`: bilinear 2x pooling of video frames).  The caller expresses either as one record per output row:
+ *   taps[r][4]  source rows (y0x0, y0x1, y1x0, y1x1) of src (bf16 [n_src_rows, lds]); frac[r][2] = (ly, lx)
+ *   out[r] = (1-ly) * ((1-lx)*src[t0] + lx*src[t1]) + ly * ((1-lx)*src[t2] + lx*src[t3])   fp32, one bf16 rounding
+ * and ly == lx == 0 copies src[t0] bit for bit.  A tap outside [0, n_src_rows) yields a zero row.  taps and frac are
+ * device arrays; E % 8 == 0.                                                                            */
+int cs_rows_bilinear(const void* src, int64_t lds, int32_t n_src_rows, const int32_t* taps, const float* frac,
+                     int32_t n_rows, int32_t E, void* out, int64_t ldo, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Variable-length non-causal attention: replaces flash_attn_varlen_func (qwen2_5_vl.py:110-120)
  * and xformers memory_efficient_attention_forward (attention.py:51).
@@ -204,7 +215,9 @@ int cs_attn_work_host(const int32_t* cu_seqlens_host, int32_t n_seg, int32_t blo
  * ---------------------------------------------------------------------------------------------- */
 /* Strided gather of non-overlapping patches (Conv2d k = s = patch, padding valid; siglip.py:30-36,
  * 94-95) from NCHW pixels [B,C,H,W] (bf16) into the GEMM operand [B*(H/p)*(W/p), ldo] with columns
- * ordered (c, ky, kx) and zero padding up to ldo.                                                 */
+ * ordered (c, ky, kx) and zero padding up to ldo.  H/p and W/p round down: pixels past the last whole
+ * patch are dropped, as the convolution drops them (384 / 14 = 27 patches a side for LLaVA-OneVision's
+ * tower).  patch and W must be even.                                                                */
 int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_t H, int32_t W, int32_t patch,
                      void* out, int64_t ldo, void* stream);
 /* The step before the Qwen2.5-VL encoder, for callers that hand over resized uint8 frames instead of float

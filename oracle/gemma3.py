@@ -66,7 +66,10 @@ def full_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, nh: int, s
     return out.transpose(1, 2).reshape(B, S, H).to(q.dtype)
 
 
-def vision_tower(sd: dict, cfg: SiglipConfig, pixel_values: torch.Tensor, dtype=torch.float32) -> torch.Tensor:
+def vision_tower(sd: dict, cfg: SiglipConfig, pixel_values: torch.Tensor, dtype=torch.float32,
+                 num_layers: int | None = None, post_norm: bool = True) -> torch.Tensor:
+    """`num_layers` / `post_norm`: a tower built only up to a feature layer, without the final LayerNorm
+    (siglip.py:301-335, as the LLaVA-family encoders build it, layers/vit.py:43-62)."""
     W = {k: v.to(dtype) for k, v in sd.items() if k.startswith(VT)}
     x = pixel_values.to(dtype)
     x = F.conv2d(x, W[VT + "embeddings.patch_embedding.weight"], W[VT + "embeddings.patch_embedding.bias"],
@@ -74,7 +77,7 @@ def vision_tower(sd: dict, cfg: SiglipConfig, pixel_values: torch.Tensor, dtype=
     x = x.flatten(2).transpose(1, 2)
     x = x + W[VT + "embeddings.position_embedding.weight"][None, : x.shape[1]]
     H, nh = cfg.hidden_size, cfg.num_attention_heads
-    for i in range(cfg.num_hidden_layers):
+    for i in range(cfg.num_hidden_layers if num_layers is None else num_layers):
         p = f"{VT}encoder.layers.{i}."
         h = F.layer_norm(x, (H,), W[p + "layer_norm1.weight"], W[p + "layer_norm1.bias"], cfg.layer_norm_eps)
         q = F.linear(h, W[p + "self_attn.q_proj.weight"], W[p + "self_attn.q_proj.bias"])
@@ -85,6 +88,8 @@ def vision_tower(sd: dict, cfg: SiglipConfig, pixel_values: torch.Tensor, dtype=
         h = F.layer_norm(x, (H,), W[p + "layer_norm2.weight"], W[p + "layer_norm2.bias"], cfg.layer_norm_eps)
         h = F.gelu(F.linear(h, W[p + "mlp.fc1.weight"], W[p + "mlp.fc1.bias"]), approximate="tanh")
         x = x + F.linear(h, W[p + "mlp.fc2.weight"], W[p + "mlp.fc2.bias"])
+    if not post_norm:
+        return x
     return F.layer_norm(x, (H,), W[VT + "post_layernorm.weight"], W[VT + "post_layernorm.bias"], cfg.layer_norm_eps)
 
 

@@ -213,9 +213,95 @@ def make_gemma3_small() -> None:
     print("gemma3_small.npz", out.shape, float(np.abs(out).mean()))
 
 
+def _hf_llava_onevision(cfg):
+    """The installed Hugging Face LlavaOnevisionModel with `cfg`'s vision tower and a minimal language model (unused)."""
+    from transformers.models.llava_onevision.configuration_llava_onevision import LlavaOnevisionConfig
+    from transformers.models.llava_onevision.modeling_llava_onevision import LlavaOnevisionModel
+    from transformers.models.qwen2.configuration_qwen2 import Qwen2Config
+    from transformers.models.siglip.configuration_siglip import SiglipVisionConfig
+
+    vc = cfg.vision_config
+    hf_vc = SiglipVisionConfig(
+        hidden_size=vc.hidden_size, intermediate_size=vc.intermediate_size, num_hidden_layers=vc.num_hidden_layers,
+        num_attention_heads=vc.num_attention_heads, image_size=vc.image_size, patch_size=vc.patch_size,
+        hidden_act=vc.hidden_act, layer_norm_eps=vc.layer_norm_eps, vision_use_head=False,
+    )
+    text = Qwen2Config(hidden_size=cfg.text_config.hidden_size, intermediate_size=64, num_hidden_layers=1,
+                       num_attention_heads=2, num_key_value_heads=2, vocab_size=64)
+    hf_cfg = LlavaOnevisionConfig(
+        vision_config=hf_vc, text_config=text, vision_feature_layer=cfg.vision_feature_layer,
+        vision_feature_select_strategy=cfg.vision_feature_select_strategy, projector_hidden_act=cfg.projector_hidden_act,
+        image_grid_pinpoints=cfg.image_grid_pinpoints, vision_aspect_ratio=cfg.vision_aspect_ratio,
+        multimodal_projector_bias=cfg.multimodal_projector_bias,
+    )
+    hf_cfg._attn_implementation = "sdpa"
+    return LlavaOnevisionModel(hf_cfg).float().eval()
+
+
+def hf_llava_onevision_forward(cfg, sd, px, sizes, videos):
+    """(per-image sequences, per-video sequences) from the Hugging Face implementation."""
+    model = _hf_llava_onevision(cfg)
+    own = model.state_dict()
+    flat_tower = not any(k.startswith("vision_tower.vision_model.") for k in own)
+    mapped = {}
+    for k, v in sd.items():
+        if flat_tower and k.startswith("vision_tower.vision_model."):
+            k = "vision_tower." + k[len("vision_tower.vision_model."):]
+        mapped[k] = v
+    inc = model.load_state_dict(mapped, strict=False)
+    bad = [k for k in inc.missing_keys if not k.startswith("language_model.") and "post_layernorm" not in k
+           and ".head." not in k]
+    assert not bad and not inc.unexpected_keys, (bad, inc.unexpected_keys)
+    S = cfg.vision_config.image_size
+    with torch.no_grad():
+        # images: padded to the largest tile count, as the Hugging Face processor batches them
+        most = max(p.shape[0] for p in px)
+        batch = torch.zeros(len(px), most, 3, S, S)
+        for i, p in enumerate(px):
+            batch[i, : p.shape[0]] = p
+        image_sizes = torch.stack(sizes)
+        out = model.get_image_features(pixel_values=batch, image_sizes=image_sizes)
+        feats = out.pooler_output if hasattr(out, "pooler_output") else out
+        feats = [f[: p.shape[0]] for f, p in zip(feats, px)] if isinstance(feats, (list, tuple)) and feats[0].dim() == 3 else feats
+        if isinstance(feats, (list, tuple)) and feats[0].dim() == 3:
+            images, _ = model.pack_image_features(list(feats), image_sizes, image_newline=model.image_newline,
+                                                  vision_aspect_ratio=cfg.vision_aspect_ratio)
+        else:  # this version already packs inside get_image_features
+            images = list(feats)
+        vids = []
+        for v in videos:
+            vo = model.get_video_features(pixel_values=v[None])
+            vf = vo.pooler_output if hasattr(vo, "pooler_output") else vo
+            vf = vf.reshape(1, -1, vf.shape[-1])
+            vids.append(torch.cat([vf, model.image_newline[None, None, :]], dim=1))
+    return [t.float() for t in images], [t.float() for t in vids]
+
+
+LLAVA_OV_SMALL_SIZES = [(70, 70), (100, 260), (280, 280), (211, 277), (277, 90)]
+LLAVA_OV_SMALL_FRAMES = [2, 3]
+
+
+def llava_onevision_small_case():
+    cfg = synth.llava_ov_config(num_hidden_layers=2, image_size=70, text_hidden=256, max_grid=4)
+    sd = synth.llava_ov_state_dict(cfg, seed=5)
+    px, sizes = synth.llava_ov_image_inputs(cfg, LLAVA_OV_SMALL_SIZES, seed=5)
+    videos = synth.llava_ov_video_inputs(cfg, LLAVA_OV_SMALL_FRAMES, seed=5)
+    return cfg, sd, px, sizes, videos
+
+
+def make_llava_onevision_small() -> None:
+    cfg, sd, px, sizes, videos = llava_onevision_small_case()
+    images, vids = hf_llava_onevision_forward(cfg, sd, px, sizes, videos)
+    arrays = {f"image{i}": t.numpy().astype(np.float32) for i, t in enumerate(images)}
+    arrays.update({f"video{i}": t.numpy().astype(np.float32) for i, t in enumerate(vids)})
+    np.savez_compressed(HERE / "llava_onevision_small.npz", seed=np.int64(5), **arrays)
+    print("llava_onevision_small.npz", [a.shape for a in arrays.values()])
+
+
 if __name__ == "__main__":
     make_index()
     make_qwen_cfg1()
     make_qwen2_vl_small()
     make_qwen3_vl_small()
     make_gemma3_small()
+    make_llava_onevision_small()

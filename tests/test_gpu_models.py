@@ -422,3 +422,78 @@ def test_layernorm_encoders_without_folded_norms(dev):
     ref = torch.stack(og.forward(sd, ocfg, px, crops, dtype=torch.bfloat16))
     check(b.flatten(0, 1), ref.flatten(0, 1), REL_BF16, "siglip unfolded vs bf16 oracle")
     check(a.flatten(0, 1), b.flatten(0, 1), REL_BF16, "siglip folded vs unfolded")
+
+
+# ---------------------------------------------------------------------------------------------------------
+# LLaVA-OneVision
+# ---------------------------------------------------------------------------------------------------------
+def build_llava(dev, layers, image_size, text_hidden, seed, max_grid=4, fold_norm=False):
+    from cornserve_amd.eric.models.llava_onevision import LlavaOneVisionEncoder
+    from oracle import llava_onevision as ol
+
+    cfg = synth.llava_ov_config(layers, image_size, text_hidden, max_grid=max_grid)
+    sd = synth.llava_ov_state_dict(cfg, seed=seed)
+    model = LlavaOneVisionEncoder(cfg, fold_norm=fold_norm).to(device=dev, dtype=torch.bfloat16).eval()
+    model.load_state_dict(sd)
+    ocfg = ol.LlavaOneVisionConfig(vision=og.SiglipConfig(num_hidden_layers=layers, image_size=image_size),
+                                   text_hidden_size=text_hidden, image_grid_pinpoints=cfg.image_grid_pinpoints)
+    return model, sd, cfg, ocfg
+
+
+def test_llava_onevision_small_against_oracle_and_golden(dev, golden_dir):
+    from oracle import llava_onevision as ol
+
+    model, sd, cfg, ocfg = build_llava(dev, 2, 70, 256, seed=5)
+    sizes = [(70, 70), (100, 260), (280, 280), (211, 277), (277, 90)]
+    px, szs = synth.llava_ov_image_inputs(cfg, sizes, seed=5)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_sizes": szs})
+    assert [tuple(o.shape) for o in out] == [(55, 256), (193, 256), (265, 256), (246, 256), (165, 256)]
+    assert all(o.dtype == torch.bfloat16 for o in out)
+    ref = ol.forward_images(sd, ocfg, px, szs, dtype=torch.bfloat16)
+    gold = np.load(golden_dir / "llava_onevision_small.npz")
+    for i, o in enumerate(out):
+        check(o, ref[i], REL_BF16, f"llava-onevision small image {i} vs bf16 oracle")
+        check(o, torch.from_numpy(gold[f"image{i}"]), REL_BF16, f"llava-onevision small image {i} vs golden")
+    # the newline rows are the parameter itself, bit for bit
+    nl = model.image_newline.cpu()
+    assert torch.equal(out[0][-1].cpu(), nl) and torch.equal(out[1][25 + 20].cpu(), nl)
+    videos = synth.llava_ov_video_inputs(cfg, [2, 3], seed=5)
+    vout = model(Modality.VIDEO, "", {"pixel_values_videos": videos})
+    assert [tuple(v.shape) for v in vout] == [(1, 19, 256), (1, 28, 256)]
+    vref = ol.forward_videos(sd, ocfg, videos, dtype=torch.bfloat16)
+    for i, v in enumerate(vout):
+        check(v[0], vref[i][0], REL_BF16, f"llava-onevision small video {i} vs bf16 oracle")
+        check(v[0], torch.from_numpy(gold[f"video{i}"][0]), REL_BF16, f"llava-onevision small video {i} vs golden")
+    # an item's result does not depend on what else is in the batch
+    alone = model(Modality.IMAGE, "", {"pixel_values": px[3:4], "image_sizes": szs[3:4]})
+    assert torch.equal(alone[0], out[3])
+    # padded tile lists (the batch dimension of the Hugging Face processor) use the leading tiles
+    padded = torch.cat([px[1], torch.zeros(3, 3, 70, 70)])
+    again = model(Modality.IMAGE, "", {"pixel_values": [padded], "image_sizes": szs[1:2]})
+    assert torch.equal(again[0], out[1])
+
+
+def test_llava_onevision_real_tile_size_images_and_video(dev):
+    """384-pixel tiles (27 x 27 tokens, 6 pixels of every side dropped by the patch convolution), 3 layers, width 3584:
+    a small image (1x1 grid), a wide one (cropped grid) and one above the token budget (shrunk grid); a 4-frame video."""
+    from oracle import llava_onevision as ol
+
+    model, sd, cfg, ocfg = build_llava(dev, 3, 384, 3584, seed=9, max_grid=6)
+    sizes = [(300, 380), (500, 1100), (1500, 1400)]
+    px, szs = synth.llava_ov_image_inputs(cfg, sizes, seed=9)
+    assert [p.shape[0] for p in px] == [2, 7, 17]
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_sizes": szs})
+    ref = ol.forward_images(sd, ocfg, px, szs, dtype=torch.bfloat16)
+    assert [tuple(o.shape) for o in out] == [tuple(r.shape) for r in ref]
+    for i, o in enumerate(out):
+        check(o, ref[i], REL_BF16, f"llava-onevision 384 image {i}")
+    videos = synth.llava_ov_video_inputs(cfg, [4], seed=9)
+    vout = model(Modality.VIDEO, "", {"pixel_values_videos": videos})
+    vref = ol.forward_videos(sd, ocfg, videos, dtype=torch.bfloat16)
+    assert tuple(vout[0].shape) == (1, 4 * 196 + 1, 3584)
+    check(vout[0][0], vref[0][0], REL_BF16, "llava-onevision 384 video")
+    folded, _, _, _ = build_llava(dev, 3, 384, 3584, seed=9, max_grid=6, fold_norm=True)
+    assert folded.fold_norm
+    fout = folded(Modality.IMAGE, "", {"pixel_values": px[:2], "image_sizes": szs[:2]})
+    for i in range(2):
+        check(fout[i], ref[i], REL_BF16, f"llava-onevision 384 image {i}, folded norms")

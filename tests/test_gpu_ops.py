@@ -460,6 +460,7 @@ def attn_ref(qkv, cu, nh, d, cos_sin=None):
     (96, [0, 200, 265]),
     (72, [0, 4096]),                        # one SigLIP image: 64 key tiles through the three-buffer ring
     (72, [0, 65, 129, 322]),                # one, two and three key tiles
+    (72, [0, 729, 1458, 2187]),             # LLaVA-OneVision tiles: 27 x 27 tokens each
 ])
 def test_attention(ops, dev, d, cu):
     nh, L = 16, cu[-1]
@@ -596,3 +597,62 @@ def test_attention_invariants_at_full_size(ops, dev):
     plan = ops.attn_plan(cu, dev)
     out = ops.attn_varlen(qkv[:256, :H], qkv[:256, H:2 * H], qkv[:256, 2 * H:], plan, nh, d, d**-0.5)
     assert torch.equal(out, qkv[:256, 2 * H:])
+
+
+# ------------------------------------------------------------------------------- weighted row gather
+def test_rows_bilinear_bit_exact(ops, dev):
+    """cs_rows_bilinear against the same formula in numpy fp32 (no fused multiply-add on either side): identical bits.
+    Copy rows (both fractions zero) keep the source bits, signed zeros and infinities included."""
+    n_src, E, R = 300, 3584, 1000
+    src = rnd((n_src, E), 1.0, 71)
+    src[5, :8] = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), 1.0, -1.0, 3.0e38, -3.0e38]).bfloat16()
+    rng = np.random.default_rng(5)
+    taps = rng.integers(0, n_src, size=(R, 4)).astype(np.int32)
+    taps[taps == 5] = 6        # row 5 (special values) is only ever copied
+    frac = rng.random((R, 2)).astype(np.float32)
+    frac[::7] = 0.0            # copies
+    taps[0] = 5                # the row with the special values
+    frac[3, 0] = 0.0           # one fraction zero is still an interpolation
+    taps[11] = [0, n_src, 1, 2]        # a tap past the source: zero row, no stray read
+    taps[12] = [-1, 0, 1, 2]
+    frac[11] = frac[12] = 0.5
+    got = ops.rows_bilinear(src.to(dev), torch.from_numpy(taps).to(dev), torch.from_numpy(frac).to(dev)).cpu()
+    s32 = src.float().numpy()
+    ok = ((taps >= 0) & (taps < n_src)).all(axis=1)
+    t = np.where(ok[:, None], taps, 0)
+    a = [s32[t[:, k]] for k in range(4)]
+    ly, lx = frac[:, 0:1], frac[:, 1:2]
+    hy, hx = np.float32(1) - ly, np.float32(1) - lx
+    with np.errstate(all="ignore"):
+        ref = hy * (hx * a[0] + lx * a[1]) + ly * (hx * a[2] + lx * a[3])
+    copy = (frac == 0).all(axis=1)
+    ref[copy] = a[0][copy]
+    ref[~ok] = 0.0
+    ref = torch.from_numpy(ref).bfloat16()
+    assert got.dtype == torch.bfloat16 and got.shape == (R, E)
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+    assert torch.equal(got[0].view(torch.int16), src[5].view(torch.int16))
+    # strided source and destination rows
+    wide = torch.zeros((n_src, E + 64), dtype=torch.bfloat16, device=dev)
+    wide[:, :E] = src.to(dev)
+    out = torch.full((R, E + 8), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.rows_bilinear(wide[:, :E], torch.from_numpy(taps).to(dev), torch.from_numpy(frac).to(dev), out=out[:, :E])
+    assert torch.equal(out[:, :E].cpu().view(torch.int16), ref.view(torch.int16)) and bool((out[:, E:] == 7.0).all())
+    empty = ops.rows_bilinear(src.to(dev), torch.zeros((0, 4), dtype=torch.int32, device=dev),
+                              torch.zeros((0, 2), dtype=torch.float32, device=dev))
+    assert empty.shape == (0, E)
+    with pytest.raises(ValueError):
+        ops.rows_bilinear(src.to(dev), torch.zeros((4, 3), dtype=torch.int32, device=dev),
+                          torch.zeros((4, 2), dtype=torch.float32, device=dev))
+    with pytest.raises(ValueError, match="invalid argument"):      # rows of 3580 values: not whole 16-byte vectors
+        ops.rows_bilinear(src.to(dev)[:, :E - 4], torch.zeros((4, 4), dtype=torch.int32, device=dev),
+                          torch.zeros((4, 2), dtype=torch.float32, device=dev))
+
+
+def test_patchify_nchw_drops_the_partial_patches(ops, dev):
+    """384 = 27 * 14 + 6: a convolution with stride = kernel and no padding ignores the last 6 rows and columns."""
+    px = rnd((3, 3, 384, 384), 1.0, 72)
+    got = ops.patchify_nchw(px.to(dev), 14, 592).cpu()
+    ref = F.unfold(px.float()[:, :, :378, :378], kernel_size=14, stride=14).transpose(1, 2).reshape(3 * 729, 588)
+    assert got.shape == (3 * 729, 592)
+    assert torch.equal(got[:, :588].float(), ref) and not got[:, 588:].any()

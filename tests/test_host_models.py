@@ -2,6 +2,7 @@
 
 import importlib
 
+import numpy as np
 import pytest
 import torch
 
@@ -13,7 +14,7 @@ from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
 
 
 def test_registry_resolves_like_the_reference_loader():
-    for model_type in ("qwen2_5_vl", "gemma3"):
+    for model_type in registry.MODEL_REGISTRY:
         entry = registry.MODEL_REGISTRY[model_type]
         module = importlib.import_module(f"cornserve_amd.eric.models.{entry.module}")
         cls = getattr(module, entry.class_name)
@@ -270,3 +271,94 @@ def test_load_model_from_local_checkpoint(tmp_path):
     w0 = adapters[str(tmp_path / "gemma")].mm_input_projection_weight
     w1 = adapters[str(tmp_path / "gemma_ft")].mm_input_projection_weight
     assert torch.equal(w0, gsd["multi_modal_projector.mm_input_projection_weight"]) and torch.equal(w1, w0 + 1)
+
+
+def test_llava_onevision_names_plans_and_errors():
+    from cornserve_amd.eric.models import llava_onevision as lv
+    from oracle import gemma3 as og
+    from oracle import llava_onevision as ol
+
+    cfg = synth.llava_ov_config(num_hidden_layers=2, image_size=70, text_hidden=64, max_grid=4)
+    model = lv.LlavaOneVisionEncoder(cfg)
+    sd = synth.llava_ov_state_dict(cfg, seed=0)
+    assert set(model.state_dict().keys()) == set(sd)        # no post_layernorm: the tower stops at the feature layer
+    model.load_state_dict(sd)
+    assert model.chunk_shape == (1, 64) and model.dtype == torch.float32
+    cfg2 = synth.llava_ov_config(num_hidden_layers=3, image_size=70, text_hidden=64)
+    cfg2.vision_feature_layer = -2
+    assert len(lv.LlavaOneVisionEncoder(cfg2).vision_tower.vision_model.encoder.layers) == 2
+    cfg2.vision_feature_layer = [1, -1]
+    assert len(lv.LlavaOneVisionEncoder(cfg2).vision_tower.vision_model.encoder.layers) == 3
+    cfg2.vision_feature_layer = "last"
+    with pytest.raises(TypeError):
+        lv.LlavaOneVisionEncoder(cfg2)
+
+    # the gather records, applied on the host, are the reference's merge (restated by the oracle) bit for bit
+    ocfg = ol.LlavaOneVisionConfig(vision=og.SiglipConfig(num_hidden_layers=2, image_size=70), text_hidden_size=64,
+                                   image_grid_pinpoints=cfg.image_grid_pinpoints)
+
+    def apply(src, taps, frac):
+        a = [src[taps[:, k]].astype(np.float32) for k in range(4)]
+        ly, lx = frac[:, 0:1], frac[:, 1:2]
+        hy, hx = np.float32(1) - ly, np.float32(1) - lx
+        return hy * (hx * a[0] + lx * a[1]) + ly * (hx * a[2] + lx * a[3])
+
+    rng = np.random.default_rng(0)
+    sizes = [(70, 70), (100, 260), (280, 280), (211, 277), (280, 140), (50, 300), (277, 90), (139, 141), (33, 280)]
+    sizes += [(int(h), int(w)) for h, w in rng.integers(10, 600, size=(40, 2)) if max(h, w) / min(h, w) < 20]
+    shrunk = 0
+    for h, w in sizes:
+        th, tw = lv.anyres_grid_shape((h, w), cfg.image_grid_pinpoints, 70)
+        n = 1 + th * tw
+        feats = rng.standard_normal((7 + n * 25 + 1, 8)).astype(np.float32)    # 7 rows of another item in front
+        taps, frac = lv.image_merge_plan(n, (h, w), 7, 7 + n * 25, 5, cfg.image_grid_pinpoints, 70)
+        assert taps.min() >= 7 and taps.max() <= 7 + n * 25
+        ref = ol.merge_image(ocfg, torch.from_numpy(feats[7:-1]).view(n, 25, 8), (h, w), torch.from_numpy(feats[-1]))
+        assert np.array_equal(apply(feats, taps, frac), ref.numpy()), (h, w)
+        shrunk += bool((frac != 0).any())
+    assert shrunk >= 5
+    # padded tile lists (more tiles than the grid needs) use the leading ones; too few are an error
+    taps_a, _ = lv.image_merge_plan(9, (100, 260), 0, 500, 5, cfg.image_grid_pinpoints, 70)
+    taps_b, _ = lv.image_merge_plan(12, (100, 260), 0, 500, 5, cfg.image_grid_pinpoints, 70)
+    assert np.array_equal(taps_a, taps_b)
+    with pytest.raises(RuntimeError, match="needs 8 tiles"):
+        lv.image_merge_plan(5, (100, 260), 0, 500, 5, cfg.image_grid_pinpoints, 70)
+    taps, frac = lv.image_merge_plan(1, (70, 70), 3, 99, 5, cfg.image_grid_pinpoints, 70)
+    assert taps[:, 0].tolist() == list(range(3, 28)) + [99] and not frac.any()
+    with pytest.raises(ValueError, match="not consistent"):
+        lv.image_merge_plan(2, (70, 70), 0, 48, 5, cfg.image_grid_pinpoints, 70, tokens_per_tile=24)
+
+    feats = rng.standard_normal((3 * 25 + 1, 8)).astype(np.float32)
+    taps, frac = lv.video_pool_plan(3, 0, 75, 5)
+    ref = ol.pool_video(ocfg, torch.from_numpy(feats[:-1]).view(3, 25, 8), torch.from_numpy(feats[-1]))
+    assert np.array_equal(apply(feats, taps, frac), ref[0].numpy())
+
+    px, szs = synth.llava_ov_image_inputs(cfg, [(70, 70)])
+    with pytest.raises(ValueError, match="Unsupported modality"):
+        model(Modality.AUDIO, "", {"pixel_values": px, "image_sizes": szs})
+    with pytest.raises(AssertionError):
+        model(Modality.IMAGE, "", {"pixel_values": [torch.zeros(2, 3, 56, 56)], "image_sizes": szs})
+    with pytest.raises(AssertionError):
+        model(Modality.IMAGE, "", {"pixel_values": px, "image_sizes": szs + szs})
+    with pytest.raises(RuntimeError, match="one frame"):
+        model(Modality.VIDEO, "", {"pixel_values_videos": synth.llava_ov_video_inputs(cfg, [1])})
+    with pytest.raises(RuntimeError, match="no CPU path"):     # the kernels are the only implementation
+        model(Modality.IMAGE, "", {"pixel_values": px, "image_sizes": szs})
+
+
+def test_load_llava_onevision_from_local_checkpoint(tmp_path):
+    from cornserve_amd.eric.loader import load_model
+    from cornserve_amd.eric.models.llava_onevision import LlavaOneVisionEncoder
+
+    cfg = synth.llava_ov_config(num_hidden_layers=2, image_size=70, text_hidden=64, max_grid=2)
+    sd = synth.llava_ov_state_dict(cfg, seed=6)
+    ckpt = dict(sd)
+    ckpt["language_model.embed.weight"] = torch.zeros(3, 3)
+    ckpt["vision_tower.vision_model.post_layernorm.weight"] = torch.ones(1152)    # in the checkpoint, not in the model
+    ckpt["vision_tower.vision_model.post_layernorm.bias"] = torch.zeros(1152)
+    _write_checkpoint(tmp_path / "llava", cfg, ckpt)
+    model = load_model(tmp_path / "llava", torch_device=torch.device("cpu"))
+    assert isinstance(model, LlavaOneVisionEncoder) and not model.training
+    assert torch.equal(model.image_newline, sd["image_newline"])
+    assert torch.equal(model.multi_modal_projector.linear_2.weight, sd["multi_modal_projector.linear_2.weight"])
+    assert model.config.image_grid_pinpoints == cfg.image_grid_pinpoints

@@ -233,3 +233,97 @@ def test_qwen3_vl_position_interpolation_closed_forms():
     want = [3.0 * hs[by * 2 + my] + 0.5 * ws[bx * 2 + mx] for by in range(2) for bx in range(5) for my in range(2) for mx in range(2)]
     assert got.shape == (80, E) and torch.allclose(got[:40, 0], torch.stack(want), atol=1e-5)
     assert torch.equal(got[:40], got[40:])                       # repeated per frame
+
+
+# ---------------------------------------------------------------------------------------------------------
+# LLaVA-OneVision (oracle/llava_onevision.py)
+# ---------------------------------------------------------------------------------------------------------
+def _llava_small():
+    from oracle import llava_onevision as ol
+
+    cfg = synth.llava_ov_config(num_hidden_layers=2, image_size=70, text_hidden=256, max_grid=4)
+    ocfg = ol.LlavaOneVisionConfig(vision=og.SiglipConfig(num_hidden_layers=2, image_size=70), text_hidden_size=256,
+                                   image_grid_pinpoints=cfg.image_grid_pinpoints)
+    return ol, cfg, ocfg
+
+
+def test_llava_onevision_small_against_golden(golden_dir):
+    """Five images (one tile grid each of 1x1, 2x4, 4x4 shrunk, 4x4 cropped and shrunk, 4x2 cropped) and two videos."""
+    ol, cfg, ocfg = _llava_small()
+    gold = np.load(golden_dir / "llava_onevision_small.npz")
+    seed = int(gold["seed"])
+    sd = synth.llava_ov_state_dict(cfg, seed=seed)
+    sizes = [(70, 70), (100, 260), (280, 280), (211, 277), (277, 90)]
+    px, szs = synth.llava_ov_image_inputs(cfg, sizes, seed=seed)
+    out = ol.forward_images(sd, ocfg, px, szs)
+    assert [tuple(o.shape) for o in out] == [(55, 256), (193, 256), (265, 256), (246, 256), (165, 256)]
+    for i, o in enumerate(out):
+        g = gold[f"image{i}"]
+        assert np.abs(o.numpy() - g).max() <= 2e-4 * np.abs(g).max(), i
+    vids = ol.forward_videos(sd, ocfg, synth.llava_ov_video_inputs(cfg, [2, 3], seed=seed))
+    assert [tuple(v.shape) for v in vids] == [(1, 19, 256), (1, 28, 256)]
+    for i, v in enumerate(vids):
+        g = gold[f"video{i}"]
+        assert np.abs(v.numpy() - g).max() <= 2e-4 * np.abs(g).max(), i
+    with pytest.raises(RuntimeError, match="one frame"):
+        ol.forward_videos(sd, ocfg, synth.llava_ov_video_inputs(cfg, [1], seed=seed))
+
+
+def test_llava_onevision_geometry_against_installed_package():
+    """select_best_resolution / get_anyres_image_grid_shape / unpad_image as the third-party package computes them."""
+    m = pytest.importorskip("transformers.models.llava_onevision.modeling_llava_onevision")
+    ol, cfg, _ = _llava_small()
+    pins = [[384 * i, 384 * j] for i in range(1, 7) for j in range(1, 7)]
+    rng = np.random.default_rng(3)
+    sizes = [(int(h), int(w)) for h, w in rng.integers(20, 3000, size=(300, 2))]
+    sizes += [(384, 384), (385, 384), (2304, 2304), (768, 383), (1, 200), (199, 1), (1000, 1001)]
+    for h, w in sizes:
+        th, tw = ol.anyres_grid_shape((h, w), pins, 384)
+        assert (th, tw) == tuple(m.get_anyres_image_grid_shape((h, w), pins, 384)), (h, w)
+        ch, cw = th * 27, tw * 27
+        marks = torch.arange(ch * cw, dtype=torch.float32).view(1, ch, cw)
+        kept = m.unpad_image(marks, (h, w))
+        y0, y1, x0, x1 = ol.unpad_bounds(ch, cw, h, w)
+        assert torch.equal(kept, marks[:, y0:y1, x0:x1]), (h, w)
+
+
+def test_llava_onevision_bilinear_resize_is_torch_interpolate():
+    from oracle import llava_onevision as ol
+
+    torch.manual_seed(0)
+    for (h, w), (oh, ow) in [((27, 27), (14, 14)), ((108, 81), (93, 70)), ((5, 9), (5, 4)), ((20, 20), (17, 17)),
+                             ((162, 54), (141, 47)), ((3, 3), (7, 5))]:
+        x = torch.randn(6, h, w)
+        ref = F.interpolate(x[None], [oh, ow], mode="bilinear")[0]
+        got = ol.bilinear_resize(x, oh, ow)
+        assert torch.allclose(got, ref, rtol=0, atol=2e-5), ((h, w), (oh, ow), (got - ref).abs().max())  # fp32 rounding
+    # a resize to the same size is the identity; a constant stays constant
+    x = torch.randn(3, 9, 11)
+    assert torch.equal(ol.bilinear_resize(x, 9, 11), x)
+    c = torch.full((2, 8, 8), 1.25)
+    assert torch.equal(ol.bilinear_resize(c, 5, 3), torch.full((2, 5, 3), 1.25))
+
+
+def test_llava_onevision_merge_special_cases():
+    """A single tile is the tile plus one newline; a 1x1 grid of a square image is the tile, then the tile again with a
+    newline behind each of its rows; the newline count equals the number of grid rows kept."""
+    ol, cfg, ocfg = _llava_small()
+    torch.manual_seed(1)
+    nl = torch.randn(8)
+    one = torch.randn(1, 25, 8)
+    out = ol.merge_image(ocfg, one, (70, 70), nl)
+    assert torch.equal(out[:25], one[0]) and torch.equal(out[25], nl) and out.shape[0] == 26
+    two = torch.randn(2, 25, 8)
+    out = ol.merge_image(ocfg, two, (70, 70), nl)
+    assert out.shape[0] == 25 + 5 * 6
+    assert torch.equal(out[:25], two[0])
+    rows = out[25:].view(5, 6, 8)
+    assert torch.equal(rows[:, :5].reshape(25, 8), two[1]) and torch.equal(rows[:, 5], nl.expand(5, 8))
+    # a wide image in a 2x4 grid: rows cropped symmetrically, every kept row ends with the newline
+    tiles = torch.randn(9, 25, 8)
+    out = ol.merge_image(ocfg, tiles, (100, 260), nl)
+    kept = (out.shape[0] - 25) // 21
+    assert (out.shape[0] - 25) % 21 == 0 and 0 < kept <= 10
+    assert torch.equal(out[25:].view(kept, 21, 8)[:, 20], nl.expand(kept, 8))
+    with pytest.raises(ValueError, match="not consistent"):
+        ol.merge_image(ocfg, torch.randn(2, 24, 8), (70, 70), nl)
