@@ -121,13 +121,14 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0) -> dict:
     }
 
 
-OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl")
+OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl", "llava_ov")
 
 
 def other_workload(name: str, steps: int, warmup: int, dev) -> dict:
     """Whole-forward throughput of one of the other configurations (inputs resident in HBM as bf16, synthetic
     weights): configs[2] (SigLIP / Gemma-3, 4 x 896x896), configs[3] (16 ragged images), configs[4] (fp8 weights,
-    two 8-frame videos), and the sibling encoders Qwen2-VL / Qwen3-VL on 8 images of 32 x 32 patches."""
+    two 8-frame videos), the sibling encoders Qwen2-VL / Qwen3-VL on 8 images of 32 x 32 patches, and LLaVA-OneVision on
+    three images cut into 7, 16 and 17 tiles."""
     import numpy as np
     import torch
 
@@ -170,6 +171,20 @@ def other_workload(name: str, steps: int, warmup: int, dev) -> dict:
         cfg = synth.qwen2_vision_config()
         run, L, items = qwen_like(Qwen2VisionTransformer, cfg, synth.qwen2_state_dict(cfg, seed=0), [(1, 32, 32)] * 8, 1176)
         what = "Qwen2-VL-7B ViT (32 blocks, full attention per frame), 8 x 448x448 images = 8192 patches"
+    elif name == "llava_ov":
+        from cornserve_amd.eric.api import Modality
+        from cornserve_amd.eric.models.llava_onevision import LlavaOneVisionEncoder
+
+        cfg = synth.llava_ov_config()
+        model = LlavaOneVisionEncoder(cfg).to(device=dev, dtype=torch.bfloat16).eval()
+        model.load_state_dict(synth.llava_ov_state_dict(cfg, seed=0))
+        sizes = [(768, 1152), (1080, 1920), (1500, 1400)]          # 2x3, 3x5 (cropped) and 4x4 (shrunk) tile grids
+        px, szs = synth.llava_ov_image_inputs(cfg, sizes, seed=0)
+        batch = {"pixel_values": [p.to(device=dev, dtype=torch.bfloat16) for p in px], "image_sizes": szs}
+        tiles = sum(p.shape[0] for p in px)
+        run, L, items = (lambda: model.forward(Modality.IMAGE, "", batch)), tiles * 729, len(sizes)
+        what = (f"LLaVA-OneVision-7B encoder (SigLIP 26 layers + projector + anyres merge), 3 images = {tiles} tiles of "
+                f"384x384 = {L} patches")
     else:
         from cornserve_amd.eric.models.qwen3_vl import Qwen3_VisionTransformer
 
