@@ -362,3 +362,54 @@ def test_load_llava_onevision_from_local_checkpoint(tmp_path):
     assert torch.equal(model.image_newline, sd["image_newline"])
     assert torch.equal(model.multi_modal_projector.linear_2.weight, sd["multi_modal_projector.linear_2.weight"])
     assert model.config.image_grid_pinpoints == cfg.image_grid_pinpoints
+
+
+def test_scheduler_batches_like_the_reference_and_bounds_patches():
+    from cornserve_amd.eric import scheduler as sc
+
+    def item(i, modality=Modality.IMAGE, model="m", grid=(1, 4, 4)):
+        return sc.ProcessedEmbeddingData(id=f"d{i}", modality=modality, model_id=model,
+                                         data={"pixel_values": torch.zeros(grid[0] * grid[1] * grid[2], 8),
+                                               "image_grid_thw": torch.tensor([grid])},
+                                         receiver_sidecar_ranks=[[i]])
+
+    s = sc.Scheduler()
+    assert not s.has_waiting_requests()
+    s.enqueue(sc.EngineEnqueueRequest("r0", [item(0), item(1)]))
+    s.enqueue(sc.EngineEnqueueRequest("r1", [item(2), item(3, Modality.VIDEO), item(4)]))
+    s.enqueue(sc.EngineEnqueueRequest("r2", [item(5, model="other")]))
+    b = s.schedule()                                    # every image at the head, up to the modality change
+    assert (b.modality, b.adapter_name, b.request_ids, b.data_ids) == (Modality.IMAGE, "m", ["r0", "r0", "r1"], ["d0", "d1", "d2"])
+    assert b.chunk_ids == [0, 0, 0] and b.num_chunks == [1, 1, 1] and b.receiver_ranks == [[[0]], [[1]], [[2]]]
+    assert len(b.data["pixel_values"]) == 3 and len(b) == 3
+    wb = b.to_worker_batch()
+    assert type(wb).__name__ == "WorkerBatch" and wb.data is b.data
+    assert s.process_batch_result(b.request_ids, b.data_ids) == ["r0"]
+    b = s.schedule()
+    assert (b.modality, b.data_ids) == (Modality.VIDEO, ["d3"])
+    assert s.process_batch_result(["r1"], ["d3"]) == []
+    b = s.schedule()                                    # the adapter changes behind d4
+    assert b.data_ids == ["d4"] and s.process_batch_result(["r1"], ["d4"]) == ["r1"]
+    b = s.schedule()
+    assert b.adapter_name == "other" and s.process_batch_result(["r2"], ["d5"]) == ["r2"]
+    assert not s.has_waiting_requests()
+    with pytest.raises(ValueError, match="different modalities"):
+        b.add_data("r9", [item(9, Modality.VIDEO)], [0], [1])
+
+    s = sc.Scheduler(max_batch_size=2)
+    s.enqueue(sc.EngineEnqueueRequest("r0", [item(i) for i in range(5)]))
+    assert s.schedule().data_ids == ["d0", "d1"]
+
+    # patch budget: 16 + 16 fit into 40, the third item does not; an item above the budget still runs, alone
+    s = sc.Scheduler(max_batch_patches=40)
+    s.enqueue(sc.EngineEnqueueRequest("r0", [item(0), item(1), item(2), item(3, grid=(2, 8, 8)), item(4)]))
+    b = s.schedule()
+    assert b.data_ids == ["d0", "d1"]
+    s.process_batch_result(b.request_ids, b.data_ids)
+    assert s.schedule().data_ids == ["d2"]               # 16 + 128 > 40
+    s.process_batch_result(["r0"], ["d2"])
+    assert s.schedule().data_ids == ["d3"]
+    with pytest.raises(ValueError):
+        sc.Scheduler(max_batch_patches=0)
+    tiles = sc.ProcessedEmbeddingData("t", Modality.IMAGE, "m", {"pixel_values": torch.zeros(3, 3, 28, 42)})
+    assert sc.patch_count(tiles) == 3 * 2 * 3 and sc.patch_count(item(0, grid=(2, 4, 6))) == 48
