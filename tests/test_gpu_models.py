@@ -187,6 +187,38 @@ def test_worker_hand_off_of_real_embeddings(dev, tmp_path):
         assert torch.equal(saved.to(dev), direct[i])
 
 
+def test_scheduler_worker_loop_with_patch_budget(dev, tmp_path):
+    """Requests queued in the scheduler, batched under a patch budget, run by the worker and handed to the mock
+    sidecar: every item's embedding equals the one from a single direct call (an item does not depend on its batch)."""
+    from cornserve_amd.eric import scheduler as sc
+    from cornserve_amd.eric.worker import MockSidecar, Worker
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=12)
+    grids = [(1, 8, 12), (1, 16, 16), (2, 4, 4), (1, 4, 6), (1, 12, 8)]
+    px, grid = synth.qwen_inputs(grids, seed=12)
+    direct = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    mapping = {f"d{i}-0": tmp_path / f"{i}.pt" for i in range(len(grids))}
+    worker = Worker(model, MockSidecar(mapping))
+    s = sc.Scheduler(max_batch_patches=300)
+    items = [sc.ProcessedEmbeddingData(id=f"d{i}", modality=Modality.IMAGE, model_id="",
+                                       data={"pixel_values": px[i], "image_grid_thw": grid[i]},
+                                       receiver_sidecar_ranks=[[0]]) for i in range(len(grids))]
+    s.enqueue(sc.EngineEnqueueRequest("r0", items[:3]))
+    s.enqueue(sc.EngineEnqueueRequest("r1", items[3:]))
+    batches, finished = [], []
+    while s.has_waiting_requests():
+        b = s.schedule()
+        batches.append(list(b.data_ids))
+        out = worker.execute_model(b.to_worker_batch())
+        for data_id, emb in zip(b.data_ids, out):
+            assert torch.equal(emb, direct[int(data_id[1:])])
+        finished += s.process_batch_result(b.request_ids, b.data_ids)
+    # 96 + 256 > 300; 256 + 32 fit, + 24 does not; 24 + 96 fit
+    assert batches == [["d0"], ["d1", "d2"], ["d3", "d4"]] and finished == ["r0", "r1"]
+    for i in range(len(grids)):
+        assert torch.equal(torch.load(mapping[f"d{i}-0"], weights_only=True).to(dev), direct[i])
+
+
 def test_load_model_from_checkpoint_directory_runs(dev, tmp_path):
     """A checkpoint directory (config.json + safetensors shards with `visual.` names among other weights) loaded by
     the loader gives the same embeddings as the model built from the same tensors directly."""
