@@ -160,7 +160,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   constexpr int NLD = A_LD + W_LD;                      // direct loads per wave and K tile
   constexpr int NFR = MT + NT;                          // fragment reads per wave and k-step
   constexpr int NMFMA = MT * NT;                        // MFMAs per wave and k-step
-  static_assert(2 * NFR <= NMFMA, "one slot after an MFMA per LDS read");
+  // Fragment reads of the second k-step go after every other MFMA where there are enough of them, else after each.
+  constexpr int READ_STRIDE = (2 * NFR <= NMFMA) ? 2 : 1;
+  static_assert(READ_STRIDE * NFR <= NMFMA, "one slot after an MFMA per LDS read");
 
   // ---- tile coordinates of virtual block vb in [0, tiles): XCD-aware remap (workgroup i runs on XCD i%8,
   //      and the persistent stride gridDim.x is a multiple of 8, so a workgroup's tiles stay on its XCD),
@@ -413,8 +415,8 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       // which goes to LDS space that the barrier has just freed
       mfmas(ic<1>{}, std::false_type{}, [&](auto n) {
         constexpr int N = decltype(n)::value;
-        if constexpr (TAIL != 1 && N < 2 * NFR && N % 2 == 0)
-          read_frag(a_base_of(1, ring), w_base_of(1, ring), 0, 0, ic<N / 2>{});
+        if constexpr (TAIL != 1 && N < READ_STRIDE * NFR && N % READ_STRIDE == 0)
+          read_frag(a_base_of(1, ring), w_base_of(1, ring), 0, 0, ic<N / READ_STRIDE>{});
         if constexpr (N < EB * PB && N % EB == EB - 1) {
           auto ld = [&]() { direct_load(k_b, a_base_of(AHEAD_B, ring), w_base_of(AHEAD_B, ring), ic<PB_FIRST + N / EB>{}); };
           if constexpr (CUR_B) ld();
@@ -753,13 +755,19 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160" or "256"
   // (the erf GELU epilogue with fp8 scales does not fit the architectural registers of the 256x160 form)
   const bool fits160 = !(a.w_fp8 && a.epilogue == CS_EPI_GELU_ERF);
-  // Row sums of squares come in CS_SUMSQ_PARTS parts, one per column tile of the 256x160 form.
+  // Few rows: 160-column tiles of 256 rows would leave half of the compute units or more without a tile (N = 1280
+  // gives 8 column tiles, so 1024 rows are 32 workgroups).  The 128x160 form has the same waves-by-columns layout,
+  // so every output element and every row-sum part is computed by the same sequence of operations: results do not
+  // depend on which of the two a batch size selects.
+  const bool few_rows = !a.w_fp8 && (int64_t)((a.M + 255) / 256) * ((a.N + 159) / 160) <= 128;
+  auto narrow = [&]() { return few_rows ? dispatch_epi<128, 160, 4, 1>(a, stream) : dispatch_epi<256, 160, 4, 1>(a, stream); };
+  // Row sums of squares come in CS_SUMSQ_PARTS parts, one per column tile of the 160-column forms.
   if (a.c_row_sumsq) {
     if (a.N > CS_SUMSQ_PARTS * 160 || a.w_fp8) return CS_ERR_UNSUPPORTED;
-    return dispatch_epi<256, 160, 4, 1>(a, stream);
+    return narrow();
   }
-  if (a.a_row_sum) return dispatch_epi<256, 160, 4, 1>(a, stream);   // see dispatch_epi_w
-  if (fits160 && (force ? force[0] == '1' : c160 < c256)) return dispatch_epi<256, 160, 4, 1>(a, stream);
+  if (a.a_row_sum) return narrow();   // see dispatch_epi_w
+  if (fits160 && (force ? force[0] == '1' : c160 < c256)) return narrow();
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller
   // tiles (256x128 or 128x192: more workgroups, each shorter).  The two launches write disjoint column
