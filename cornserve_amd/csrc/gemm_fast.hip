@@ -18,7 +18,7 @@
 //   * 256x256 tile: five 32 KB units = A(kt), W(kt), A(kt+1), W(kt+1) and one in flight.  A(kt+2) is
 //     requested in the first half of iteration kt, W(kt+2) in the second half, into the unit that the
 //     barrier has just freed.
-//   * narrower tiles (256x160, 256x128, 128x192): three whole stages.  The second half of K tile kt+2 is
+//   * narrower tiles (256x160, 128x160, 256x128, 128x192): three whole stages.  The second half of K tile kt+2 is
 //     requested in the first half of iteration kt, the first half of K tile kt+3 in the second half.
 // The sequence of K tiles runs on across output tiles: the next output tile's first K tiles are requested
 // in the last iterations of the current one and travel while the epilogue runs.  Waits use the in-order
