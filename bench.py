@@ -18,6 +18,7 @@ with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
                         the instrumented pass applied to the timed step
   host_inputs           the same step with the batch handed over as fp32 host tensors (PCIe-inclusive)
   host_inputs_uint8_frames  the same step from resized uint8 frames on the host (PCIe-inclusive; GPU patch layout)
+  single_image          latency of a batch of one image of the same size (inputs resident in HBM)
   (--workload cfg3 | cfg4 | cfg5 | qwen2_vl | qwen3_vl prints a shorter line -- throughput only -- for the other
   configurations; the default, cfg2, is the headline benchmark)
   cpu_baseline          the CPU oracle (a port of the reference's algorithm, plain PyTorch) timed on this
@@ -288,6 +289,17 @@ def main() -> None:
             model.forward(Modality.IMAGE, "", frame_batch)
         torch.cuda.synchronize()
         frames_ms = (time.perf_counter() - t0) / 5 * 1e3
+        # latency of a batch of one: a single image of the same size, resident in HBM (the serving case when the
+        # queue is short; the N = 1280 GEMMs then run on a quarter of the compute units)
+        one_px, one_grid = pixel_values[: GRID[1] * GRID[2]], grid_np[:1]
+        for _ in range(2):
+            model.forward_device(one_px, one_grid)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            model.forward_device(one_px, one_grid)
+        torch.cuda.synchronize()
+        one_ms = (time.perf_counter() - t0) / 10 * 1e3
     stage_ms = {k: sum(v) / 3 for k, v in full.durations_ms().items()}
     mfma_keys = [k for k in stage_ms if k.startswith("gemm_") or k.startswith("attn_") or k == "patch_embed"]
     # The instrumented pass records an event between stages, which costs a little device time per mark: its
@@ -340,6 +352,8 @@ def main() -> None:
         "note": "same shapes handed over as pageable uint8 host frames [1,448,448,3] (PCIe copy, then rescale + "
                 "normalise + patch layout on the GPU inside the call)",
     }
+    result["single_image"] = {"ms": one_ms, "patches": GRID[1] * GRID[2],
+                              "note": "one 448x448 image alone (1024 patches), inputs resident in HBM"}
     if args.calibrate_copy:
         src = torch.zeros(256 * 1024 * 1024, dtype=torch.int32, device=dev)  # 1 GiB read + 1 GiB written per copy
         for _ in range(3):
