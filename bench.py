@@ -92,9 +92,10 @@ class EventMarks:
         return out
 
 
-def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0) -> dict:
+def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: list | None = None) -> dict:
     """Time the CPU oracle (bf16, all host threads) on `n_sample_images` of the batch's 8 images, repeating
-    the pass until about `min_seconds` of CPU work have been measured."""
+    the pass until about `min_seconds` of CPU work have been measured.  `gpu_out`: the embeddings of the timed
+    GPU step for the same (leading) images; the oracle's output then also serves as the checker at full size."""
     import torch
 
     from cornserve_amd import synth
@@ -115,11 +116,32 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0) -> dict:
         dt += time.perf_counter() - t0
         iters += 1
         assert len(out) == n_sample_images
-    return {
+    res = {
         "value": patches * iters / dt, "unit": "patches/s", "cores": threads, "kind": "port",
         "sample": f"{n_sample_images} of the 8 images ({patches} patches) through the full 32-block encoder, "
                   f"bf16 step-wise CPU oracle, {iters} iteration(s), {dt:.1f} s in total",
     }
+    if gpu_out is not None:
+        # Full-size check (untimed): the GPU embeddings and this bf16 oracle pass, each against the oracle in fp32 on
+        # the same bf16-rounded weights and inputs.  At 32 blocks of random-init weights the bf16 oracle itself sits
+        # at the edge of the max-error bar, so its distance is printed beside the GPU's.
+        def dist(a, b):
+            return {"cosine": torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0).item(),
+                    "max_rel_err": ((a - b).abs().max() / b.abs().max()).item()}
+
+        sd32 = {k: v.float() for k, v in sd16.items()}
+        px32 = [p.to(torch.bfloat16).float() for p in px]
+        ref32 = torch.cat(oq.forward(sd32, ocfg, px32, grid, dtype=torch.float32))
+        ref16 = torch.cat([o.float() for o in out])
+        got = torch.cat([o.float() for o in gpu_out[:n_sample_images]])
+        res["gpu_vs_oracle"] = {
+            "gpu_vs_fp32_oracle": dist(got, ref32),
+            "bf16_oracle_vs_fp32_oracle": dist(ref16, ref32),
+            "gpu_vs_bf16_oracle": dist(got, ref16),
+            "bar": "cosine >= 0.999, max |err| / max |ref| <= 2e-2 (tested at 2-4 blocks in tests/; here 32 blocks)",
+            "what": f"embeddings of the timed GPU step, {n_sample_images} images, 32 blocks",
+        }
+    return res
 
 
 OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl", "llava_ov")
@@ -259,6 +281,7 @@ def main() -> None:
         dt = time.perf_counter() - t0
         assert len(out) == N_IMAGES and out[0].shape == (256, 3584)
         assert torch.isfinite(out[0].float()).all()
+        timed_out = [o.float().cpu() for o in out]
         gu = marks.durations_ms()["gemm_gate_up"]
         gu_ms = sum(gu) / len(gu)
 
@@ -363,7 +386,7 @@ def main() -> None:
     if not args.no_cpu_baseline:
         del model
         torch.cuda.empty_cache()
-        result["cpu_baseline"] = cpu_baseline(sd, args.cpu_sample_images)
+        result["cpu_baseline"] = cpu_baseline(sd, args.cpu_sample_images, gpu_out=timed_out)
     print(json.dumps(result))
 
 
