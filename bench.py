@@ -22,7 +22,8 @@ with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
   (--workload cfg3 | cfg4 | cfg5 | qwen2_vl | qwen3_vl prints a shorter line -- throughput only -- for the other
   configurations; the default, cfg2, is the headline benchmark)
   cpu_baseline          the CPU oracle (a port of the reference's algorithm, plain PyTorch) timed on this
-                        host's cores on a bounded sample of the same workload
+                        host's cores on a bounded sample of the same workload; its `gpu_vs_oracle` entry is the
+                        full-size check of the timed step's embeddings (untimed extra fp32 oracle pass)
 """
 
 from __future__ import annotations
