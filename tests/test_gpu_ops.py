@@ -656,3 +656,60 @@ def test_patchify_nchw_drops_the_partial_patches(ops, dev):
     ref = F.unfold(px.float()[:, :, :378, :378], kernel_size=14, stride=14).transpose(1, 2).reshape(3 * 729, 588)
     assert got.shape == (3 * 729, 592)
     assert torch.equal(got[:, :588].float(), ref) and not got[:, 588:].any()
+
+
+def test_gemm_random_shapes_epilogues_and_folds(ops, dev):
+    """A seeded sweep over row counts either side of every tile height (1 .. 5000), widths, depths, epilogues and the
+    folded-norm forms, against fp32 torch arithmetic with the reference's rounding points."""
+    rng = np.random.default_rng(11)
+    rbf = lambda x: x.bfloat16().float()
+    ran = folded = 0
+    for it in range(90):
+        M = int(rng.choice([1, 7, 64, 100, 127, 128, 129, 255, 256, 257, 300, 511, 513, 1000, 1024, 1500, 2048, 3000, 4096, 4100, 5000]))
+        N = int(rng.choice([8, 64, 160, 168, 320, 520, 640, 1152, 1280, 1288, 2304, 3456, 3840]))
+        K = int(rng.choice([64, 128, 192, 200, 256, 320, 448, 1152, 1176, 1280]))
+        epi = int(rng.choice([ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_SWIGLU, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU]))
+        fold = int(rng.choice([0, 0, 1, 2, 3]))
+        if epi == ops.EPI_SWIGLU and (N // 2) % 8:
+            continue
+        a, w, b = rnd((M, K), 1.0, it, dev), rnd((N, K), 0.05, it + 1000, dev), rnd((N,), 0.05, it + 2000, dev)
+        res = rnd((M, N), 1.0, it + 3000, dev) if epi == ops.EPI_RESIDUAL else None
+        af, wf = a.float().cpu(), w.float().cpu()
+        acc = af @ wf.t()
+        eps, kw = 1e-6, {}
+        fast = K % 64 == 0 and K >= 192
+        if fold == 1 and epi in (ops.EPI_BIAS, ops.EPI_SWIGLU) and fast:
+            ss = torch.zeros((M, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev)
+            ops.row_sumsq(a, ss)
+            kw = dict(a_row_sumsq=ss, norm_eps=eps)
+            acc = acc * torch.rsqrt((af * af).sum(1, keepdim=True) / K + eps)
+        elif fold == 2 and epi in (ops.EPI_RESIDUAL, ops.EPI_BIAS) and fast and N <= 1280:
+            kw = dict(c_row_sumsq=torch.zeros((M, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev))
+        elif fold == 3 and epi in (ops.EPI_BIAS, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU) and fast:
+            ss = torch.zeros((M, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev)
+            sm = torch.zeros_like(ss)
+            ops.row_stats(a, ss, sm)
+            kw = dict(a_row_sumsq=ss, a_row_sum=sm, w_col_sum=wf.sum(1).to(dev), norm_eps=eps)
+            mean = af.mean(1, keepdim=True)
+            var = ((af * af).mean(1, keepdim=True) - mean * mean).clamp_min(0)
+            acc = torch.rsqrt(var + eps) * (acc - mean * wf.sum(1)[None, :])
+        folded += bool(kw)
+        got = ops.gemm(a, w, b, epilogue=epi, residual=res, **kw).float().cpu()
+        v = acc + b.float().cpu()
+        if epi == ops.EPI_RESIDUAL:
+            ref = rbf(v) + res.float().cpu()
+        elif epi == ops.EPI_SWIGLU:
+            ref = F.silu(rbf(v[:, 0::2])) * rbf(v[:, 1::2])
+        elif epi == ops.EPI_GELU_ERF:
+            ref = F.gelu(rbf(v))
+        elif epi == ops.EPI_GELU_TANH:
+            ref = F.gelu(rbf(v), approximate="tanh")
+        elif epi == ops.EPI_QUICK_GELU:
+            ref = rbf(v) * torch.sigmoid(1.702 * rbf(v))
+        else:
+            ref = v
+        close(got, ref, 2**-6, f"gemm {M}x{N}x{K} epilogue {epi} fold {fold}")
+        if "c_row_sumsq" in kw:
+            close(kw["c_row_sumsq"].sum(1), (got * got).sum(1), 1e-3, f"row sums of squares {M}x{N}x{K}")
+        ran += 1
+    assert ran >= 70 and folded >= 10
