@@ -713,3 +713,32 @@ def test_gemm_random_shapes_epilogues_and_folds(ops, dev):
             close(kw["c_row_sumsq"].sum(1), (got * got).sum(1), 1e-3, f"row sums of squares {M}x{N}x{K}")
         ran += 1
     assert ran >= 70 and folded >= 10
+
+
+def test_attention_random_segments(ops, dev):
+    """A seeded sweep over head dims, segment-length mixes (1 .. 3000 rows, lengths either side of the 64-key tile and
+    the 64/128-row query blocks) and rotary on/off, against fp32 softmax attention."""
+    rng = np.random.default_rng(17)
+    for it in range(24):
+        d = int(rng.choice([64, 72, 80, 96]))
+        nh = int(rng.choice([2, 4, 16]))
+        kind = it % 4
+        if kind == 0:      # many short segments (the window kernel)
+            lens = rng.integers(1, 65, size=int(rng.integers(3, 40))).tolist()
+        elif kind == 1:    # a few long ones (the full kernels)
+            lens = rng.integers(100, 3000, size=int(rng.integers(1, 4))).tolist()
+        elif kind == 2:    # lengths at the tile edges
+            lens = [int(x) for x in rng.choice([63, 64, 65, 127, 128, 129, 191, 192, 193, 256, 729], size=5)]
+        else:              # short and long mixed
+            lens = rng.integers(1, 700, size=int(rng.integers(2, 10))).tolist()
+        cu = [0] + np.cumsum(lens).tolist()
+        L, H = cu[-1], nh * d
+        qkv = rnd((L, 3 * H), 1.0, 100 + it, dev)
+        rotary = bool(rng.integers(0, 2)) and d % 16 == 0
+        ang = cs = None
+        if rotary:
+            ang = torch.rand(L, d // 2, generator=torch.Generator().manual_seed(it)) * 50
+            cs = torch.cat([ang.cos(), ang.sin()], -1).contiguous().to(dev)
+        plan = ops.attn_plan(np.array(cu, np.int32), dev)
+        got = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], plan, nh, d, d**-0.5, cs)
+        close(got, attn_ref(qkv, cu, nh, d, ang), 2**-6, f"attention d={d} heads={nh} lens={lens[:8]} rotary={rotary}")
