@@ -722,7 +722,11 @@ int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
 
 template <int BM, int BN, int WAVES_M, int WAVES_N>
 int dispatch_epi(const CsGemmArgs& a, hipStream_t s) {
-  if (a.w_fp8) return dispatch_epi_w<BM, BN, WAVES_M, WAVES_N, true>(a, s);
+  if (a.w_fp8) {
+    // (the few-rows form is only dispatched for bf16 weights: its fp8 kernels are not built)
+    if constexpr (BM == 128 && BN == 160) return CS_ERR_UNSUPPORTED;
+    else return dispatch_epi_w<BM, BN, WAVES_M, WAVES_N, true>(a, s);
+  }
   return dispatch_epi_w<BM, BN, WAVES_M, WAVES_N, false>(a, s);
 }
 
