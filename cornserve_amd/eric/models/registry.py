@@ -46,62 +46,29 @@ class RegistryEntry:
             raise ValueError(f"Registry entry for {self.class_name} must have `adapter_attr` set if `adapter_prefixes` is specified.")
 
 
+def _entry(module: str, class_name: str, resolution: ViTResolutionType, required: list[str],
+           modalities: tuple[Modality, ...], *, strip: bool = True, ignored: tuple[str, ...] = (),
+           adapter_attr: str | None = None, adapter_prefixes: tuple[str, ...] = ()) -> RegistryEntry:
+    weight = WeightInfo(required_prefixes=list(required), ignored_prefixes=list(ignored),
+                        adapter_prefixes=list(adapter_prefixes), strip_prefixes=strip)
+    return RegistryEntry(module=module, class_name=class_name, adapter_attr=adapter_attr, vit_resolution_type=resolution,
+                         weight=weight, modality={m: ModalityEntry() for m in modalities})
+
+
+_IMAGE_VIDEO = (Modality.IMAGE, Modality.VIDEO)
+_SIGLIP_POST_NORM = ("vision_tower.vision_model.post_layernorm",)
+
+# model_type of the checkpoint's config.json -> how to build and fill the encoder (the reference's entries for the
+# encoders built here, registry.py:59-233: same modules, class names, prefixes and modalities).
 MODEL_REGISTRY: dict[str, RegistryEntry] = {
-    "qwen2_vl": RegistryEntry(
-        module="qwen2_vl",
-        class_name="Qwen2VisionTransformer",
-        adapter_attr=None,
-        vit_resolution_type=ViTResolutionType.DYNAMIC,
-        weight=WeightInfo(required_prefixes=["visual."], strip_prefixes=True),
-        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
-    ),
-    "qwen2_5_vl": RegistryEntry(
-        module="qwen2_5_vl",
-        class_name="Qwen2_5_VisionTransformer",
-        adapter_attr=None,
-        vit_resolution_type=ViTResolutionType.DYNAMIC,
-        weight=WeightInfo(required_prefixes=["visual."], strip_prefixes=True),
-        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
-    ),
-    "qwen3_vl": RegistryEntry(
-        module="qwen3_vl",
-        class_name="Qwen3_VisionTransformer",
-        adapter_attr=None,
-        vit_resolution_type=ViTResolutionType.DYNAMIC,
-        weight=WeightInfo(required_prefixes=["model.visual."], strip_prefixes=True),
-        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
-    ),
-    "qwen3_vl_moe": RegistryEntry(
-        module="qwen3_vl",
-        class_name="Qwen3_VisionTransformer",
-        adapter_attr=None,
-        vit_resolution_type=ViTResolutionType.DYNAMIC,
-        weight=WeightInfo(required_prefixes=["model.visual."], strip_prefixes=True),
-        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
-    ),
-    "llava_onevision": RegistryEntry(
-        module="llava_onevision",
-        class_name="LlavaOneVisionEncoder",
-        adapter_attr=None,
-        vit_resolution_type=ViTResolutionType.FIXED,
-        weight=WeightInfo(
-            required_prefixes=["vision_tower.", "multi_modal_projector.", "image_newline"],
-            ignored_prefixes=["vision_tower.vision_model.post_layernorm"],
-            strip_prefixes=False,
-        ),
-        modality={Modality.IMAGE: ModalityEntry(), Modality.VIDEO: ModalityEntry()},
-    ),
-    "gemma3": RegistryEntry(
-        module="gemma3",
-        class_name="Gemma3VisionEncoder",
-        adapter_attr="multi_modal_projector",
-        vit_resolution_type=ViTResolutionType.FIXED,
-        weight=WeightInfo(
-            required_prefixes=["vision_tower.", "multi_modal_projector."],
-            ignored_prefixes=["vision_tower.vision_model.post_layernorm"],
-            adapter_prefixes=["multi_modal_projector."],
-            strip_prefixes=False,
-        ),
-        modality={Modality.IMAGE: ModalityEntry()},
-    ),
+    "qwen2_vl": _entry("qwen2_vl", "Qwen2VisionTransformer", ViTResolutionType.DYNAMIC, ["visual."], _IMAGE_VIDEO),
+    "qwen2_5_vl": _entry("qwen2_5_vl", "Qwen2_5_VisionTransformer", ViTResolutionType.DYNAMIC, ["visual."], _IMAGE_VIDEO),
+    "qwen3_vl": _entry("qwen3_vl", "Qwen3_VisionTransformer", ViTResolutionType.DYNAMIC, ["model.visual."], _IMAGE_VIDEO),
+    "qwen3_vl_moe": _entry("qwen3_vl", "Qwen3_VisionTransformer", ViTResolutionType.DYNAMIC, ["model.visual."], _IMAGE_VIDEO),
+    "llava_onevision": _entry("llava_onevision", "LlavaOneVisionEncoder", ViTResolutionType.FIXED,
+                              ["vision_tower.", "multi_modal_projector.", "image_newline"], _IMAGE_VIDEO,
+                              strip=False, ignored=_SIGLIP_POST_NORM),
+    "gemma3": _entry("gemma3", "Gemma3VisionEncoder", ViTResolutionType.FIXED, ["vision_tower.", "multi_modal_projector."],
+                     (Modality.IMAGE,), strip=False, ignored=_SIGLIP_POST_NORM, adapter_attr="multi_modal_projector",
+                     adapter_prefixes=("multi_modal_projector.",)),
 }
