@@ -145,7 +145,77 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: l
     return res
 
 
-OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl", "llava_ov")
+def hbm_kernels(dev, rows_list=(8192, 131072), reps: int = 20) -> dict:
+    """Achieved bytes/s of the HBM-bound kernels (norms, rotary, gathers, patch layout) at config 2's row count, where
+    the operands of a looped launch stay in the 256 MB last-level cache, and at 16x that, where they do not:
+    algorithmic bytes per launch / average duration between two HIP events on the launch stream."""
+    import numpy as np
+    import torch
+
+    from cornserve_amd import ops
+
+    H, heads, d = 1280, 16, 80
+    out = {}
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e-3
+
+    for L in rows_list:
+        g = torch.Generator().manual_seed(0)
+        x = torch.randn((L, H), generator=g).to(device=dev, dtype=torch.bfloat16)
+        y = torch.empty_like(x)
+        w = torch.ones(H, dtype=torch.bfloat16, device=dev)
+        b = torch.zeros(H, dtype=torch.bfloat16, device=dev)
+        res = {}
+
+        def put(name, nbytes, fn):
+            t = timed(fn)
+            res[name] = {"us": round(t * 1e6, 2), "GB_per_s": round(nbytes / t / 1e9, 1), "bytes": int(nbytes)}
+
+        put("rmsnorm", 2 * L * H * 2, lambda: ops.rmsnorm(x, w, 1e-6, out=y))
+        put("layernorm", 2 * L * H * 2, lambda: ops.layernorm(x, w, b, 1e-6, out=y))
+        ss = torch.zeros((L, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev)
+        put("row_sumsq", L * H * 2 + L * 32, lambda: ops.row_sumsq(x, ss))
+        qkv = torch.randn((L, 3 * H), generator=g).to(device=dev, dtype=torch.bfloat16)
+        ang = torch.rand((L, d // 2), generator=g) * 6
+        cs = torch.cat([ang.cos(), ang.sin()], -1).contiguous().to(dev)
+        put("rope_qk (q and k of a packed qkv buffer, in place)", 2 * L * 2 * H * 2 + L * d * 4,
+            lambda: ops.rope_qk_(qkv, cs, heads, d))
+        perm = torch.randperm(L, generator=g).to(device=dev, dtype=torch.int32)
+        put("row_gather (random permutation of rows)", 2 * L * H * 2 + L * 4, lambda: ops.row_gather(x, perm))
+        T = 3584
+        src = torch.randn((L // 4, T), generator=g).to(device=dev, dtype=torch.bfloat16)
+        R = L // 4
+        taps = torch.randint(0, R, (R, 4), generator=g, dtype=torch.int32)
+        taps_copy = taps[:, :1].repeat(1, 4).contiguous().to(dev)
+        frac0 = torch.zeros((R, 2), dtype=torch.float32, device=dev)
+        frac = torch.rand((R, 2), generator=g).to(dev)
+        dst = torch.empty_like(src)
+        put("rows_bilinear (copy records)", 2 * R * T * 2 + R * 24, lambda: ops.rows_bilinear(src, taps_copy, frac0, out=dst))
+        taps_d = taps.to(dev)
+        put("rows_bilinear (four-tap records)", 5 * R * T * 2 + R * 24, lambda: ops.rows_bilinear(src, taps_d, frac, out=dst))
+        side = int(np.sqrt(L)) // 2 * 2          # patches per side, even: the frame's sides are multiples of 28
+        frames = torch.randint(0, 256, (1, side * 14, side * 14, 3), dtype=torch.uint8).to(dev)
+        table = torch.linspace(-2, 2, 768).reshape(3, 256).contiguous().to(dev)
+        n_patch = (frames.shape[1] // 14) * (frames.shape[2] // 14)
+        put("qwen_patchify_u8 (one frame -> bf16 patch rows)", frames.numel() + n_patch * 1176 * 2,
+            lambda: ops.qwen_patchify_u8(frames, table, 14, 2, 2))
+        out[f"rows_{L}"] = res
+    return {"metric": "achieved GB/s of the HBM-bound kernels on 1 MI355X", "unit": "GB/s", "n_gpus": 1, "peak_GB_per_s": 8000,
+            "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "hidden 1280, 16 heads of 80 (config 2's shapes); merged rows of 3584 for the row mixes"},
+            "kernels": out}
+
+
+OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl", "llava_ov", "hbm_kernels")
 
 
 def other_workload(name: str, steps: int, warmup: int, dev) -> dict:
@@ -256,6 +326,9 @@ def main() -> None:
 
     lib.load()
     dev = torch.device("cuda:0")
+    if args.workload == "hbm_kernels":
+        print(json.dumps(hbm_kernels(dev)))
+        return
     if args.workload != "cfg2":
         print(json.dumps(other_workload(args.workload, args.steps, args.warmup, dev)))
         return

@@ -41,50 +41,61 @@ __global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict_
 // the table with it).  Rows are ordered (t, block row, block col, row in block, col in block) with blocks of
 // merge x merge patches, columns (channel, temporal, y, x); temporal slot tt of row group t shows frame
 // min(t*temporal + tt, T-1): an image is one frame repeated, a video's last frame is repeated to fill a group.
-// One thread writes two neighbouring x of one output row; the table sits in LDS.
-template <typename OUT>
+// One workgroup writes one output row (its place in the frame is worked out once, uniformly); a thread writes two
+// neighbouring x at a time.  P and TPS are the patch size and the temporal patch size as constants (the column
+// decomposition is then divisions by constants), or 0 for any value.  The table sits in LDS.
+template <typename OUT, int P, int TPS>
 __global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __restrict__ frames, int T, int H, int W,
-                                                               int p, int m, int tps, const float* __restrict__ table,
-                                                               OUT* __restrict__ out, int64_t ldo, int64_t total_pairs) {
+                                                               int p_any, int m, int tps_any, const float* __restrict__ table,
+                                                               OUT* __restrict__ out, int64_t ldo) {
   __shared__ float lut[3 * 256];
   for (int i = threadIdx.x; i < 3 * 256; i += 256) lut[i] = table[i];
   __syncthreads();
-  int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= total_pairs) return;
+  const int p = P ? P : p_any, tps = TPS ? TPS : tps_any;
   const int hp = p >> 1;
-  const int xp = (int)(i % hp);
-  i /= hp;
-  const int py = (int)(i % p);
-  i /= p;
-  const int tt = (int)(i % tps);
-  i /= tps;
-  const int c = (int)(i % 3);
-  int64_t row = i / 3;
-  const int col = ((c * tps + tt) * p + py) * p + 2 * xp;
   const int bw = W / (p * m), bh = H / (p * m);
-  int64_t r = row;
-  const int mx = (int)(r % m);
+  int r = blockIdx.x;             // output row -> (t, block row, block column, row in block, column in block)
+  const int mx = r % m;
   r /= m;
-  const int my = (int)(r % m);
+  const int my = r % m;
   r /= m;
-  const int bx = (int)(r % bw);
+  const int bx = r % bw;
   r /= bw;
-  const int by = (int)(r % bh);
-  const int t = (int)(r / bh);
-  const int f = min(t * tps + tt, T - 1);
-  const int y = (by * m + my) * p + py, x = (bx * m + mx) * p + 2 * xp;
-  const uint8_t* src = frames + (((int64_t)f * H + y) * W + x) * 3 + c;
-  const float v0 = lut[c * 256 + src[0]], v1 = lut[c * 256 + src[3]];
-  OUT* dst = out + row * ldo + col;
-  if constexpr (sizeof(OUT) == 2) {
-    bf16x2_t o;
-    o[0] = f2bf(v0);
-    o[1] = f2bf(v1);
-    *(bf16x2_t*)dst = o;
-  } else {
-    dst[0] = v0;
-    dst[1] = v1;
+  const int by = r % bh;
+  const int t = r / bh;
+  const int y0 = (by * m + my) * p, x0 = (bx * m + mx) * p;
+  OUT* const dst_row = out + (int64_t)blockIdx.x * ldo;
+  const int pairs = 3 * tps * p * hp;
+  for (int q = threadIdx.x; q < pairs; q += 256) {   // q -> (channel, temporal slot, y, x pair), x fastest
+    const int xp = q % hp, q1 = q / hp;
+    const int py = q1 % p, q2 = q1 / p;
+    const int tt = q2 % tps, c = q2 / tps;
+    const int f = min(t * tps + tt, T - 1);
+    const uint8_t* src = frames + (((int64_t)f * H + (y0 + py)) * W + (x0 + 2 * xp)) * 3 + c;
+    const float v0 = lut[c * 256 + src[0]], v1 = lut[c * 256 + src[3]];
+    OUT* dst = dst_row + 2 * q;   // column ((c*tps + tt)*p + py)*p + 2*xp == 2*q
+    if constexpr (sizeof(OUT) == 2) {
+      bf16x2_t o;
+      o[0] = f2bf(v0);
+      o[1] = f2bf(v1);
+      *(bf16x2_t*)dst = o;
+    } else {
+      dst[0] = v0;
+      dst[1] = v1;
+    }
   }
+}
+
+template <typename OUT>
+void launch_qwen_patchify_u8(dim3 grid, hipStream_t stream, const uint8_t* frames, int T, int H, int W, int p, int m,
+                             int tps, const float* table, OUT* out, int64_t ldo) {
+  const dim3 block(256);
+  if (p == 14 && tps == 2)
+    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 14, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo);
+  else if (p == 16 && tps == 2)
+    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 16, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo);
+  else
+    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 0, 0>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo);
 }
 
 }  // namespace
@@ -100,15 +111,12 @@ extern "C" int cs_qwen_patchify_u8(const void* frames, int32_t T, int32_t H, int
   if (ldo < cols || ldo % 2 || ((uintptr_t)out & (out_fp32 ? 7 : 3)) || ((uintptr_t)table & 3)) return CS_ERR_INVALID_ARG;
   if (T == 0) return CS_OK;
   const int64_t rows = (int64_t)((T + temporal - 1) / temporal) * (H / patch) * (W / patch);
-  const int64_t pairs = rows * cols / 2;
-  if ((pairs + 255) / 256 > 0x7fffffff) return CS_ERR_TOO_LARGE;
-  const dim3 grid((unsigned)((pairs + 255) / 256)), block(256);
+  if (rows > 0x7fffffff) return CS_ERR_TOO_LARGE;
+  const dim3 grid((unsigned)rows);
   if (out_fp32)
-    hipLaunchKernelGGL(qwen_patchify_u8_kernel<float>, grid, block, 0, stream, (const uint8_t*)frames, T, H, W, patch,
-                       merge, temporal, table, (float*)out, ldo, pairs);
+    launch_qwen_patchify_u8<float>(grid, stream, (const uint8_t*)frames, T, H, W, patch, merge, temporal, table, (float*)out, ldo);
   else
-    hipLaunchKernelGGL(qwen_patchify_u8_kernel<bf16_t>, grid, block, 0, stream, (const uint8_t*)frames, T, H, W, patch,
-                       merge, temporal, table, (bf16_t*)out, ldo, pairs);
+    launch_qwen_patchify_u8<bf16_t>(grid, stream, (const uint8_t*)frames, T, H, W, patch, merge, temporal, table, (bf16_t*)out, ldo);
   return cs_launch_status();
 }
 
