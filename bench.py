@@ -19,8 +19,9 @@ with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
   host_inputs           the same step with the batch handed over as fp32 host tensors (PCIe-inclusive)
   host_inputs_uint8_frames  the same step from resized uint8 frames on the host (PCIe-inclusive; GPU patch layout)
   single_image          latency of a batch of one image of the same size (inputs resident in HBM)
-  (--workload cfg3 | cfg4 | cfg5 | qwen2_vl | qwen3_vl prints a shorter line -- throughput only -- for the other
-  configurations; the default, cfg2, is the headline benchmark)
+  (--workload cfg3 | cfg4 | cfg5 | qwen2_vl | qwen3_vl | llava_ov prints a shorter line -- throughput only -- for the
+  other configurations, --workload hbm_kernels the achieved GB/s of the HBM-bound kernels; the default, cfg2, is the
+  headline benchmark)
   cpu_baseline          the CPU oracle (a port of the reference's algorithm, plain PyTorch) timed on this
                         host's cores on a bounded sample of the same workload; its `gpu_vs_oracle` entry is the
                         full-size check of the timed step's embeddings (untimed extra fp32 oracle pass)
