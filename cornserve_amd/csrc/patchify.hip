@@ -41,39 +41,50 @@ __global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict_
 // the table with it).  Rows are ordered (t, block row, block col, row in block, col in block) with blocks of
 // merge x merge patches, columns (channel, temporal, y, x); temporal slot tt of row group t shows frame
 // min(t*temporal + tt, T-1): an image is one frame repeated, a video's last frame is repeated to fill a group.
-// One workgroup writes one output row (its place in the frame is worked out once, uniformly); a thread writes two
-// neighbouring x at a time.  P and TPS are the patch size and the temporal patch size as constants (the column
-// decomposition is then divisions by constants), or 0 for any value.  The table sits in LDS.
+// One workgroup writes QP_ROWS output rows (a row's place in the frame is worked out once and kept in LDS, as is
+// the table); a thread writes two neighbouring x at a time.
+// P and TPS are the patch size and the temporal patch size as constants (the column decomposition is then divisions
+// by constants), or 0 for any value.
+constexpr int QP_ROWS = 8;
 template <typename OUT, int P, int TPS>
 __global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __restrict__ frames, int T, int H, int W,
                                                                int p_any, int m, int tps_any, const float* __restrict__ table,
-                                                               OUT* __restrict__ out, int64_t ldo) {
+                                                               OUT* __restrict__ out, int64_t ldo, int rows) {
   __shared__ float lut[3 * 256];
   for (int i = threadIdx.x; i < 3 * 256; i += 256) lut[i] = table[i];
   __syncthreads();
   const int p = P ? P : p_any, tps = TPS ? TPS : tps_any;
   const int hp = p >> 1;
-  const int bw = W / (p * m), bh = H / (p * m);
-  int r = blockIdx.x;             // output row -> (t, block row, block column, row in block, column in block)
-  const int mx = r % m;
-  r /= m;
-  const int my = r % m;
-  r /= m;
-  const int bx = r % bw;
-  r /= bw;
-  const int by = r % bh;
-  const int t = r / bh;
-  const int y0 = (by * m + my) * p, x0 = (bx * m + mx) * p;
-  OUT* const dst_row = out + (int64_t)blockIdx.x * ldo;
   const int pairs = 3 * tps * p * hp;
-  for (int q = threadIdx.x; q < pairs; q += 256) {   // q -> (channel, temporal slot, y, x pair), x fastest
+  // where each of this workgroup's rows sits in the frame: (first frame of the group, top pixel row, left pixel column)
+  __shared__ int where[QP_ROWS][3];
+  const int row0 = blockIdx.x * QP_ROWS;
+  const int n_rows = min(rows - row0, QP_ROWS);
+  if (threadIdx.x < n_rows) {
+    const int bw = W / (p * m), bh = H / (p * m);
+    int r = row0 + threadIdx.x;   // output row -> (t, block row, block column, row in block, column in block)
+    const int mx = r % m;
+    r /= m;
+    const int my = r % m;
+    r /= m;
+    const int bx = r % bw;
+    r /= bw;
+    const int by = r % bh;
+    where[threadIdx.x][0] = (r / bh) * tps;
+    where[threadIdx.x][1] = (by * m + my) * p;
+    where[threadIdx.x][2] = (bx * m + mx) * p;
+  }
+  __syncthreads();
+  // work item -> (row of the workgroup, channel, temporal slot, y, x pair), x fastest: 2*q is the output column
+  for (int i = threadIdx.x; i < n_rows * pairs; i += 256) {
+    const int k = i / pairs, q = i - k * pairs;
     const int xp = q % hp, q1 = q / hp;
     const int py = q1 % p, q2 = q1 / p;
     const int tt = q2 % tps, c = q2 / tps;
-    const int f = min(t * tps + tt, T - 1);
-    const uint8_t* src = frames + (((int64_t)f * H + (y0 + py)) * W + (x0 + 2 * xp)) * 3 + c;
+    const int f = min(where[k][0] + tt, T - 1);
+    const uint8_t* src = frames + (((int64_t)f * H + (where[k][1] + py)) * W + (where[k][2] + 2 * xp)) * 3 + c;
     const float v0 = lut[c * 256 + src[0]], v1 = lut[c * 256 + src[3]];
-    OUT* dst = dst_row + 2 * q;   // column ((c*tps + tt)*p + py)*p + 2*xp == 2*q
+    OUT* dst = out + (int64_t)(row0 + k) * ldo + 2 * q;
     if constexpr (sizeof(OUT) == 2) {
       bf16x2_t o;
       o[0] = f2bf(v0);
@@ -87,15 +98,15 @@ __global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __
 }
 
 template <typename OUT>
-void launch_qwen_patchify_u8(dim3 grid, hipStream_t stream, const uint8_t* frames, int T, int H, int W, int p, int m,
+void launch_qwen_patchify_u8(int rows, hipStream_t stream, const uint8_t* frames, int T, int H, int W, int p, int m,
                              int tps, const float* table, OUT* out, int64_t ldo) {
-  const dim3 block(256);
+  const dim3 grid((unsigned)((rows + QP_ROWS - 1) / QP_ROWS)), block(256);
   if (p == 14 && tps == 2)
-    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 14, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo);
+    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 14, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
   else if (p == 16 && tps == 2)
-    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 16, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo);
+    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 16, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
   else
-    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 0, 0>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo);
+    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 0, 0>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
 }
 
 }  // namespace
@@ -112,11 +123,10 @@ extern "C" int cs_qwen_patchify_u8(const void* frames, int32_t T, int32_t H, int
   if (T == 0) return CS_OK;
   const int64_t rows = (int64_t)((T + temporal - 1) / temporal) * (H / patch) * (W / patch);
   if (rows > 0x7fffffff) return CS_ERR_TOO_LARGE;
-  const dim3 grid((unsigned)rows);
   if (out_fp32)
-    launch_qwen_patchify_u8<float>(grid, stream, (const uint8_t*)frames, T, H, W, patch, merge, temporal, table, (float*)out, ldo);
+    launch_qwen_patchify_u8<float>((int)rows, stream, (const uint8_t*)frames, T, H, W, patch, merge, temporal, table, (float*)out, ldo);
   else
-    launch_qwen_patchify_u8<bf16_t>(grid, stream, (const uint8_t*)frames, T, H, W, patch, merge, temporal, table, (bf16_t*)out, ldo);
+    launch_qwen_patchify_u8<bf16_t>((int)rows, stream, (const uint8_t*)frames, T, H, W, patch, merge, temporal, table, (bf16_t*)out, ldo);
   return cs_launch_status();
 }
 
