@@ -209,6 +209,10 @@ def hbm_kernels(dev, rows_list=(8192, 131072), reps: int = 20) -> dict:
         n_patch = (frames.shape[1] // 14) * (frames.shape[2] // 14)
         put("qwen_patchify_u8 (one frame -> bf16 patch rows)", frames.numel() + n_patch * 1176 * 2,
             lambda: ops.qwen_patchify_u8(frames, table, 14, 2, 2))
+        tiles = max(1, L // 729)
+        pxl = torch.randn((tiles, 3, 384, 384), generator=g).to(device=dev, dtype=torch.bfloat16)
+        put("patchify_nchw (384x384 tiles, patch 14)", tiles * 3 * 378 * 378 * 2 + tiles * 729 * 592 * 2,
+            lambda: ops.patchify_nchw(pxl, 14, 592))
         out[f"rows_{L}"] = res
     return {"metric": "achieved GB/s of the HBM-bound kernels on 1 MI355X", "unit": "GB/s", "n_gpus": 1, "peak_GB_per_s": 8000,
             "higher_is_better": True, "dtype": "bf16", "data": "synthetic",

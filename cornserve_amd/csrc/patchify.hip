@@ -14,8 +14,8 @@ namespace {
 __global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict__ px, int B, int C, int H, int W,
                                                        int p, bf16_t* __restrict__ out, int64_t ldo) {
   const int gw = W / p, gh = H / p;
-  const int64_t total = (int64_t)B * gh * C * p * gw;
-  int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const unsigned total = (unsigned)B * gh * C * p * gw;   // < 2^31, checked on the host: 32-bit index arithmetic
+  unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const int x = i % gw;
   i /= gw;
@@ -138,6 +138,7 @@ extern "C" int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_
     return CS_ERR_INVALID_ARG;
   if (B == 0) return CS_OK;
   const int64_t total = (int64_t)B * (H / patch) * C * patch * (W / patch);
+  if (total > 0x7fffffff) return CS_ERR_TOO_LARGE;
   hipLaunchKernelGGL(patchify_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
                      (const bf16_t*)pixels, B, C, H, W, patch, (bf16_t*)out, ldo);
   return cs_launch_status();

@@ -85,10 +85,10 @@ __global__ __launch_bounds__(256) void pos_embed_interp_kernel(const bf16_t* __r
   const int mm = merge * merge;
   const int h = it.gh * merge, w = it.gw * merge;
   const int64_t n = (int64_t)it.t * h * w * chunks;
-  const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;   // (below 2^31: checked on the host)
   if (idx >= n) return;
-  const int c = (int)(idx % chunks);
-  const int pl = (int)(idx / chunks);         // patch within the item, in patch (block-major) order
+  const int pl = (int)(idx / (unsigned)chunks);   // patch within the item, in patch (block-major) order
+  const int c = (int)(idx - (unsigned)pl * chunks);
   const int ul = pl / mm, s = pl - ul * mm;
   const int rem = ul % (it.gh * it.gw);
   const int y = (rem / it.gw) * merge + s / merge, x = (rem % it.gw) * merge + s % merge;
@@ -305,7 +305,7 @@ extern "C" int cs_pos_embed_interp(const void* table, int32_t side, int32_t E, c
   if (n_items == 0 || max_units_per_item == 0) return CS_OK;
   if (n_items > 65535) return CS_ERR_TOO_LARGE;
   const int64_t work = (int64_t)max_units_per_item * merge * merge * (E / 8);
-  if ((work + 255) / 256 > 0x7fffffff) return CS_ERR_TOO_LARGE;
+  if (work > 0x7fffff00) return CS_ERR_TOO_LARGE;   // the kernel indexes its work with 32 bits
   const dim3 grid((unsigned)((work + 255) / 256), n_items), block(256);
   hipLaunchKernelGGL(pos_embed_interp_kernel, grid, block, 0, stream, (const bf16_t*)table, side, E,
                      (const ItemMeta*)item_meta, merge, (bf16_t*)out, ldo);
