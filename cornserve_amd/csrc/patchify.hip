@@ -5,33 +5,57 @@
 // NCHW pixels equals a GEMM between the flattened non-overlapping patches and the [E, C*p*p] weight.
 // This kernel lays the patches out as the GEMM's A operand: row m = (b, py, px), column (c, ky, kx),
 // zero-padded to the leading dimension so the GEMM's 16-byte loads stay aligned (C*p*p = 588 is not a
-// multiple of 8).  Consecutive threads take consecutive px of one image row, so the reads of a wave
-// cover one contiguous 64*p*2-byte span of the source image.
+// multiple of 8).  A workgroup takes a run of up to npx neighbouring patches of one patch row: it copies
+// their C*p image-row segments (contiguous npx*p pixels each) into LDS with coalesced loads, then writes the
+// npx output rows (one contiguous span of npx*ldo elements) with coalesced stores of V elements per lane,
+// gathering the pairs from LDS.
 #include "common.h"
 
 namespace {
 
-__global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict__ px, int B, int C, int H, int W,
-                                                       int p, bf16_t* __restrict__ out, int64_t ldo) {
-  const int gw = W / p, gh = H / p;
-  const unsigned total = (unsigned)B * gh * C * p * gw;   // < 2^31, checked on the host: 32-bit index arithmetic
-  unsigned i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= total) return;
-  const int x = i % gw;
-  i /= gw;
-  const int ky = i % p;
-  i /= p;
-  const int c = i % C;
-  i /= C;
-  const int y = i % gh;
-  const int b = (int)(i / gh);
-  const bf16_t* src = px + (((int64_t)b * C + c) * H + (y * p + ky)) * W + x * p;
-  bf16_t* dst = out + ((int64_t)(b * gh + y) * gw + x) * ldo + (c * p + ky) * p;
-  for (int kx = 0; kx < p; kx += 2) *(bf16x2_t*)(dst + kx) = *(const bf16x2_t*)(src + kx);
-  // the thread that owns the last (c, ky) slice of a patch also clears the row's padding
-  if (c == C - 1 && ky == p - 1) {
-    bf16_t* row = out + ((int64_t)(b * gh + y) * gw + x) * ldo;
-    for (int k = C * p * p; k < ldo; ++k) row[k] = f2bf(0.f);
+// P is the patch size as a constant (divisions by constants), or 0 for any even value; V = elements per store.
+template <int P, int V>
+__global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict__ px, int C, int H, int W, int p_any,
+                                                       int gh, int gw, int npx, int chunks,
+                                                       bf16_t* __restrict__ out, int ldo) {
+  extern __shared__ bf16x2_t band[];   // [C*p][n*p/2] pixel pairs
+  const int p = P ? P : p_any;
+  const int hp = p >> 1;
+  unsigned wg = blockIdx.x;            // -> (image, patch row, run of patches)
+  const int ch = wg % (unsigned)chunks;
+  wg /= (unsigned)chunks;
+  const int y = wg % (unsigned)gh, b = wg / (unsigned)gh;
+  const int x0 = ch * npx;
+  const int n = min(npx, gw - x0);
+  const int hw = n * hp;               // pairs per image-row segment
+  const int rows = C * p;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  for (int r = wave; r < rows; r += 4) {   // one wave per image-row segment
+    const int c = r / p, ky = r - c * p;
+    const bf16_t* src = px + (((int64_t)b * C + c) * H + (y * p + ky)) * W + x0 * p;
+    for (int xx = lane; xx < hw; xx += 64) band[r * hw + xx] = *(const bf16x2_t*)(src + 2 * xx);
+  }
+  __syncthreads();
+  const int K = rows * p;
+  const unsigned upr = (unsigned)ldo / V;   // stores per output row
+  bf16_t* span = out + ((int64_t)(b * gh + y) * gw + x0) * ldo;
+  for (unsigned i = threadIdx.x; i < (unsigned)n * upr; i += 256) {
+    const int kp = i / upr;
+    const int k0 = (int)(i - kp * upr) * V;
+    int v[V / 2];
+#pragma unroll
+    for (int e = 0; e < V / 2; ++e) {
+      const int k = k0 + 2 * e;   // output column -> (image-row segment c*p + ky, kx); a pair never straddles segments (p even)
+      const int r = k / p, kx = k - r * p;
+      v[e] = k < K ? __builtin_bit_cast(int, band[r * hw + kp * hp + (kx >> 1)]) : 0;   // bf16 zero is all-zero bits
+    }
+    bf16_t* dst = span + (int64_t)i * V;
+    if constexpr (V == 8) {
+      i32x4_t o = {v[0], v[1], v[2], v[3]};
+      *(i32x4_t*)dst = o;
+    } else {
+      *(int*)dst = v[0];
+    }
   }
 }
 
@@ -137,9 +161,28 @@ extern "C" int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_
       W < patch || W % 2 || ldo < (int64_t)C * patch * patch || ldo % 2 || (((uintptr_t)pixels | (uintptr_t)out) & 3))
     return CS_ERR_INVALID_ARG;
   if (B == 0) return CS_OK;
-  const int64_t total = (int64_t)B * (H / patch) * C * patch * (W / patch);
-  if (total > 0x7fffffff) return CS_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(patchify_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream,
-                     (const bf16_t*)pixels, B, C, H, W, patch, (bf16_t*)out, ldo);
+  const int gh = H / patch, gw = W / patch;
+  if (ldo > 0x7fffffff / 16 || (int64_t)C * patch * patch > 0x7fffffff / 16) return CS_ERR_TOO_LARGE;
+  // patches per workgroup: eight, fewer when the image-row segments of eight would not fit 64 KB of LDS
+  int npx = 8;
+  while (npx > 1 && (int64_t)C * patch * npx * patch * 2 > 65536) npx >>= 1;
+  const int64_t lds = (int64_t)C * patch * npx * patch * 2;
+  if (lds > 65536) return CS_ERR_TOO_LARGE;
+  const int chunks = (gw + npx - 1) / npx;
+  const int64_t wgs = (int64_t)B * gh * chunks;
+  if (wgs > 0x7fffffff) return CS_ERR_TOO_LARGE;
+  const bool wide = ldo % 8 == 0 && ((uintptr_t)out & 15) == 0;
+  const dim3 grid((unsigned)wgs), block(256);
+#define CS_PATCHIFY(P, V)                                                                                       \
+  hipLaunchKernelGGL((patchify_kernel<P, V>), grid, block, (size_t)lds, stream, (const bf16_t*)pixels, C, H, W, \
+                     patch, gh, gw, npx, chunks, (bf16_t*)out, (int)ldo)
+  if (patch == 14) {
+    if (wide) CS_PATCHIFY(14, 8); else CS_PATCHIFY(14, 2);
+  } else if (patch == 16) {
+    if (wide) CS_PATCHIFY(16, 8); else CS_PATCHIFY(16, 2);
+  } else {
+    if (wide) CS_PATCHIFY(0, 8); else CS_PATCHIFY(0, 2);
+  }
+#undef CS_PATCHIFY
   return cs_launch_status();
 }

@@ -658,6 +658,24 @@ def test_patchify_nchw_drops_the_partial_patches(ops, dev):
     assert torch.equal(got[:, :588].float(), ref) and not got[:, 588:].any()
 
 
+@pytest.mark.parametrize("B,C,H,W,patch,ldo", [
+    (2, 3, 896, 896, 14, 592),    # config-3 tiles: 64 patches per row, eight runs of eight
+    (1, 3, 70, 154, 14, 590),     # 11 patches per row (last run has three), rows that are not whole 16-byte vectors
+    (2, 3, 64, 176, 16, 768),     # patch 16, no padding columns
+    (1, 5, 30, 50, 10, 504),      # any even patch size, five channels, partial patches dropped
+    (1, 3, 12, 36, 6, 110),       # narrow stores with padding
+    (1, 40, 56, 56, 28, 31360),   # eight patches' row segments exceed the LDS budget: fewer patches per workgroup
+])
+def test_patchify_nchw_shapes(ops, dev, B, C, H, W, patch, ldo):
+    px = rnd((B, C, H, W), 1.0, 73)
+    got = ops.patchify_nchw(px.to(dev), patch, ldo).cpu()
+    gh, gw, K = H // patch, W // patch, C * patch * patch
+    ref = F.unfold(px.float()[:, :, :gh * patch, :gw * patch], kernel_size=patch, stride=patch)
+    ref = ref.transpose(1, 2).reshape(B * gh * gw, K)
+    assert got.shape == (B * gh * gw, ldo)
+    assert torch.equal(got[:, :K].float(), ref) and not got[:, K:].any()
+
+
 def test_gemm_random_shapes_epilogues_and_folds(ops, dev):
     """A seeded sweep over row counts either side of every tile height (1 .. 5000), widths, depths, epilogues and the
     folded-norm forms, against fp32 torch arithmetic with the reference's rounding points."""
