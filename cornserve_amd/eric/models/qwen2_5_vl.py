@@ -314,9 +314,12 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         win = self.window_size // merge // self.patch_size
         dev = self.device
         sl = ops.vit_seqlens_host(grid_thw, merge, win)
-        meta = ops.host_to_device(sl.item_meta, dev)
+        (work_win, max_win), (work_full, max_full) = ops.attn_work_host(sl.cu_window), ops.attn_work_host(sl.cu_full)
+        # one host-to-device copy for the three small arrays
+        meta, dwin, dfull = ops.host_to_device_packed([sl.item_meta, work_win, work_full], dev)
         ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, merge, win, self._ensure_packed()["inv_freq"])
-        return ix, ops.attn_plan(sl.cu_window, dev), ops.attn_plan(sl.cu_full, dev), sl.total_patches
+        return (ix, ops.AttnPlan(dwin, work_win.shape[0], max_win), ops.AttnPlan(dfull, work_full.shape[0], max_full),
+                sl.total_patches)
 
     def forward_device(self, pixel_values: torch.Tensor, grid_thw: np.ndarray, mark=None) -> list[torch.Tensor]:
         """pixel_values: bf16 [L, C*T*P*P] already on the device; grid_thw: host int64 [n,3].

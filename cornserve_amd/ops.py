@@ -39,6 +39,28 @@ def host_to_device(a: np.ndarray, device: torch.device) -> torch.Tensor:
     return staged.to(device, non_blocking=True)
 
 
+def host_to_device_packed(arrays: list[np.ndarray], device: torch.device) -> list[torch.Tensor]:
+    """Several small host arrays -> device tensors with ONE asynchronous copy: the arrays are laid end to end
+    (256-byte aligned) in one pinned staging buffer and the results are views of one device buffer."""
+    arrays = [np.ascontiguousarray(a) for a in arrays]
+    offs, total = [], 0
+    for a in arrays:
+        offs.append(total)
+        total += (a.nbytes + 255) // 256 * 256
+    if total == 0:
+        return [torch.from_numpy(a.copy()).to(device) for a in arrays]
+    staged = torch.empty((total,), dtype=torch.uint8, pin_memory=True)
+    host = staged.numpy()
+    for a, o in zip(arrays, offs):
+        host[o : o + a.nbytes] = a.reshape(-1).view(np.uint8)
+    dev = staged.to(device, non_blocking=True)
+    out = []
+    for a, o in zip(arrays, offs):
+        dt = torch.from_numpy(a[:0].reshape(-1)).dtype
+        out.append(dev[o : o + a.nbytes].view(dt).view(a.shape))
+    return out
+
+
 def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
@@ -376,12 +398,13 @@ class AttnPlan:
     max_seqlen: int
 
 
-def attn_plan(cu_seqlens_host: np.ndarray, device: torch.device) -> AttnPlan:
+def attn_work_host(cu_seqlens_host: np.ndarray) -> tuple[np.ndarray, int]:
+    """Host half of attn_plan: the work list int32 [n_work, 4] (still on the host) and the longest segment."""
     lib = _l.load()
     cu = np.ascontiguousarray(cu_seqlens_host, dtype=np.int32)
     n_seg = cu.shape[0] - 1
     if n_seg <= 0:
-        return AttnPlan(torch.zeros((0, 4), dtype=torch.int32, device=device), 0, 1)
+        return np.zeros((0, 4), np.int32), 1
     lens = np.diff(cu)
     max_seqlen = int(lens.max())
     bq = lib.cs_attn_block_q(max_seqlen)
@@ -390,7 +413,12 @@ def attn_plan(cu_seqlens_host: np.ndarray, device: torch.device) -> AttnPlan:
     n_work = ctypes.c_int32(0)
     _l.check(lib.cs_attn_work_host(cu.ctypes.data, n_seg, bq, work.ctypes.data, cap, ctypes.byref(n_work)),
              "cs_attn_work_host")
-    return AttnPlan(host_to_device(work[: n_work.value], device), n_work.value, max_seqlen)
+    return work[: n_work.value], max_seqlen
+
+
+def attn_plan(cu_seqlens_host: np.ndarray, device: torch.device) -> AttnPlan:
+    work, max_seqlen = attn_work_host(cu_seqlens_host)
+    return AttnPlan(host_to_device(work, device), work.shape[0], max_seqlen)
 
 
 def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan, heads: int, head_dim: int,
