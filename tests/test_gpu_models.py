@@ -167,6 +167,64 @@ def test_qwen_fp8_weights(dev):
     check(out[0], ref[0], REL_FP8, "fp8 weights vs de-quantised fp32 oracle")
 
 
+def test_full_size_configs_through_properties(dev):
+    """The benchmark configurations at their full size (32 blocks, full attention at 7/15/23/31), where the CPU oracle
+    is too slow for the whole batch, through properties that do not depend on the size: an item's embedding is the
+    same bits alone and in the batch, a permuted batch gives permuted outputs, equal items give equal outputs; and
+    one image of the batch against the oracle, with the distance of the reference's own bf16 arithmetic to the fp32
+    result as the yardstick (at 64 residual additions in bf16 that distance itself is about the 2e-2 bar)."""
+    full = (7, 15, 23, 31)
+    model, sd, ocfg = build_qwen(dev, 32, full, seed=21)
+
+    def run(px, grid, modality=Modality.IMAGE):
+        key = "pixel_values" if modality == Modality.IMAGE else "pixel_values_videos"
+        gkey = "image_grid_thw" if modality == Modality.IMAGE else "video_grid_thw"
+        return model(modality, "", {key: px, gkey: grid})
+
+    # config 2: 8 images of 448 x 448
+    px, grid = synth.qwen_inputs([(1, 32, 32)] * 8, seed=21)
+    out = run(px, grid)
+    assert len(out) == 8 and all(o.shape == (256, 3584) and torch.isfinite(o.float()).all() for o in out)
+    perm = [3, 0, 7, 5, 1, 6, 2, 4]
+    out_p = run([px[i] for i in perm], [grid[i] for i in perm])
+    assert all(torch.equal(out_p[j], out[i]) for j, i in enumerate(perm)), "a permuted batch permutes the outputs"
+    alone = run([px[5]], [grid[5]])[0]
+    assert torch.equal(alone, out[5]), "an item alone equals the item in the batch"
+    assert not torch.equal(out[0], out[1])
+    sd16 = {k: v.bfloat16() for k, v in sd.items()}
+    sd32 = {k: v.float() for k, v in sd16.items()}
+    px5 = px[5].bfloat16()
+    ref16 = oq.forward(sd16, ocfg, [px5], [grid[5]], dtype=torch.bfloat16)[0].float()
+    ref32 = oq.forward(sd32, ocfg, [px5.float()], [grid[5]], dtype=torch.float32)[0]
+    got = out[5].float().cpu()
+    dist = lambda a, b: ((a - b).abs().max() / b.abs().max()).item()
+    cos = lambda a, b: F.cosine_similarity(a.flatten(), b.flatten(), dim=0).item()
+    assert cos(got, ref32) >= COS_MIN and cos(got, ref16) >= COS_MIN
+    yard = dist(ref16, ref32)
+    assert dist(got, ref32) <= max(REL_BF16, 1.25 * yard), (dist(got, ref32), yard)
+
+    # config 4: 16 images with sides drawn from the multiples of 28 in [224, 1344]
+    grids = synth.ragged_grids(16, seed=4)
+    px, grid = synth.qwen_inputs(grids, seed=22)
+    out = run(px, grid)
+    assert [tuple(o.shape) for o in out] == [(h * w // 4, 3584) for _, h, w in grids]
+    assert all(torch.isfinite(o.float()).all() for o in out)
+    order = sorted(range(16), key=lambda i: grids[i][1] * grids[i][2])
+    for i in (order[0], order[8], order[-1]):   # smallest, median and largest image
+        assert torch.equal(run([px[i]], [grid[i]])[0], out[i]), f"ragged item {i} {grids[i]}"
+    del out
+
+    # config 5: fp8-e4m3 weights, two video clips of 16 frames at 336 x 588
+    del model
+    torch.cuda.empty_cache()
+    model, _, _ = build_qwen(dev, 32, full, seed=21, weight_format="fp8_e4m3")
+    px, grid = synth.qwen_inputs([(8, 24, 42)] * 2, seed=23)
+    out = run(px, grid, Modality.VIDEO)
+    assert all(o.shape == (2016, 3584) and torch.isfinite(o.float()).all() for o in out)
+    twice = run([px[1], px[1]], [grid[1], grid[1]], Modality.VIDEO)
+    assert torch.equal(twice[0], twice[1]) and torch.equal(twice[0], out[1]), "equal clips give equal embeddings"
+
+
 def test_worker_hand_off_of_real_embeddings(dev, tmp_path):
     """Embeddings of a real forward pass through the worker's hand-off to the mock sidecar: contiguous device
     tensors (what the reference's sender exports by IPC handle), saved and reloaded bit-exactly."""
@@ -417,6 +475,33 @@ def test_gemma3_real_resolution_and_crops(dev):
         check(out[i], ref[i], REL_BF16, f"gemma3 896 item {i}")
     with pytest.raises(ValueError, match="not found"):
         model(Modality.IMAGE, "missing", {"pixel_values": px, "num_crops": crops})
+
+
+def test_gemma3_full_size_through_properties(dev):
+    """Config 3 at its full size (27 layers, four 896 x 896 images): a permuted batch gives permuted outputs, an
+    image alone equals the image in the batch (bit for bit), and one image against the oracle with the distance of
+    the bf16 oracle to the fp32 oracle as the yardstick."""
+    model, sd, ocfg = build_gemma(dev, 27, 896, 2560, 256, seed=31)
+    px = [synth.uniform(31, f"img{i}", (1, 3, 896, 896), -1, 1) for i in range(4)]
+    crops = [torch.tensor([0])] * 4
+    out = model(Modality.IMAGE, "a", {"pixel_values": px, "num_crops": crops})
+    assert len(out) == 4 and all(o.shape == (256, 2560) and torch.isfinite(o.float()).all() for o in out)
+    perm = [2, 0, 3, 1]
+    out_p = model(Modality.IMAGE, "a", {"pixel_values": [px[i] for i in perm], "num_crops": crops})
+    assert all(torch.equal(out_p[j], out[i]) for j, i in enumerate(perm))
+    alone = model(Modality.IMAGE, "a", {"pixel_values": [px[2]], "num_crops": [crops[2]]})[0]
+    assert torch.equal(alone, out[2])
+    sd16 = {k: v.bfloat16() for k, v in sd.items()}
+    sd32 = {k: v.float() for k, v in sd16.items()}
+    p2 = px[2].bfloat16()
+    ref16 = og.forward(sd16, ocfg, [p2], [crops[2]], dtype=torch.bfloat16)[0].float()
+    ref32 = og.forward(sd32, ocfg, [p2.float()], [crops[2]], dtype=torch.float32)[0]
+    got = out[2].float().cpu()
+    dist = lambda a, b: ((a - b).abs().max() / b.abs().max()).item()
+    cos = lambda a, b: F.cosine_similarity(a.flatten(), b.flatten(), dim=0).item()
+    assert cos(got, ref32) >= COS_MIN and cos(got, ref16) >= COS_MIN
+    yard = dist(ref16, ref32)
+    assert dist(got, ref32) <= max(REL_BF16, 1.25 * yard), (dist(got, ref32), yard)
 
 
 def test_layernorm_encoders_without_folded_norms(dev):
