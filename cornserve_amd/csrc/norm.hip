@@ -111,6 +111,30 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const bf16_t* __restrict
   }
 }
 
+// Eight per-lane partial sums -> their eight totals over the wave, with 10 lane exchanges instead of 48: each of
+// the first three exchanges (lane ^ 32, ^ 16, ^ 8) hands the partner the half of the values it keeps, so the number
+// of live values halves; three more exchanges finish the one value left.  Lane l returns the total of part l >> 3.
+static_assert(CS_SUMSQ_PARTS == 8, "wave_sum_parts halves eight values three times");
+CS_DEVICE float wave_sum_parts(const float (&part)[8], int lane) {
+  const bool b5 = lane & 32, b4 = lane & 16, b3 = lane & 8;
+  float a[4], b[2];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const float keep = b5 ? part[4 + i] : part[i], give = b5 ? part[i] : part[4 + i];
+    a[i] = keep + __shfl_xor(give, 32, 64);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const float keep = b4 ? a[2 + i] : a[i], give = b4 ? a[i] : a[2 + i];
+    b[i] = keep + __shfl_xor(give, 16, 64);
+  }
+  float c = (b3 ? b[1] : b[0]) + __shfl_xor(b3 ? b[0] : b[1], 8, 64);
+  c += __shfl_xor(c, 4, 64);
+  c += __shfl_xor(c, 2, 64);
+  c += __shfl_xor(c, 1, 64);
+  return c;
+}
+
 // Sums of squares of a row in parts of 160 columns (20 chunks): the variance term of RMSNorm in the form
 // that a GEMM with CsGemmArgs.a_row_sumsq consumes.  out is [rows][CS_SUMSQ_PARTS].
 template <bool WITH_SUM>
@@ -144,20 +168,12 @@ __global__ __launch_bounds__(256) void row_sumsq_kernel(const bf16_t* __restrict
       if (WITH_SUM) spart[WITH_SUM ? q : 0] += (q == q_of_chunk) ? sm : 0.f;
     }
   }
-#pragma unroll
-  for (int q = 0; q < CS_SUMSQ_PARTS; ++q) {
-    part[q] = wave_sum(part[q]);
-    if (WITH_SUM) spart[WITH_SUM ? q : 0] = wave_sum(spart[WITH_SUM ? q : 0]);
-  }
-  if (lane == 0) {
-    float* o = out + (int64_t)row * CS_SUMSQ_PARTS;
-#pragma unroll
-    for (int q = 0; q < CS_SUMSQ_PARTS; q += 4) *(f32x4_t*)(o + q) = f32x4_t{part[q], part[q + 1], part[q + 2], part[q + 3]};
-    if constexpr (WITH_SUM) {
-      float* so = sum_out + (int64_t)row * CS_SUMSQ_PARTS;
-#pragma unroll
-      for (int q = 0; q < CS_SUMSQ_PARTS; q += 4) *(f32x4_t*)(so + q) = f32x4_t{spart[q], spart[q + 1], spart[q + 2], spart[q + 3]};
-    }
+  // lane l ends up with the total of part l / 8: eight lanes each store one value
+  const float tot = wave_sum_parts(part, lane);
+  if ((lane & 7) == 0) out[(int64_t)row * CS_SUMSQ_PARTS + (lane >> 3)] = tot;
+  if constexpr (WITH_SUM) {
+    const float stot = wave_sum_parts(spart, lane);
+    if ((lane & 7) == 0) sum_out[(int64_t)row * CS_SUMSQ_PARTS + (lane >> 3)] = stot;
   }
 }
 
