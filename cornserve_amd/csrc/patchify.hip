@@ -68,7 +68,7 @@ __global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict_
 // One workgroup writes QP_ROWS output rows (a row's place in the frame is worked out once and kept in LDS, as is
 // the table); a thread writes two neighbouring x at a time.
 // P and TPS are the patch size and the temporal patch size as constants (the column decomposition is then divisions
-// by constants), or 0 for any value.
+// by constants), or 0 for any value.  This form serves the sizes the segment kernel below does not take.
 constexpr int QP_ROWS = 8;
 template <typename OUT, int P, int TPS>
 __global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __restrict__ frames, int T, int H, int W,
@@ -121,14 +121,128 @@ __global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __
   }
 }
 
+typedef uint32_t u32x4a_t __attribute__((ext_vector_type(4), aligned(4)));   // four words at 4-byte alignment
+
+// The same operation for the usual patch sizes (P = 14, 16), organised by source segments: the 3*P bytes of one
+// image row of one patch hold the P pixels of all three channels, i.e. three runs of P output values.  A workgroup
+// takes a few output rows (seg_rows_per_workgroup) = rows * tps * P segments; it copies the aligned 4-byte words that cover every segment
+// into LDS with coalesced loads (consecutive lanes take consecutive 16-byte pieces of a segment; every word loaded holds at
+// least one byte of the frames, so no load leaves the allocation), then one lane per segment shifts its words into
+// place, looks the 3*P bytes up in the table and stores the three runs.  About a fifth of the instructions per output
+// value of the per-value kernel above.
+// Output rows per workgroup of the segment kernel: with the usual temporal size 2 a row has 2 * P segments, and the
+// workgroup has one lane per segment (P = 14: 9 rows = 252 segments, P = 16: 8 rows = 256).
+constexpr int seg_rows_per_workgroup(int p) { return 256 / (2 * p); }
+
+template <typename OUT, int P>
+__global__ __launch_bounds__(256) void qwen_patchify_u8_seg_kernel(const uint8_t* __restrict__ frames, int T, int H, int W,
+                                                                   int m, int tps, const float* __restrict__ table,
+                                                                   OUT* __restrict__ out, int64_t ldo, int rows) {
+  constexpr int ROWS = seg_rows_per_workgroup(P);
+  constexpr int SEG = 3 * P;               // bytes per segment
+  constexpr int NDW = (SEG + 3 + 3) / 4;   // words that cover a segment starting at byte 0..3 of a word
+  constexpr int ND = (SEG + 3) / 4;        // words of a segment once shifted into place
+  __shared__ float lut[3 * 256];
+  __shared__ int where[ROWS][3];
+  extern __shared__ __attribute__((aligned(16))) char dyn[];   // int64 segment offsets, then NDW words per segment
+  for (int i = threadIdx.x; i < 3 * 256; i += 256) lut[i] = table[i];
+  const int row0 = blockIdx.x * ROWS;
+  const int n_rows = min(rows - row0, ROWS);
+  if (threadIdx.x < n_rows) {
+    const int bw = W / (P * m), bh = H / (P * m);
+    int r = row0 + threadIdx.x;   // output row -> (t, block row, block column, row in block, column in block)
+    const int mx = r % m;
+    r /= m;
+    const int my = r % m;
+    r /= m;
+    const int bx = r % bw;
+    r /= bw;
+    const int by = r % bh;
+    where[threadIdx.x][0] = (r / bh) * tps;
+    where[threadIdx.x][1] = (by * m + my) * P;
+    where[threadIdx.x][2] = (bx * m + mx) * P;
+  }
+  __syncthreads();
+  const int spr = tps * P;              // segments per output row
+  const int nseg = n_rows * spr;
+  const int max_seg = (ROWS * spr + 1) & ~1;   // even: the words behind the offsets stay 16-byte aligned
+  int64_t* segoff = (int64_t*)dyn;      // byte offset of each segment in frames
+  uint32_t* words = (uint32_t*)(dyn + (size_t)max_seg * 8);
+  for (int s = threadIdx.x; s < nseg; s += 256) {
+    const int k = s / spr, rem = s - k * spr;
+    const int tt = rem / P, py = rem - tt * P;
+    const int f = min(where[k][0] + tt, T - 1);
+    segoff[s] = (((int64_t)f * H + (where[k][1] + py)) * W + where[k][2]) * 3;
+  }
+  __syncthreads();
+  // four words per lane and load (words need 4-byte alignment only); a chunk's tail is left out word by word where it
+  // would lie past the segment's last byte
+  constexpr int NCH = (NDW + 3) / 4;
+  for (int i = threadIdx.x; i < nseg * NCH; i += 256) {
+    const int s = i / NCH, q = i - s * NCH;
+    const uintptr_t addr = (uintptr_t)frames + segoff[s];
+    const int last = ((int)(addr & 3) + SEG - 1) >> 2;   // index of the last word that holds a byte of the segment
+    const uint32_t* src = (const uint32_t*)(addr & ~(uintptr_t)3) + 4 * q;
+    uint32_t* dst = words + s * NDW + 4 * q;
+    const int n = min(last - 4 * q + 1, min(4, NDW - 4 * q));   // words of this chunk to fetch (>= 1 for the chunks of P = 14, 16)
+    uint32_t w[4] = {0, 0, 0, 0};
+    if (n >= 4) {
+      const u32x4a_t v = *(const u32x4a_t*)src;
+      w[0] = v[0], w[1] = v[1], w[2] = v[2], w[3] = v[3];
+    } else {
+      if (n > 0) w[0] = src[0];
+      if (n > 1) w[1] = src[1];
+      if (n > 2) w[2] = src[2];
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (4 * q + j < NDW) dst[j] = w[j];
+  }
+  __syncthreads();
+  for (int s = threadIdx.x; s < nseg; s += 256) {
+    const int lead = (int)(((uintptr_t)frames + segoff[s]) & 3);
+    uint32_t raw[NDW + 1], d[ND];
+#pragma unroll
+    for (int j = 0; j < NDW; ++j) raw[j] = words[s * NDW + j];
+    raw[NDW] = 0;
+#pragma unroll
+    for (int j = 0; j < ND; ++j) d[j] = __builtin_amdgcn_alignbyte(raw[j + 1], raw[j], lead);   // bytes lead.. of (raw[j+1]:raw[j])
+    const int k = s / spr, rem = s - k * spr;   // rem = tt * P + py: the run's place inside a channel's columns
+    OUT* dst = out + (int64_t)(row0 + k) * ldo + rem * P;
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      OUT* o = dst + c * spr * P;
+#pragma unroll
+      for (int x = 0; x < P; x += 2) {
+        const int b0 = 3 * x + c, b1 = 3 * (x + 1) + c;
+        const float v0 = lut[c * 256 + ((d[b0 >> 2] >> (8 * (b0 & 3))) & 255)];
+        const float v1 = lut[c * 256 + ((d[b1 >> 2] >> (8 * (b1 & 3))) & 255)];
+        if constexpr (sizeof(OUT) == 2) {
+          bf16x2_t q;
+          q[0] = f2bf(v0);
+          q[1] = f2bf(v1);
+          *(bf16x2_t*)(o + x) = q;
+        } else {
+          o[x] = v0;
+          o[x + 1] = v1;
+        }
+      }
+    }
+  }
+}
+
 template <typename OUT>
 void launch_qwen_patchify_u8(int rows, hipStream_t stream, const uint8_t* frames, int T, int H, int W, int p, int m,
                              int tps, const float* table, OUT* out, int64_t ldo) {
   const dim3 grid((unsigned)((rows + QP_ROWS - 1) / QP_ROWS)), block(256);
-  if (p == 14 && tps == 2)
-    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 14, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
-  else if (p == 16 && tps == 2)
-    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 16, 2>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
+  // segment form: LDS for the offsets and words of the segments of a workgroup's rows
+  const int seg_rows = (p == 14 || p == 16) ? seg_rows_per_workgroup(p) : 1;
+  const size_t seg_lds = (size_t)((seg_rows * tps * p + 1) & ~1) * (8 + 4 * ((3 * p + 6) / 4));
+  const dim3 seg_grid((unsigned)((rows + seg_rows - 1) / seg_rows));
+  if (p == 14 && seg_lds <= 48 * 1024)
+    hipLaunchKernelGGL((qwen_patchify_u8_seg_kernel<OUT, 14>), seg_grid, block, seg_lds, stream, frames, T, H, W, m, tps, table, out, ldo, rows);
+  else if (p == 16 && seg_lds <= 48 * 1024)
+    hipLaunchKernelGGL((qwen_patchify_u8_seg_kernel<OUT, 16>), seg_grid, block, seg_lds, stream, frames, T, H, W, m, tps, table, out, ldo, rows);
   else
     hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 0, 0>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
 }

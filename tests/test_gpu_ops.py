@@ -100,6 +100,9 @@ def test_patchify_bit_exact(ops, dev):
     (8, 336, 588, 14, 2, 2),    # config-5 style video
     (5, 56, 84, 14, 2, 2),      # odd frame count: the last frame fills the last group
     (7, 24, 36, 2, 3, 3),       # other patch / merge / temporal sizes
+    (3, 64, 96, 16, 2, 2),      # patch 16
+    (9, 28, 56, 14, 1, 3),      # patch 14 with another merge / temporal size
+    (20, 28, 28, 14, 2, 10),    # temporal size beyond what the segment form stages: per-value form
 ])
 def test_qwen_patchify_u8_bit_exact(ops, dev, t, h, w, patch, merge, temporal):
     from cornserve_amd.eric import frames as fr
@@ -116,6 +119,25 @@ def test_qwen_patchify_u8_bit_exact(ops, dev, t, h, w, patch, merge, temporal):
         assert torch.equal(got16.cpu(), torch.from_numpy(ref).bfloat16())   # the reference's .to(dtype), :415-419
     with pytest.raises(ValueError):
         ops.qwen_patchify_u8(torch.zeros((1, 30, 28, 3), dtype=torch.uint8, device=dev), table.to(dev), 14, 2, 2)
+
+
+@pytest.mark.parametrize("patch", [14, 16])
+def test_qwen_patchify_u8_unaligned_frames(ops, dev, patch):
+    """Frames that start at any byte offset of a 4-byte word (a view into a larger buffer), last frame at the very end
+    of the buffer."""
+    from cornserve_amd.eric import frames as fr
+    from oracle import qwen_preprocess as qp
+
+    t, h, w = 3, 2 * patch * 2, 3 * patch * 2
+    table = fr.byte_table(arithmetic="numpy")
+    n = t * h * w * 3
+    for lead in range(4):
+        buf = np.random.default_rng(100 + lead).integers(0, 256, lead + n, dtype=np.uint8)
+        frames = buf[lead:].reshape(t, h, w, 3)
+        ref, _ = qp.patchify_frames(frames, qp.normalization_table(arithmetic="numpy"), patch, 2, 2)
+        dbuf = torch.from_numpy(buf).to(dev)
+        got = ops.qwen_patchify_u8(dbuf[lead:].view(t, h, w, 3), table.to(dev), patch, 2, 2, dtype=torch.float32)
+        assert np.array_equal(got.cpu().numpy(), ref), lead
 
 
 @pytest.mark.parametrize("rows,H", [(1, 1280), (1023, 1280), (64, 1152), (5, 64), (7, 5120)])
