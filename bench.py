@@ -11,7 +11,7 @@ with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
                         block, which the library runs as two back-to-back launches over disjoint column
                         ranges): algorithmic FLOPs per call / average duration of the call's launches, measured
                         with HIP events on the launch stream inside the timed region, against the bf16 dense
-                        MFMA peak
+                        MFMA peak; `power_limit_probe`: the same call on all-zero weights against real ones
   breakdown             per-stage device time from a separately instrumented pass (an event between stages,
                         which makes that pass a little longer than a timed step), and the MFMA fraction over
                         GEMM+attention time (the target the build is held to) = the GEMM+attention share of
@@ -92,6 +92,34 @@ class EventMarks:
             if self.only is None or name in self.only:
                 out[name].append(ev.elapsed_time(nxt))
         return out
+
+
+def power_limit_probe(torch, ops, model, L: int, launches: int = 200) -> dict:
+    """The dominant GEMM (gate|up of block 0, same shapes, epilogue and folded-norm form as in the model) launched
+    back to back on random activations, once with the block's weights and once with all-zero weights: instruction
+    stream, addresses and memory traffic are identical, only the switching activity of the multipliers differs.
+    The difference between the two is the part's power limit under MFMA load, not the kernel's schedule; the
+    zero-weight figure bounds what a better schedule could reach."""
+    pk = model._ensure_packed()
+    lin = pk["blocks"][0]["gu"]
+    dev = lin["w"].device
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((L, lin["w"].shape[1]), generator=g).to(device=dev, dtype=torch.bfloat16)
+    hmid = torch.empty((L, pk["Ip"]), dtype=torch.bfloat16, device=dev)
+    ss = ops.row_sumsq(x, out=torch.zeros((L, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev))
+    res = {}
+    for name, w in (("random", lin["w"]), ("zero_weights", torch.zeros_like(lin["w"]))):
+        call = lambda: ops.gemm(x, w, lin["b"], epilogue=ops.EPI_SWIGLU, out=hmid, a_row_sumsq=ss, norm_eps=model.norm_eps)
+        for _ in range(launches // 2):
+            call()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(launches):
+            call()
+        b.record()
+        torch.cuda.synchronize()
+        res[name] = a.elapsed_time(b) / launches
+    return res
 
 
 def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: list | None = None) -> dict:
@@ -326,7 +354,7 @@ def main() -> None:
     import numpy as np
     import torch
 
-    from cornserve_amd import lib, synth
+    from cornserve_amd import lib, ops, synth
     from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
 
     lib.load()
@@ -402,6 +430,7 @@ def main() -> None:
             model.forward_device(one_px, one_grid)
         torch.cuda.synchronize()
         one_ms = (time.perf_counter() - t0) / 10 * 1e3
+        probe = power_limit_probe(torch, ops, model, L) if model.fold_norm else None
     stage_ms = {k: sum(v) / 3 for k, v in full.durations_ms().items()}
     mfma_keys = [k for k in stage_ms if k.startswith("gemm_") or k.startswith("attn_") or k == "patch_embed"]
     # The instrumented pass records an event between stages, which costs a little device time per mark: its
@@ -445,6 +474,15 @@ def main() -> None:
             "mfma_frac_over_whole_step": flops["total"] / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         },
     }
+    if probe is not None:
+        result["roofline"]["power_limit_probe"] = {
+            "random_weights_ms": probe["random"], "zero_weights_ms": probe["zero_weights"],
+            "frac_random": flops["gemm_gate_up"] / (probe["random"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "frac_zero_weights": flops["gemm_gate_up"] / (probe["zero_weights"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "note": "the same gate|up call, 200 launches back to back outside the timed region, with the block's weights "
+                    "and with all-zero weights (identical instructions, addresses and traffic): the gap is the part's "
+                    "power limit under MFMA load; the zero-weight figure bounds what the schedule could reach",
+        }
     result["host_inputs"] = {
         "ms_per_step": host_ms, "patches_per_s": L / (host_ms * 1e-3),
         "note": "same batch handed over as pageable fp32 host tensors (PCIe copy + cast inside the call)",
