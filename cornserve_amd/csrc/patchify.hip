@@ -67,17 +67,15 @@ __global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict_
 // min(t*temporal + tt, T-1): an image is one frame repeated, a video's last frame is repeated to fill a group.
 // One workgroup writes QP_ROWS output rows (a row's place in the frame is worked out once and kept in LDS, as is
 // the table); a thread writes two neighbouring x at a time.
-// P and TPS are the patch size and the temporal patch size as constants (the column decomposition is then divisions
-// by constants), or 0 for any value.  This form serves the sizes the segment kernel below does not take.
+// This form takes any even patch size and any temporal size; the segment kernel below serves the usual ones.
 constexpr int QP_ROWS = 8;
-template <typename OUT, int P, int TPS>
+template <typename OUT>
 __global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __restrict__ frames, int T, int H, int W,
-                                                               int p_any, int m, int tps_any, const float* __restrict__ table,
+                                                               int p, int m, int tps, const float* __restrict__ table,
                                                                OUT* __restrict__ out, int64_t ldo, int rows) {
   __shared__ float lut[3 * 256];
   for (int i = threadIdx.x; i < 3 * 256; i += 256) lut[i] = table[i];
   __syncthreads();
-  const int p = P ? P : p_any, tps = TPS ? TPS : tps_any;
   const int hp = p >> 1;
   const int pairs = 3 * tps * p * hp;
   // where each of this workgroup's rows sits in the frame: (first frame of the group, top pixel row, left pixel column)
@@ -244,7 +242,7 @@ void launch_qwen_patchify_u8(int rows, hipStream_t stream, const uint8_t* frames
   else if (p == 16 && seg_lds <= 48 * 1024)
     hipLaunchKernelGGL((qwen_patchify_u8_seg_kernel<OUT, 16>), seg_grid, block, seg_lds, stream, frames, T, H, W, m, tps, table, out, ldo, rows);
   else
-    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT, 0, 0>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
+    hipLaunchKernelGGL((qwen_patchify_u8_kernel<OUT>), grid, block, 0, stream, frames, T, H, W, p, m, tps, table, out, ldo, rows);
 }
 
 }  // namespace
