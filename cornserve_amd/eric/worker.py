@@ -10,6 +10,10 @@ what the reference's sender needs to export them by IPC handle (sidecar/api.py:2
 CORNSERVE_MOCK_SIDECAR=1 and CORNSERVE_MOCK_SIDECAR_MAPPING='{"<id>-<chunk>": "<path>", ...}' every tensor is
 saved with torch.save to the mapped path (other values as JSON), so the encoders can be exercised by the
 reference's executor test harness without a running sidecar.
+
+`Worker.upload` is this build's addition on the inbound side: it starts the host-to-device copy of a batch's
+pixel tensors (floating point or uint8) on a side stream through pinned staging buffers, so that the copy of batch k+1 runs while the encoder works
+on batch k; `execute_model` then makes the compute stream wait for that copy only.
 """
 
 from __future__ import annotations
@@ -38,6 +42,7 @@ class WorkerBatch:
     receiver_ranks: list[list[list[int]] | None] = field(default_factory=list)
     data: dict[str, list[torch.Tensor]] = field(default_factory=dict)
     _dump_prefix: str | None = None
+    _uploaded: Any = None   # event recorded after the batch's host-to-device copies (set by Worker.upload)
 
     def __len__(self) -> int:
         return len(self.data_ids)
@@ -76,12 +81,50 @@ class Worker:
         if sender_sidecar_client is None and mock_sidecar_enabled():
             sender_sidecar_client = MockSidecar()
         self.sender_sidecar_client = sender_sidecar_client
+        self._copy_stream: torch.cuda.Stream | None = None
+
+    def upload(self, batch: WorkerBatch) -> WorkerBatch:
+        """Start copying the batch's host tensors to the model's device and return at once.  Every host tensor is
+        staged in pinned memory (a copy from pageable memory would block the host until it is done) and copied on
+        a side stream of default priority; an event recorded behind the copies travels with the batch, and
+        `execute_model` makes the compute stream wait for it.  Call it for batch k+1 before `execute_model(batch k)`
+        returns control to the device queue, and the copy overlaps the encoder's work.  Device tensors pass through."""
+        device = self.model.device
+        if device.type != "cuda":
+            raise RuntimeError("upload needs the model on a GPU")
+        if self._copy_stream is None:
+            self._copy_stream = torch.cuda.Stream(device=device)
+        staged: dict[str, list[torch.Tensor]] = {}
+        with torch.cuda.stream(self._copy_stream):
+            for key, tensors in batch.data.items():
+                out = []
+                for t in tensors:
+                    if (isinstance(t, torch.Tensor) and t.device.type == "cpu" and t.numel() > 0
+                            and (t.is_floating_point() or t.dtype == torch.uint8)):
+                        pinned = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+                        pinned.copy_(t)
+                        out.append(pinned.to(device, non_blocking=True))
+                    else:
+                        out.append(t)   # integer tensors (grids, crop counts) stay on the host, where they are read
+                staged[key] = out
+            done = torch.cuda.Event()
+            done.record(self._copy_stream)
+        batch.data = staged
+        batch._uploaded = done
+        return batch
 
     @torch.inference_mode()
     def execute_model(self, batch: WorkerBatch) -> list[torch.Tensor]:
         n = len(batch)
         if not (len(batch.chunk_ids) == len(batch.num_chunks) == len(batch.receiver_ranks) == n):
             raise ValueError("data_ids, chunk_ids, num_chunks and receiver_ranks must have one entry per item")
+        if batch._uploaded is not None:
+            compute = torch.cuda.current_stream(self.model.device)
+            compute.wait_event(batch._uploaded)
+            for tensors in batch.data.values():   # the copies were allocated on the side stream
+                for t in tensors:
+                    if isinstance(t, torch.Tensor) and t.is_cuda:
+                        t.record_stream(compute)
         output = self.model(modality=batch.modality, adapter_name=batch.adapter_name, batch=batch.data)
         if len(output) != n:
             raise RuntimeError(f"the model returned {len(output)} embeddings for {n} items")

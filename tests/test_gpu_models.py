@@ -245,6 +245,46 @@ def test_worker_hand_off_of_real_embeddings(dev, tmp_path):
         assert torch.equal(saved.to(dev), direct[i])
 
 
+def test_worker_upload_ahead(dev):
+    """Batches whose host tensors were sent ahead on the side stream give the same bits as batches handed over on
+    the host, for float pixel values, uint8 frames and a Gemma-3 batch (crop counts stay on the host), with the
+    upload of the next batch enqueued before the current one runs."""
+    from cornserve_amd.eric.worker import Worker, WorkerBatch
+
+    def wb(modality, data, n, adapter=""):
+        return WorkerBatch(modality=modality, adapter_name=adapter, request_ids=["r"] * n, data_ids=[f"d{i}" for i in range(n)],
+                           chunk_ids=[0] * n, num_chunks=[1] * n, receiver_ranks=[None] * n, data=data)
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=14)
+    worker = Worker(model)
+    batches = []
+    for s, grids in enumerate([[(1, 8, 12), (1, 16, 16)], [(1, 32, 32)], [(1, 4, 4), (1, 6, 10), (1, 2, 2)]]):
+        px, grid = synth.qwen_inputs(grids, seed=40 + s)
+        batches.append({"pixel_values": px, "image_grid_thw": grid})
+    frames = [torch.randint(0, 256, (1, 56, 84, 3), dtype=torch.uint8, generator=torch.Generator().manual_seed(3))]
+    direct = [model(Modality.IMAGE, "", b) for b in batches]
+    direct_frames = model(Modality.IMAGE, "", {"pixel_frames": frames})
+    pending = worker.upload(wb(Modality.IMAGE, dict(batches[0]), len(batches[0]["pixel_values"])))
+    for k in range(len(batches)):
+        nxt = None
+        if k + 1 < len(batches):
+            nxt = worker.upload(wb(Modality.IMAGE, dict(batches[k + 1]), len(batches[k + 1]["pixel_values"])))
+        assert all(t.is_cuda for t in pending.data["pixel_values"]) and not pending.data["image_grid_thw"][0].is_cuda
+        out = worker.execute_model(pending)
+        assert all(torch.equal(o, d) for o, d in zip(out, direct[k]))
+        pending = nxt
+    out = worker.execute_model(worker.upload(wb(Modality.IMAGE, {"pixel_frames": frames}, 1)))
+    assert torch.equal(out[0], direct_frames[0])
+
+    gmodel, _, _ = build_gemma(dev, 2, 224, 640, 16, seed=2)
+    px, crops = synth.gemma3_inputs(2, 224, seed=2)
+    ref = gmodel(Modality.IMAGE, "a", {"pixel_values": px, "num_crops": crops})
+    gb = Worker(gmodel).upload(wb(Modality.IMAGE, {"pixel_values": px, "num_crops": crops}, 2, adapter="a"))
+    assert not gb.data["num_crops"][0].is_cuda
+    out = Worker(gmodel).execute_model(gb)
+    assert all(torch.equal(o, r) for o, r in zip(out, ref))
+
+
 def test_scheduler_worker_loop_with_patch_budget(dev, tmp_path):
     """Requests queued in the scheduler, batched under a patch budget, run by the worker and handed to the mock
     sidecar: every item's embedding equals the one from a single direct call (an item does not depend on its batch)."""
