@@ -369,7 +369,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 mark("gemm_qkv")
                 self._g(n, b["qkv"], out=qkv)
             mark("attn_full" if full else "attn_window")
-            ops.attn_varlen(qkv[:, :H], qkv[:, H : 2 * H], qkv[:, 2 * H :], plan, nh, d, scale, cos_sin=ix.cos_sin, out=att)
+            ops.attn_varlen_rotary_(qkv, plan, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")
             if fold:
                 self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss)

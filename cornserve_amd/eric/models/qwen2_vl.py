@@ -177,7 +177,7 @@ class Qwen2VisionTransformer(QwenVisionBase):
                 mark("gemm_qkv")
                 self._g(n, b["qkv"], out=qkv)
             mark("attn_full")
-            ops.attn_varlen(qkv[:, :E], qkv[:, E : 2 * E], qkv[:, 2 * E :], plan, nh, d, scale, cos_sin=ix.cos_sin, out=att)
+            ops.attn_varlen_rotary_(qkv, plan, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")
             self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **(stats_out if fold else {}))
             if fold:

@@ -445,6 +445,21 @@ def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPla
     return out
 
 
+def attn_varlen_rotary_(qkv: torch.Tensor, plan: AttnPlan, heads: int, head_dim: int, scale: float,
+                        cos_sin: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """Rotary + attention over a packed [L, 3*heads*head_dim] buffer whose q and k the caller no longer needs.
+    Segments of at most 64 rows (window attention) take the kernel that rotates while it stages q and k; longer
+    segments rotate q and k in place once (every query block of a segment would otherwise rotate the segment's keys
+    again) and take the kernel that streams K/V tiles straight into LDS.  Both routes give the same bits."""
+    E = heads * head_dim
+    q, k, v = qkv[:, :E], qkv[:, E : 2 * E], qkv[:, 2 * E :]
+    if plan.max_seqlen <= 64:
+        return attn_varlen(q, k, v, plan, heads, head_dim, scale, cos_sin=cos_sin, out=out)
+    rope_qk_(qkv, cos_sin, heads, head_dim)
+    return attn_varlen(q, k, v, plan, heads, head_dim, scale, out=out)
+
+
+
 # ------------------------------------------------------------------------------------------ SigLIP
 def qwen_patchify_u8(frames: torch.Tensor, table: torch.Tensor, patch: int, merge: int, temporal: int, *,
                      out: torch.Tensor | None = None, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:

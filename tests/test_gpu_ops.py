@@ -121,6 +121,30 @@ def test_qwen_patchify_u8_bit_exact(ops, dev, t, h, w, patch, merge, temporal):
         ops.qwen_patchify_u8(torch.zeros((1, 30, 28, 3), dtype=torch.uint8, device=dev), table.to(dev), 14, 2, 2)
 
 
+@pytest.mark.parametrize("heads,d", [(16, 80), (4, 64), (2, 96)])
+def test_attn_rotary_in_place_route_equals_fused_route(ops, dev, heads, d):
+    """Long segments: rotating q and k in place and running the kernel without rotary gives the bits of the kernel
+    that rotates while staging (ragged segment lengths either side of the tile sizes)."""
+    lens = [100, 1024, 65, 300, 128, 1, 777]
+    cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
+    L, E = int(cu[-1]), heads * d
+    g = torch.Generator().manual_seed(heads * 100 + d)
+    qkv = torch.randn((L, 3 * E), generator=g).bfloat16().to(dev)
+    ang = torch.rand((L, d // 2), generator=g) * 6.2831853
+    cs = torch.cat([ang.cos(), ang.sin()], dim=1).float().to(dev).contiguous()
+    plan = ops.attn_plan(cu, dev)
+    fused = ops.attn_varlen(qkv[:, :E], qkv[:, E:2 * E], qkv[:, 2 * E:], plan, heads, d, d ** -0.5, cos_sin=cs)
+    buf = qkv.clone()
+    got = ops.attn_varlen_rotary_(buf, plan, heads, d, d ** -0.5, cs)
+    assert torch.equal(got, fused)
+    assert not torch.equal(buf[:, :E], qkv[:, :E]) and torch.equal(buf[:, 2 * E:], qkv[:, 2 * E:])   # q, k rotated; v untouched
+    short = ops.attn_plan(np.arange(0, 64 * 5 + 1, 64, dtype=np.int32), dev)   # window route: the buffer stays as it is
+    buf = qkv[:320].clone()
+    got = ops.attn_varlen_rotary_(buf, short, heads, d, d ** -0.5, cs[:320].contiguous())
+    ref = ops.attn_varlen(qkv[:320, :E], qkv[:320, E:2 * E], qkv[:320, 2 * E:], short, heads, d, d ** -0.5, cos_sin=cs[:320].contiguous())
+    assert torch.equal(got, ref) and torch.equal(buf, qkv[:320])
+
+
 @pytest.mark.parametrize("patch", [14, 16])
 def test_qwen_patchify_u8_unaligned_frames(ops, dev, patch):
     """Frames that start at any byte offset of a 4-byte word (a view into a larger buffer), last frame at the very end
