@@ -104,7 +104,7 @@ def _check_no_missing_kernels(lib: Path) -> None:
         raise RuntimeError(f"{lib.name} has undefined symbols of its own (dropped kernels?):\n  " + "\n  ".join(own))
 
 
-def build_library(force: bool = True, jobs: int = 6) -> Path:
+def build_library(force: bool = True, jobs: int = 8) -> Path:
     """Compile every .hip source under csrc/ and link the shared library. Returns its path."""
     hipcc = _hipcc()
     OBJ_DIR.mkdir(exist_ok=True)

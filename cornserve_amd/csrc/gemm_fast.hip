@@ -1,734 +1,19 @@
-// Fast-path bf16 MFMA GEMM for gfx950:  C[M,N] = epilogue(A[M,K] . W[N,K]^T),  K % 64 == 0, bf16 weights.
-//
-// Shape of a workgroup.  FOUR waves, one per SIMD, each with all 512 registers of a lane: the 256
-// accumulation registers hold the wave's accumulators (up to 128x128 outputs), the architectural registers
-// hold two sets of operand fragments and the addresses.  The accumulators are driven by inline assembly in a
-// fixed instruction order: the compiler never sees them, so it cannot copy, rotate or spill them, and the LDS
-// reads and direct loads sit at chosen places between the MFMAs.  One workgroup per CU (LDS-bound), the
-// kernel is persistent over output tiles.
-//
-// Pipeline.  K is walked in steps of 64.  Tiles go global -> LDS directly (buffer_load_dwordx4 ... lds: each
-// lane fetches 16 bytes and the hardware stores the wave's 64 chunks contiguously at M0 + lane*16).  The loop
-// is skewed: the single barrier of an iteration sits BEFORE its last k-step, so the first fragments of the
-// next K tile are read while the matrix cores work on that last step.  The four waves share the CU's one
-// memory pipeline, and a K tile costs it about half an iteration, so the direct loads must not come in
-// bursts: LDS is organised as a RING with more than two K tiles of room, which lets the loads of a K tile be
-// issued in two different half-iterations, evenly spaced between the MFMAs, and gives them a whole
-// iteration more to land (the weights of an encoder block come from HBM, not from a cache):
-//   * 256x256 tile: five 32 KB units = A(kt), W(kt), A(kt+1), W(kt+1) and one in flight.  A(kt+2) is
-//     requested in the first half of iteration kt, W(kt+2) in the second half, into the unit that the
-//     barrier has just freed.
-//   * narrower tiles (256x160, 128x160, 256x128, 128x192): three whole stages.  The second half of K tile kt+2 is
-//     requested in the first half of iteration kt, the first half of K tile kt+3 in the second half.
-// The sequence of K tiles runs on across output tiles: the next output tile's first K tiles are requested
-// in the last iterations of the current one and travel while the epilogue runs.  Waits use the in-order
-// completion of loads: "K tile j has landed" == "at most the loads issued after it are outstanding".
-//
-// Matrix cores.  v_mfma_f32_16x16x32_bf16 (k = 32 per instruction: each accumulator register is touched
-// half as often as with the 32x32x16 form).  W rows are the MFMA "A" operand and activation rows the "B"
-// operand, so a lane owns output row m = lane%16 of a 16x16 block.  The W rows that feed the fragments of a
-// wave are PERMUTED in groups of G fragments (G = 2 when the wave has an even number of them): fragment j,
-// fragment row 4q+r holds W row (j/G)*16G + q*4G + (j%G)*4 + r of the wave's rows.  The 4G accumulator
-// values a lane holds for one output row and group are then CONSECUTIVE in n, and the four lanes of that
-// output row hold 16G consecutive columns: with G = 2 every store instruction writes 16 bytes per lane and
-// 64 contiguous bytes per output row, with no trip through LDS.
-//
-// LDS layout.  A tile row is 128 bytes = 8 chunks of 16 bytes; logical chunk c of row r lives in slot
-// c ^ key(r).  The LDS has 64 four-byte banks, so a 16-byte-per-lane read is served 16 lanes at a time and
-// is conflict-free when those lanes hit 16 distinct 16-byte groups of a 256-byte span; with 128-byte rows
-// the row parity picks the half and the key must differ across the 8 rows of equal parity.  Activation
-// fragments read 16 consecutive rows (key = (r>>1)&7); W fragments read rows q*4G + r plus a multiple of 4
-// (key = q*2 + ((r>>1)&1)).  Since a direct-to-LDS load fixes the LDS side (lane -> consecutive chunk),
-// the swizzle is applied on the GLOBAL side: the lane that lands in slot s of row r fetches chunk s ^ key(r).
+// Fast-path bf16 MFMA GEMM for gfx950: choice of the tile form.  The kernel itself is in gemm_fast_impl.h; each tile
+// form is built in its own translation unit (gemm_fast_t*.hip).
 #include <stdlib.h>
-
-#include <type_traits>
-#include <utility>
 
 #include "gemm_common.h"
 
+// Epilogue / folded-norm dispatch of one tile form each (gemm_fast_t<rows>x<cols>.hip).
+int cs_gemm_fast_tile_256x256(const CsGemmArgs& a, hipStream_t stream);
+int cs_gemm_fast_tile_256x160(const CsGemmArgs& a, hipStream_t stream);
+int cs_gemm_fast_tile_128x160(const CsGemmArgs& a, hipStream_t stream);
+int cs_gemm_fast_tile_128x192(const CsGemmArgs& a, hipStream_t stream);
+int cs_gemm_fast_tile_256x128(const CsGemmArgs& a, hipStream_t stream);
+
 namespace {
 
-using namespace csgemm;
-
-constexpr int CS_EPI_BIAS_POS = 100;  // internal: CS_EPI_BIAS plus the (row % pos_period) position addend
-constexpr int NW = 4;                 // waves per workgroup, one per SIMD
-constexpr int LDS_BYTES = 160 * 1024;
-
-// s_waitcnt encodings (gfx9): vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8.
-constexpr int waitcnt_vm(int n) { return ((n & 0xF) | ((n >> 4) << 14)) | 0x0F70; }       // vmcnt(n) only
-constexpr int waitcnt_vm_lgkm0(int n) { return ((n & 0xF) | ((n >> 4) << 14)) | 0x0070; }  // vmcnt(n) lgkmcnt(0)
-constexpr int WAITCNT_LGKM0 = 0xC07F;                                                      // lgkmcnt(0) only
-
-typedef __attribute__((address_space(3))) void lds_void_t;
-
-// Workgroup barrier without the full memory fence of __syncthreads(): the callers order LDS traffic with
-// explicit waits, and the asm statements keep the compiler from moving memory operations across it.
-CS_DEVICE void wg_barrier() {
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-}
-
-#ifdef CS_GEMM_TS
-__device__ long long* cs_ts_buf;  // [tiles][8]: 4 wall-clock stamps + 4 shader-clock stamps by wave 0 (profiling builds only)
-#define CS_TS(slot) do { if (tid == 0 && cs_ts_buf) { cs_ts_buf[vb * 8 + (slot)] = wall_clock64(); cs_ts_buf[vb * 8 + 4 + (slot)] = clock64(); } } while (0)
-#else
-#define CS_TS(slot) do { } while (0)
-#endif
-
-// every accumulation register, as an inline-asm clobber list
-#define CS_ALL_ACC_REGS \
-  "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", \
-  "a16", "a17", "a18", "a19", "a20", "a21", "a22", "a23", "a24", "a25", "a26", "a27", "a28", "a29", "a30", "a31", \
-  "a32", "a33", "a34", "a35", "a36", "a37", "a38", "a39", "a40", "a41", "a42", "a43", "a44", "a45", "a46", "a47", \
-  "a48", "a49", "a50", "a51", "a52", "a53", "a54", "a55", "a56", "a57", "a58", "a59", "a60", "a61", "a62", "a63", \
-  "a64", "a65", "a66", "a67", "a68", "a69", "a70", "a71", "a72", "a73", "a74", "a75", "a76", "a77", "a78", "a79", \
-  "a80", "a81", "a82", "a83", "a84", "a85", "a86", "a87", "a88", "a89", "a90", "a91", "a92", "a93", "a94", "a95", \
-  "a96", "a97", "a98", "a99", "a100", "a101", "a102", "a103", "a104", "a105", "a106", "a107", "a108", "a109", "a110", "a111", \
-  "a112", "a113", "a114", "a115", "a116", "a117", "a118", "a119", "a120", "a121", "a122", "a123", "a124", "a125", "a126", "a127", \
-  "a128", "a129", "a130", "a131", "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", \
-  "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159", \
-  "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173", "a174", "a175", \
-  "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", \
-  "a192", "a193", "a194", "a195", "a196", "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", \
-  "a208", "a209", "a210", "a211", "a212", "a213", "a214", "a215", "a216", "a217", "a218", "a219", "a220", "a221", "a222", "a223", \
-  "a224", "a225", "a226", "a227", "a228", "a229", "a230", "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", \
-  "a240", "a241", "a242", "a243", "a244", "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255"
-
-template <int V>
-using ic = std::integral_constant<int, V>;
-template <class F, int... Is>
-CS_DEVICE void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
-  (f(ic<Is>{}), ...);
-}
-// f(ic<0>{}), f(ic<1>{}), ... f(ic<N-1>{}): a loop whose index is a constant expression in the body
-template <int N, class F>
-CS_DEVICE void static_for(F&& f) {
-  static_for_impl(f, std::make_integer_sequence<int, N>{});
-}
-
-// LDS organisation of a tile shape (shared by the kernel and its launcher).
-template <int BM, int BN, bool W_FP8>
-struct RingShape {
-  static constexpr int A_BYTES = BM * BK * 2, W_BYTES = BN * BK * (W_FP8 ? 1 : 2);
-  static constexpr bool FIVE_UNITS = A_BYTES == W_BYTES && 5 * A_BYTES <= LDS_BYTES && 3 * (A_BYTES + W_BYTES) > LDS_BYTES;
-  static constexpr int BYTES = FIVE_UNITS ? 5 * A_BYTES : 3 * (A_BYTES + W_BYTES);
-  static_assert(BYTES <= LDS_BYTES, "tile does not fit a ring");
-};
-
-// W_FP8: the weights are e4m3 bytes with a per-output-channel fp32 scale.  W tiles travel and sit in LDS as bytes
-// (half the traffic); a fragment is converted to bf16 in registers right before its MFMAs (exact: every e4m3
-// value is a bf16 value) and the scale is applied to the fp32 accumulators in the epilogue.
-//
-// FUSE: 0 = plain; FUSE_NORM_A = the rows of A stand for their RMS-normalised form: the accumulators are multiplied
-// by rsqrt(sum of squares of the A row / K + eps) before the bias (the norm's weight is folded into W by the
-// caller); FUSE_SUMSQ_C = besides C, the sum of squares of every output row over this tile's columns goes to
-// c_row_sumsq (what the next FUSE_NORM_A launch reads).
-// FUSE_LN_A / FUSE_STATS_C: the same for LayerNorm -- the producer also emits the row sums, the consumer computes
-// rstd * (acc - mean * w_col_sum[n]) + bias[n] with mean and rstd from the two sets of parts (the norm's weight is
-// folded into W, its bias into the GEMM bias, and w_col_sum[n] = sum_k W'[n,k] carries the mean term).
-constexpr int FUSE_NORM_A = 1, FUSE_SUMSQ_C = 2, FUSE_LN_A = 3, FUSE_STATS_C = 4;
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE>
-__global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) {
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-  static_assert(WAVES_M * WAVES_N == NW, "four waves, one per SIMD");
-  using Ring = RingShape<BM, BN, W_FP8>;
-  constexpr int A_BYTES = Ring::A_BYTES, W_BYTES = Ring::W_BYTES;
-  constexpr bool RING5 = Ring::FIVE_UNITS;
-  // Byte offsets of operand tile slots.  Three-stage ring: slot s holds A at s*STAGE and W behind it.
-  // Five-unit ring: every unit is one operand tile.
-  constexpr int STAGE = A_BYTES + W_BYTES;
-  constexpr int WTM = BM / WAVES_M, WTN = BN / WAVES_N;
-  static_assert(WTM % 16 == 0 && WTN % 16 == 0 && BM % 8 == 0 && BN % 8 == 0, "tile shape");
-  constexpr int MT = WTM / 16, NT = WTN / 16;
-  static_assert(MT * NT * 4 <= 256, "the accumulators of a wave live in its 256 accumulation registers");
-  // W fragments come in groups of G: fragment j, fragment row 4q+r holds W row (j/G)*16G + q*4G + (j%G)*4 + r of
-  // the wave's rows, so a lane owns 4G consecutive output columns per group and the four lanes q = 0..3 of
-  // one output row own 16G consecutive columns.
-  constexpr int G = (NT % 2 == 0) ? 2 : NT;
-  auto piece_col = [](int j) { return (j / G) * 16 * G + (j % G) * 4; };  // first column of fragment j's piece
-  constexpr int W_ROW = W_FP8 ? BK : BK * 2;     // bytes per W tile row
-  constexpr int W_ROWS_LD = 1024 / W_ROW;         // W rows per direct load (one load moves 64 x 16 bytes)
-  static_assert(BN % W_ROWS_LD == 0, "tile shape");
-  constexpr int A_BLK = BM / 8, W_BLK = BN / W_ROWS_LD;  // row blocks = direct loads per operand tile
-  static_assert(A_BLK % NW == 0, "every wave issues the same number of direct loads");
-  // When W_BLK is not a multiple of the wave count, the waves that have no block left repeat the last one
-  // (the same bytes to the same place): every wave must issue the same number of loads, because the waits
-  // count loads.
-  constexpr int A_LD = A_BLK / NW, W_LD = (W_BLK + NW - 1) / NW;  // per wave
-  constexpr int NLD = A_LD + W_LD;                      // direct loads per wave and K tile
-  constexpr int NFR = MT + NT;                          // fragment reads per wave and k-step
-  constexpr int NMFMA = MT * NT;                        // MFMAs per wave and k-step
-  // Fragment reads of the second k-step go after every other MFMA where there are enough of them, else after each.
-  constexpr int READ_STRIDE = (2 * NFR <= NMFMA) ? 2 : 1;
-  static_assert(READ_STRIDE * NFR <= NMFMA, "one slot after an MFMA per LDS read");
-
-  // ---- tile coordinates of virtual block vb in [0, tiles): XCD-aware remap (workgroup i runs on XCD i%8,
-  //      and the persistent stride gridDim.x is a multiple of 8, so a workgroup's tiles stay on its XCD),
-  //      then bands of 8 tile-rows walked column-major so the 32 workgroups resident on one XCD share
-  //      8 A panels and 4 W panels through that XCD's L2.
-  const int ntiles = p.tiles_m * p.tiles_n;
-  auto tile_origin = [&](int vb, int& m0, int& n0) {
-    const int per = ntiles >> 3;
-    if (vb < per * 8) vb = (vb & 7) * per + (vb >> 3);
-    constexpr int GM = 8;
-    const int band_sz = GM * p.tiles_n;
-    const int band = vb / band_sz;
-    const int within = vb - band * band_sz;
-    const int rows_in_band = min(GM, p.tiles_m - band * GM);
-    m0 = (band * GM + within % rows_in_band) * BM;
-    n0 = (within / rows_in_band) * BN;
-  };
-
-  // The accumulation registers a[0:255] belong to the inline assembly below (MFMAs in the main loop,
-  // v_accvgpr_read in the epilogue), accumulator (i, j) in a[4(i*NT+j) .. +3].  The compiler is told once
-  // that they are in use, so that the kernel's register allocation covers them; it has no reason to touch
-  // them itself as long as the rest of the kernel fits the 256 architectural registers, and the build
-  // checks the generated code for exactly that.
-  asm volatile("" ::: CS_ALL_ACC_REGS);
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int wm = wave % WAVES_M, wn = wave / WAVES_M;
-
-  // ---- global sources of the direct loads.  Row block rb = j*NW + wave covers tile rows 8rb..8rb+7; the
-  //      lane lands in slot lane%8 of row 8rb + lane/8 and fetches chunk (lane%8) ^ key(row).  Buffer
-  //      loads: a 32-bit per-lane byte offset plus a scalar K offset on a scalar descriptor, so an address
-  //      costs one register and no vector arithmetic.
-  const int l_row = lane >> 3, l_slot = lane & 7;
-  uint32_t a_src[A_LD];
-  uint32_t w_src[W_LD];
-  auto setup_sources = [&](int m0, int n0) {
-#pragma unroll
-    for (int j = 0; j < A_LD; ++j) {
-      const int row = (j * NW + wave) * 8 + l_row;  // tile-local
-      const int key = (row >> 1) & 7;
-      const int r = min(m0 + row, p.M - 1);
-      a_src[j] = (uint32_t)(((int64_t)r * p.lda + ((l_slot ^ key) << 3)) * 2);
-    }
-#pragma unroll
-    for (int j = 0; j < W_LD; ++j) {
-      const int blk = min(j * NW + wave, W_BLK - 1);
-      if constexpr (W_FP8) {  // 64-byte rows: the lane lands in slot lane%4 of row 16 blk + lane/4
-        const int row = blk * 16 + (lane >> 2);
-        const int key = ((row % (16 * G)) / (4 * G)) & 3;
-        const int r = min(n0 + row, p.N - 1);
-        w_src[j] = (uint32_t)((int64_t)r * p.ldw + (((lane & 3) ^ key) << 4));
-      } else {
-        const int row = blk * 8 + l_row;
-        const int key = ((((row % (16 * G)) / (4 * G)) & 3) << 1) | ((row >> 1) & 1);
-        const int r = min(n0 + row, p.N - 1);
-        w_src[j] = (uint32_t)(((int64_t)r * p.ldw + ((l_slot ^ key) << 3)) * 2);
-      }
-    }
-  };
-  const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, -1, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void*)p.W, 0, -1, 0x00020000);
-  // (The builtin is called from non-generic lambdas on purpose: inside a generic lambda the host pass of the
-  // compiler rejects the device-only builtin, silently drops the kernel and leaves its launch stub undefined.)
-  auto load_a = [&](int kt, char* lds_dst, uint32_t off) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_void_t*)lds_dst, 16, off, kt * (BK * 2), 0, 0);
-  };
-  auto load_w = [&](int kt, char* lds_dst, uint32_t off) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_w, (lds_void_t*)lds_dst, 16, off, kt * W_ROW, 0, 0);
-  };
-  // Direct load number IDX (A row blocks first, then W row blocks) of K tile kt; a_base / w_base are the
-  // LDS byte offsets of the operand tiles it goes to.
-  auto direct_load = [&](int kt, int a_base, int w_base, auto idx_c) {
-    constexpr int IDX = decltype(idx_c)::value;
-    if constexpr (IDX < A_LD) {
-      load_a(kt, smem + a_base + (IDX * NW + wave) * 1024, a_src[IDX]);
-    } else {
-      constexpr int J = IDX - A_LD;
-      load_w(kt, smem + w_base + min(J * NW + wave, W_BLK - 1) * 1024, w_src[J]);
-    }
-  };
-
-  // ---- fragment addressing.  Lane (a = lane%16, kq = lane/16) reads chunk ks*4 + kq of its fragment row.
-  //      Both keys depend only on the lane, so the per-lane part of the address is loop-invariant.
-  const int fa = lane & 15, kq = lane >> 4;
-  const int fq = fa >> 2, fr = fa & 3;
-  const int x_key = (fa >> 1) & 7;
-  const int w_key = (fq << 1) | ((fr >> 1) & 1);
-  // byte offset inside an operand tile of fragment (i or j), k-step ks: row*128 + (((ks*4 + kq) ^ key) << 4)
-  int x_off[2], w_off[2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    x_off[ks] = (wm * WTM + fa) * 128 + (((ks * 4 + kq) ^ x_key) << 4);
-    if constexpr (W_FP8)  // 8 bytes: half (kq%2) of chunk 2ks + kq/2, which sits in slot chunk ^ q
-      w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 2 + (kq >> 1)) ^ fq) << 4) + (kq & 1) * 8;
-    else
-      w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 4 + kq) ^ w_key) << 4);
-  }
-  // Operand fragments: two sets.  fp8 weights are read as 8 raw bytes per fragment and converted into one of
-  // two bf16 registers sets right before use.
-  bf16x8_t wf[2][W_FP8 ? 1 : NT], xf[2][MT];
-  i32x2_t wraw[2][W_FP8 ? NT : 1];
-  bf16x8_t wcv[2];
-  // Fragment read number IDX of k-step ks into set b.  bf16 weights: W fragments first (MFMAs run i-major and
-  // need every W fragment at once); fp8 weights: activation fragments first (MFMAs run j-major).
-  auto read_frag = [&](int a_base, int w_base, int ks, int b, auto idx_c) {
-    constexpr int IDX = decltype(idx_c)::value;
-    if constexpr (W_FP8) {
-      if constexpr (IDX < MT) xf[b][IDX] = *(const bf16x8_t*)(smem + a_base + x_off[ks] + IDX * 16 * 128);
-      else wraw[b][IDX - MT] = *(const i32x2_t*)(smem + w_base + w_off[ks] + piece_col(IDX - MT) * W_ROW);
-    } else {
-      if constexpr (IDX < NT) wf[b][IDX] = *(const bf16x8_t*)(smem + w_base + w_off[ks] + piece_col(IDX) * W_ROW);
-      else xf[b][IDX - NT] = *(const bf16x8_t*)(smem + a_base + x_off[ks] + (IDX - NT) * 16 * 128);
-    }
-  };
-  auto convert_w = [&](int b, auto j_c) {  // 8 e4m3 bytes -> 8 bf16 (exact)
-    constexpr int J = decltype(j_c)::value;
-    bf16x8_t o;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const auto p0 = __builtin_amdgcn_cvt_pk_f32_fp8(wraw[b][W_FP8 ? J : 0][h], false);
-      const auto p1 = __builtin_amdgcn_cvt_pk_f32_fp8(wraw[b][W_FP8 ? J : 0][h], true);
-      o[4 * h + 0] = (bf16_t)p0[0];
-      o[4 * h + 1] = (bf16_t)p0[1];
-      o[4 * h + 2] = (bf16_t)p1[0];
-      o[4 * h + 3] = (bf16_t)p1[1];
-    }
-    wcv[J & 1] = o;
-  };
-  // The MFMAs of one k-step on fragment set B, in program order (asm volatile statements keep it), with a
-  // hook call after each: that is where LDS reads and direct loads are placed.  ZERO: the first k-step of an
-  // output tile takes a zero addend, which saves clearing the accumulators.
-  auto mfmas = [&](auto b_c, auto zero_c, auto&& hook) {
-    constexpr int B = decltype(b_c)::value;
-    constexpr bool ZERO = decltype(zero_c)::value;
-    if constexpr (W_FP8) convert_w(B, ic<0>{});
-    static_for<NMFMA>([&](auto n) {
-      constexpr int N = decltype(n)::value;
-      // bf16 weights: i-major; fp8 weights: j-major, the next W fragment is converted while this one is used
-      constexpr int I = W_FP8 ? N % MT : N / NT, J = W_FP8 ? N / MT : N % NT, R = (I * NT + J) * 4;
-      const bf16x8_t& w = W_FP8 ? wcv[J & 1] : wf[B][W_FP8 ? 0 : J];
-      // A register written by a vector instruction must not be read by an MFMA in the next few cycles; the
-      // compiler pads that for its own MFMAs but cannot see into these.  Only the first MFMA after a
-      // conversion can be that close.
-      if constexpr (W_FP8 && I == 0) asm volatile("s_nop 3");
-      if constexpr (ZERO)
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
-      else
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
-      if constexpr (W_FP8 && I == 0 && J + 1 < NT) convert_w(B, ic<J + 1>{});
-      hook(n);
-    });
-  };
-
-  // ---- ring state.  `ring` is the slot of the current K tile: a stage number (three-stage ring) or the
-  //      unit of A(kt) with W(kt), A(kt+1), W(kt+1), A(kt+2) following cyclically (five-unit ring).  It
-  //      keeps rotating across output tiles.
-  constexpr int RING_N = RING5 ? 5 : 3;
-  auto slot_add = [](int s, int d) { return (s + d) % RING_N; };
-  auto a_base_of = [&](int tile_ahead, int ring) {  // LDS offset of the A tile of K tile kt + tile_ahead
-    return RING5 ? slot_add(ring, 2 * tile_ahead) * A_BYTES : slot_add(ring, tile_ahead) * STAGE;
-  };
-  auto w_base_of = [&](int tile_ahead, int ring) {
-    return RING5 ? slot_add(ring, 2 * tile_ahead + 1) * A_BYTES : slot_add(ring, tile_ahead) * STAGE + A_BYTES;
-  };
-  // Loads of a K tile are issued in two portions; PA of them in the first half of an iteration.
-  // Five-unit ring: A(kt+2) in the first half, W(kt+2) in the second (same K tile, AHEAD_B == AHEAD_A).
-  // Three-stage ring: the second portion of K tile kt+2 in the first half, the first portion of K tile kt+3
-  // in the second half.
-  constexpr int PA = RING5 ? A_LD : NLD - NLD / 2;  // loads issued in a first half
-  constexpr int PB = NLD - PA;                       // loads issued in a second half
-  constexpr int PA_FIRST = RING5 ? 0 : PB;           // index of the first load of the first-half portion
-  constexpr int PB_FIRST = RING5 ? A_LD : 0;
-  constexpr int AHEAD_A = 2, AHEAD_B = RING5 ? 2 : 3;
-  constexpr int EA = NMFMA / PA, EB = NMFMA / PB;    // MFMAs per direct load in each half
-  static_assert(EA >= 1 && EB >= 1, "one slot after an MFMA per direct load");
-  // Loads outstanding by design at the two wait points: everything issued after the K tile that is needed.
-  constexpr int PENDING_AT_BARRIER = RING5 ? PA : NLD;           // after K tile kt+1
-  constexpr int PENDING_AT_TILE_START = RING5 ? NLD : NLD + PB;  // after K tile 0 of an output tile
-
-  const int nk = p.K / BK;  // >= 3 (checked on the host)
-  int vb = blockIdx.x;
-  int m0, n0;
-  tile_origin(vb, m0, n0);
-  setup_sources(m0, n0);
-  int ring = 0;
-  // in flight before the first iteration: K tiles 0 and 1, and what a second half would have requested
-  static_for<NLD>([&](auto n) { direct_load(0, a_base_of(0, ring), w_base_of(0, ring), n); });
-  static_for<NLD>([&](auto n) { direct_load(1, a_base_of(1, ring), w_base_of(1, ring), n); });
-  if constexpr (!RING5)
-    static_for<PB>([&](auto n) { direct_load(2, a_base_of(2, ring), w_base_of(2, ring), ic<PB_FIRST + decltype(n)::value>{}); });
-
-  for (;;) {  // persistent loop over this workgroup's output tiles (vb, vb + gridDim.x, ...)
-    const int vb_next = vb + gridDim.x;
-    const bool has_next = vb_next < ntiles;
-    int m0_next = 0, n0_next = 0;
-
-    CS_TS(0);
-    // K tile 0 has landed once at most the loads issued after it are outstanding.  (Loads complete in
-    // order; stores of the previous epilogue that are still in flight only make this wait longer.)
-    __builtin_amdgcn_s_waitcnt(waitcnt_vm(PENDING_AT_TILE_START));
-    wg_barrier();
-    CS_TS(1);
-    static_for<NFR>([&](auto n) { read_frag(a_base_of(0, ring), w_base_of(0, ring), 0, 0, n); });
-
-    // One K iteration.  TAIL 0: steady state.  TAIL t > 0: t iterations before the end of the output tile,
-    // where the K tiles being requested belong to the next output tile (if there is one).
-    auto iteration = [&](int kt, auto first_c, auto tail_c) {
-      constexpr bool FIRST = decltype(first_c)::value;
-      constexpr int TAIL = decltype(tail_c)::value;
-      // Does the portion requested in each half belong to this output tile?  K tile kt + AHEAD exists iff
-      // AHEAD < TAIL (or TAIL == 0).
-      constexpr bool CUR_A = TAIL == 0 || AHEAD_A < TAIL, CUR_B = TAIL == 0 || AHEAD_B < TAIL;
-      const int k_a = CUR_A ? kt + AHEAD_A : AHEAD_A - TAIL;  // K tile number inside its output tile
-      const int k_b = CUR_B ? kt + AHEAD_B : AHEAD_B - TAIL;
-      // The sources switch to the next output tile once, right before its first load is issued: that is the
-      // second-half portion when it runs further ahead than the first-half portion, else the first-half one.
-      constexpr bool SWITCH_BEFORE_B = AHEAD_B > AHEAD_A && TAIL == AHEAD_B;
-      constexpr bool SWITCH_BEFORE_A = AHEAD_B == AHEAD_A && TAIL == AHEAD_A;
-      auto switch_sources = [&]() {
-        if (has_next) {
-          tile_origin(vb_next, m0_next, n0_next);
-          setup_sources(m0_next, n0_next);
-        }
-      };
-      if constexpr (SWITCH_BEFORE_A) switch_sources();
-      __builtin_amdgcn_sched_barrier(0);
-      // first k-step; meanwhile the fragments of the second k-step and the first-half portion of loads
-      mfmas(ic<0>{}, std::bool_constant<FIRST>{}, [&](auto n) {
-        constexpr int N = decltype(n)::value;
-        if constexpr (N < NFR) read_frag(a_base_of(0, ring), w_base_of(0, ring), 1, 1, n);
-        if constexpr (N < EA * PA && N % EA == EA - 1) {
-          auto ld = [&]() { direct_load(k_a, a_base_of(AHEAD_A, ring), w_base_of(AHEAD_A, ring), ic<PA_FIRST + N / EA>{}); };
-          if constexpr (CUR_A) ld();
-          else if (has_next) ld();
-        }
-      });
-      // K tile kt+1 has landed in this wave's part of LDS once at most the loads issued after it are
-      // outstanding, and this wave has received its last fragments of K tile kt.
-      if constexpr (TAIL == 1) {
-        __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);  // nothing more is read from LDS for this output tile
-      } else if (!CUR_A && !has_next) {
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));  // nothing was requested after K tile kt+1
-      } else {
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(PENDING_AT_BARRIER));
-      }
-      wg_barrier();
-      if constexpr (SWITCH_BEFORE_B) switch_sources();
-      // second k-step; meanwhile the first fragments of K tile kt+1 and the second-half portion of loads,
-      // which goes to LDS space that the barrier has just freed
-      mfmas(ic<1>{}, std::false_type{}, [&](auto n) {
-        constexpr int N = decltype(n)::value;
-        if constexpr (TAIL != 1 && N < READ_STRIDE * NFR && N % READ_STRIDE == 0)
-          read_frag(a_base_of(1, ring), w_base_of(1, ring), 0, 0, ic<N / READ_STRIDE>{});
-        if constexpr (N < EB * PB && N % EB == EB - 1) {
-          auto ld = [&]() { direct_load(k_b, a_base_of(AHEAD_B, ring), w_base_of(AHEAD_B, ring), ic<PB_FIRST + N / EB>{}); };
-          if constexpr (CUR_B) ld();
-          else if (has_next) ld();
-        }
-      });
-      ring = slot_add(ring, RING5 ? 2 : 1);
-    };
-    {
-      constexpr std::true_type T{};
-      constexpr std::false_type F{};
-      // the last AHEAD_B iterations are tails; everything before is steady state
-      if (nk == 3 && AHEAD_B == 3) {
-        iteration(0, T, ic<3>{});
-      } else {
-        iteration(0, T, ic<0>{});
-        for (int kt = 1; kt < nk - AHEAD_B; ++kt) iteration(kt, F, ic<0>{});
-        if constexpr (AHEAD_B == 3) iteration(nk - 3, F, ic<3>{});
-      }
-      iteration(nk - 2, F, ic<2>{});
-      iteration(nk - 1, F, ic<1>{});
-    }
-    // inline-asm MFMAs are opaque to the compiler's hazard tracking: let the last results land before the
-    // epilogue reads the accumulation registers
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    CS_TS(2);
-
-    // ---- epilogue.  Accumulator (i, j), element r = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
-    //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
-    //      The loads the epilogue needs (row map, bias, residual / position rows) are issued ahead of the
-    //      stores that follow them, from clamped addresses so that no branch guards a load: a load inside the
-    //      store loop would make the compiler wait for ALL outstanding memory operations (vmcnt counts stores
-    //      too), i.e. for every store issued so far and for the next tile's prefetch, once per row block.
-    {
-      const bf16_t* const pBias = (const bf16_t*)p.bias;
-      bf16_t* const pC = (bf16_t*)p.C;
-      const int n_lane = n0 + wn * WTN + kq * (4 * G);
-      int mrow[MT];
-      int crow[MT];  // 32-bit row numbers; the 64-bit address is formed at the store
-#pragma unroll
-      for (int i = 0; i < MT; ++i) {
-        mrow[i] = m0 + wm * WTM + i * 16 + fa;
-        const int mc = min(mrow[i], p.M - 1);
-        crow[i] = p.c_rows ? p.c_rows[mc] : mc;
-      }
-      constexpr bool NORM_A = FUSE == FUSE_NORM_A || FUSE == FUSE_LN_A;
-      float rstd[NORM_A ? MT : 1];
-      float nmean_rstd[FUSE == FUSE_LN_A ? MT : 1];   // -mean * rstd
-      if constexpr (FUSE == FUSE_LN_A) {
-        auto total = [](const float* parts) {
-          const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
-          return ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
-        };
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-          const int64_t row = (int64_t)min(mrow[i], p.M - 1) * CS_SUMSQ_PARTS;
-          const float mean = total(p.a_row_sum + row) / (float)p.K;
-          const float var = fmaxf(total(p.a_row_sumsq + row) / (float)p.K - mean * mean, 0.f);
-          rstd[i] = rsqrtf(var + p.norm_eps);
-          nmean_rstd[i] = -mean * rstd[i];
-        }
-      }
-      if constexpr (FUSE == FUSE_NORM_A) {
-#pragma unroll
-        for (int i = 0; i < MT; ++i) {
-          const float* parts = p.a_row_sumsq + (int64_t)min(mrow[i], p.M - 1) * CS_SUMSQ_PARTS;
-          const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
-          const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
-          rstd[i] = rsqrtf(ss / (float)p.K + p.norm_eps);
-        }
-      }
-      f32x4_t csum_v[FUSE == FUSE_LN_A ? NT : 1];
-      if constexpr (FUSE == FUSE_LN_A) {
-#pragma unroll
-        for (int j = 0; j < NT; ++j) csum_v[j] = *(const f32x4_t*)(p.w_col_sum + min(n_lane + piece_col(j), p.N - 4));
-      }
-      bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
-#pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        const int nc = min(n_lane + piece_col(j), p.N - 4);
-        bias_v[j] = bf16x4_t{0, 0, 0, 0};
-        if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + nc);
-      }
-      f32x4_t scale_v[W_FP8 ? NT : 1];
-      if constexpr (W_FP8) {
-#pragma unroll
-        for (int j = 0; j < NT; ++j) scale_v[j] = *(const f32x4_t*)(p.w_scale + min(n_lane + piece_col(j), p.N - 4));
-      }
-      constexpr bool ADDEND = (EPI == CS_EPI_RESIDUAL) || (EPI == CS_EPI_BIAS_POS);
-      bf16x4_t addend[ADDEND ? MT : 1][ADDEND ? NT : 1];
-      auto load_addend = [&](auto i_c) {
-        constexpr int i = decltype(i_c)::value;
-        const int mc = min(mrow[i], p.M - 1);
-        const bf16_t* row = (EPI == CS_EPI_RESIDUAL)
-                                ? (const bf16_t*)p.residual + (int64_t)mc * p.ldr
-                                : (const bf16_t*)p.pos + (int64_t)(mc % p.pos_period) * p.ldpos;
-#pragma unroll
-        for (int j = 0; j < NT; ++j)
-          addend[ADDEND ? i : 0][ADDEND ? j : 0] = *(const bf16x4_t*)(row + min(n_lane + piece_col(j), p.N - 4));
-      };
-      // The kernel must stay inside the architectural registers (the accumulation registers are not the
-      // compiler's to use), so the addend rows are fetched in two batches.
-      constexpr int ADD_BATCH = MT / 2;
-      if constexpr (ADDEND) static_for<ADD_BATCH>(load_addend);
-      static_for<MT>([&](auto i_c) {
-        constexpr int i = decltype(i_c)::value;
-        if constexpr (ADDEND && i == ADD_BATCH)
-          static_for<MT - ADD_BATCH>([&](auto k_c) { load_addend(ic<ADD_BATCH + decltype(k_c)::value>{}); });
-        const bool mok = mrow[i] < p.M;
-        f32x4_t racc[NT];
-        static_for<NT * 4>([&](auto e_c) {
-          constexpr int E = decltype(e_c)::value;
-          float t;
-          asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(i * NT * 4 + E));
-          racc[E / 4][E % 4] = t;
-        });
-        bf16x4_t out[NT];
-#pragma unroll
-        for (int j = 0; j < NT; ++j) {
-          float v[4];
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            float t = racc[j][r];
-            if constexpr (W_FP8) t *= scale_v[W_FP8 ? j : 0][r];
-            if constexpr (NORM_A) t *= rstd[NORM_A ? i : 0];
-            if constexpr (FUSE == FUSE_LN_A) t += nmean_rstd[FUSE == FUSE_LN_A ? i : 0] * csum_v[FUSE == FUSE_LN_A ? j : 0][r];
-            v[r] = t + bf2f(bias_v[j][r]);
-          }
-          if (EPI == CS_EPI_SWIGLU) {
-            // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the
-            // product stay in fp32 until the single output rounding
-            const float g0 = silu(rbf(v[0])), u0 = rbf(v[1]);
-            const float g1 = silu(rbf(v[2])), u1 = rbf(v[3]);
-            out[j][0] = f2bf(g0 * u0);
-            out[j][1] = f2bf(g1 * u1);
-          } else {
-            if (EPI == CS_EPI_GELU_ERF) {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = gelu_erf(rbf(v[r]));
-            } else if (EPI == CS_EPI_GELU_TANH) {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(rbf(v[r]));
-            } else if (EPI == CS_EPI_QUICK_GELU) {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = quick_gelu(rbf(v[r]));
-            } else if (ADDEND) {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = rbf(v[r]) + bf2f(addend[ADDEND ? i : 0][ADDEND ? j : 0][r]);
-            }
-#pragma unroll
-            for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
-          }
-        }
-        if constexpr (FUSE == FUSE_SUMSQ_C || FUSE == FUSE_STATS_C) {
-          // Sum of squares of the row's ROUNDED outputs over this wave's columns: lane-local over the lane's
-          // pieces, then over the four lanes of the row (fixed order: the result does not depend on timing).
-          static_assert(WAVES_N == 1 && EPI != CS_EPI_SWIGLU, "one wave spans the tile's columns: one part per tile");
-          float ss = 0.f, sm = 0.f;
-#pragma unroll
-          for (int j = 0; j < NT; ++j) {
-            const bool nok = n_lane + piece_col(j) < p.N;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const float o = nok ? bf2f(out[j][r]) : 0.f;
-              ss += o * o;
-              if constexpr (FUSE == FUSE_STATS_C) sm += o;
-            }
-          }
-          ss += __shfl_xor(ss, 16);
-          ss += __shfl_xor(ss, 32);
-          if (mok && kq == 0) p.c_row_sumsq[(int64_t)crow[i] * CS_SUMSQ_PARTS + n0 / BN] = ss;
-          if constexpr (FUSE == FUSE_STATS_C) {
-            sm += __shfl_xor(sm, 16);
-            sm += __shfl_xor(sm, 32);
-            if (mok && kq == 0) p.c_row_sum[(int64_t)crow[i] * CS_SUMSQ_PARTS + n0 / BN] = sm;
-          }
-        }
-        // With G == 2 the pieces of fragments 2g and 2g+1 are adjacent: one 16-byte store per lane, and the
-        // four lanes of an output row write 64 consecutive bytes (32 with the halved SwiGLU output).
-        if (EPI == CS_EPI_SWIGLU) {
-          bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + (n_lane >> 1);
-          if constexpr (G == 2) {
-#pragma unroll
-            for (int j = 0; j < NT; j += 2) {
-              if (mok && n_lane + piece_col(j) < p.N) {
-                bf16x4_t o = {out[j][0], out[j][1], out[j + 1][0], out[j + 1][1]};
-                *(bf16x4_t*)(dst + (piece_col(j) >> 1)) = o;
-              }
-            }
-          } else {
-#pragma unroll
-            for (int j = 0; j < NT; ++j) {
-              if (mok && n_lane + piece_col(j) < p.N) {
-                bf16x2_t o;
-                o[0] = out[j][0];
-                o[1] = out[j][1];
-                *(bf16x2_t*)(dst + (piece_col(j) >> 1)) = o;
-              }
-            }
-          }
-        } else {
-          bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + n_lane;
-          if constexpr (G == 2) {
-#pragma unroll
-            for (int j = 0; j < NT; j += 2) {
-              if (mok && n_lane + piece_col(j) < p.N) {
-                bf16x8_t o = {out[j][0], out[j][1], out[j][2], out[j][3], out[j + 1][0], out[j + 1][1], out[j + 1][2], out[j + 1][3]};
-                *(bf16x8_t*)(dst + piece_col(j)) = o;
-              }
-            }
-          } else {
-#pragma unroll
-            for (int j = 0; j < NT; ++j)
-              if (mok && n_lane + piece_col(j) < p.N) *(bf16x4_t*)(dst + piece_col(j)) = out[j];
-          }
-        }
-      });
-    }
-    CS_TS(3);
-    if (!has_next) break;
-    vb = vb_next;
-    m0 = m0_next;
-    n0 = n0_next;
-  }
-}
-
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE = 0>
-int launch(const CsGemmArgs& a, hipStream_t stream) {
-  CsGemmArgs p = a;
-  p.tiles_m = (p.M + BM - 1) / BM;
-  p.tiles_n = (p.N + BN - 1) / BN;
-  constexpr int lds = RingShape<BM, BN, W_FP8>::BYTES;
-  static bool attr_set = false;
-  auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE>;
-  if (!attr_set) {
-    if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-      return CS_ERR_LAUNCH;
-    attr_set = true;
-  }
-  const int tiles = p.tiles_m * p.tiles_n;
-  // One resident workgroup per CU (LDS-bound); with more tiles than CUs the kernel is persistent.
-  const int grid = tiles <= 256 ? tiles : 256;
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, p);
-  return cs_launch_status();
-}
-
-template <int BM, int BN, int WAVES_M, int WAVES_N, bool W_FP8>
-int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
-  if constexpr (!W_FP8) {
-    // the fused-norm forms exist for the epilogues an encoder block pairs them with
-    if (a.a_row_sum) {   // LayerNorm in front of this GEMM
-      if (!a.a_row_sumsq || !a.w_col_sum || a.pos || a.c_row_sumsq || a.c_row_sum) return CS_ERR_UNSUPPORTED;
-      // (the per-column sums take 4 registers per piece on top of the bias: with the 64 pieces of a 256x256 tile's
-      // wave the epilogue no longer fits the architectural registers, so that tile is not built; cs_gemm_fast
-      // sends these launches to the 256x160 tile)
-      if constexpr (BM == 256 && BN == 256) return CS_ERR_UNSUPPORTED;
-      else switch (a.epilogue) {
-        case CS_EPI_BIAS: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_LN_A>(a, s);
-        case CS_EPI_GELU_TANH: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_TANH, false, FUSE_LN_A>(a, s);
-        case CS_EPI_QUICK_GELU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_QUICK_GELU, false, FUSE_LN_A>(a, s);
-        default: return CS_ERR_UNSUPPORTED;
-      }
-    }
-    if (a.c_row_sum) {   // ... and behind it: sums and sums of squares of the output rows
-      if (!a.c_row_sumsq || a.pos) return CS_ERR_UNSUPPORTED;
-      if constexpr (BN == 160 && WAVES_N == 1) {
-        if (a.epilogue == CS_EPI_RESIDUAL) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_STATS_C>(a, s);
-      }
-      return CS_ERR_UNSUPPORTED;
-    }
-    if (a.a_row_sumsq) {
-      if (a.pos || a.c_row_sumsq) return CS_ERR_UNSUPPORTED;
-      if (a.epilogue == CS_EPI_BIAS) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_NORM_A>(a, s);
-      if (a.epilogue == CS_EPI_SWIGLU) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_SWIGLU, false, FUSE_NORM_A>(a, s);
-      return CS_ERR_UNSUPPORTED;
-    }
-    if (a.c_row_sumsq) {
-      if constexpr (BN == 160 && WAVES_N == 1) {
-        if (a.epilogue == CS_EPI_RESIDUAL) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_SUMSQ_C>(a, s);
-        if (a.epilogue == CS_EPI_BIAS && !a.pos) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_SUMSQ_C>(a, s);
-      }
-      return CS_ERR_UNSUPPORTED;
-    }
-  } else {
-    if (a.a_row_sumsq || a.c_row_sumsq || a.a_row_sum || a.c_row_sum) return CS_ERR_UNSUPPORTED;
-  }
-  switch (a.epilogue) {
-    case CS_EPI_BIAS:
-      if constexpr (!W_FP8) {
-        if (a.pos) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS_POS, false>(a, s);
-      }
-      return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, W_FP8>(a, s);
-    case CS_EPI_RESIDUAL: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, W_FP8>(a, s);
-    case CS_EPI_SWIGLU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_SWIGLU, W_FP8>(a, s);
-    case CS_EPI_GELU_ERF:
-      if constexpr (W_FP8 && BN == 160) return CS_ERR_UNSUPPORTED;  // never dispatched, see cs_gemm_fast
-      else return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_ERF, W_FP8>(a, s);
-    case CS_EPI_GELU_TANH: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_TANH, W_FP8>(a, s);
-    case CS_EPI_QUICK_GELU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_QUICK_GELU, W_FP8>(a, s);
-    default: return CS_ERR_INVALID_ARG;
-  }
-}
-
-template <int BM, int BN, int WAVES_M, int WAVES_N>
-int dispatch_epi(const CsGemmArgs& a, hipStream_t s) {
-  if (a.w_fp8) {
-    // (the few-rows form is only dispatched for bf16 weights: its fp8 kernels are not built)
-    if constexpr (BM == 128 && BN == 160) return CS_ERR_UNSUPPORTED;
-    else return dispatch_epi_w<BM, BN, WAVES_M, WAVES_N, true>(a, s);
-  }
-  return dispatch_epi_w<BM, BN, WAVES_M, WAVES_N, false>(a, s);
-}
+using csgemm::BK;
 
 // Time of a launch in units of "one 256x256 tile on every CU": rounds of 256 workgroups times tile area.
 double rounds_cost(int M, int N, int bm, int bn) {
@@ -764,7 +49,7 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   // so every output element and every row-sum part is computed by the same sequence of operations: results do not
   // depend on which of the two a batch size selects.
   const bool few_rows = !a.w_fp8 && (int64_t)((a.M + 255) / 256) * ((a.N + 159) / 160) <= 128;
-  auto narrow = [&]() { return few_rows ? dispatch_epi<128, 160, 4, 1>(a, stream) : dispatch_epi<256, 160, 4, 1>(a, stream); };
+  auto narrow = [&]() { return few_rows ? cs_gemm_fast_tile_128x160(a, stream) : cs_gemm_fast_tile_256x160(a, stream); };
   // Row sums of squares come in CS_SUMSQ_PARTS parts, one per column tile of the 160-column forms.
   if (a.c_row_sumsq) {
     if (a.N > CS_SUMSQ_PARTS * 160 || a.w_fp8) return CS_ERR_UNSUPPORTED;
@@ -808,11 +93,11 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
       if (a.residual) hi.residual = (const char*)a.residual + (int64_t)n1 * 2;
       if (a.pos) hi.pos = (const char*)a.pos + (int64_t)n1 * 2;
       hi.C = (char*)a.C + (int64_t)(a.epilogue == CS_EPI_SWIGLU ? n1 / 2 : n1) * 2;
-      const int st = dispatch_epi<256, 256, 2, 2>(lo, stream);
+      const int st = cs_gemm_fast_tile_256x256(lo, stream);
       if (st != CS_OK) return st;
-      if (best_192) return dispatch_epi<128, 192, 2, 2>(hi, stream);
-      return dispatch_epi<256, 128, 2, 2>(hi, stream);
+      if (best_192) return cs_gemm_fast_tile_128x192(hi, stream);
+      return cs_gemm_fast_tile_256x128(hi, stream);
     }
   }
-  return dispatch_epi<256, 256, 2, 2>(a, stream);
+  return cs_gemm_fast_tile_256x256(a, stream);
 }

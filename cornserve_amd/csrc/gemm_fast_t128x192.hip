@@ -1,0 +1,6 @@
+// The 128x192 tile form (2x2 waves) of the fast bf16 / fp8-weight MFMA GEMM: every epilogue and folded-norm
+// variant of this tile shape.  The accumulators live in accumulation registers that only inline assembly touches
+// (CS_ALL_ACC_REGS: the build checks this file's compiler output for stray uses of them).
+#include "gemm_fast_impl.h"
+
+int cs_gemm_fast_tile_128x192(const CsGemmArgs& a, hipStream_t stream) { return dispatch_epi<128, 192, 2, 2>(a, stream); }
