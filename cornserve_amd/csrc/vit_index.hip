@@ -179,27 +179,26 @@ __global__ __launch_bounds__(256) void row_gather_kernel(const char* __restrict_
 }
 
 // In-place rotary on the q and k column blocks of a packed [L, 3*heads*d] buffer.  One thread owns
-// VEC (8, or 4 when d/2 is not a multiple of 8) consecutive j of one (row, q|k, head): it reads x[j..j+VEC) and x[d/2+j..), rotates in fp32 and
-// writes both halves back with a single bf16 rounding.
+// VEC (8, or 4 when d/2 is not a multiple of 8) consecutive j of one (row, head) in BOTH q and k: it fetches the
+// cosines and sines once, reads x[j..j+VEC) and x[d/2+j..) of q and of k, rotates in fp32 and writes the halves back
+// with a single bf16 rounding.  Work items are numbered with 32 bits (checked on the host).
 template <int VEC>
 __global__ __launch_bounds__(256) void rope_qk_kernel(bf16_t* __restrict__ qkv, int64_t ld,
                                                       const float* __restrict__ cos_sin, int L, int heads, int d) {
   typedef __attribute__((__vector_size__(VEC * sizeof(__bf16)))) __bf16 vec_t;
   const int half = d >> 1;
-  const int cpr = half / VEC;  // chunks per (row, head, tensor)
-  const int64_t total = (int64_t)L * 2 * heads * cpr;
-  int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const unsigned cpr = (unsigned)half / VEC;  // chunks per (row, head)
+  const unsigned per_row = (unsigned)heads * cpr;
+  const unsigned total = (unsigned)L * per_row;
+  const unsigned idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
-  const int jc = idx % cpr;
-  idx /= cpr;
-  const int h = idx % heads;
-  idx /= heads;
-  const int which = idx % 2;
-  const int64_t l = idx / 2;
-  bf16_t* base = qkv + l * ld + (int64_t)which * heads * d + h * d + jc * VEC;
-  const float* cs = cos_sin + l * d + jc * VEC;
-  const vec_t x1 = *(const vec_t*)base;
-  const vec_t x2 = *(const vec_t*)(base + half);
+  const unsigned l = idx / per_row, rem = idx - l * per_row;
+  const unsigned h = rem / cpr, jc = rem - h * cpr;
+  bf16_t* qb = qkv + (int64_t)l * ld + h * d + jc * VEC;
+  bf16_t* kb = qb + heads * d;
+  const float* cs = cos_sin + (int64_t)l * d + jc * VEC;
+  const vec_t q1 = *(const vec_t*)qb, q2 = *(const vec_t*)(qb + half);
+  const vec_t k1 = *(const vec_t*)kb, k2 = *(const vec_t*)(kb + half);
   float co[VEC], si[VEC];
 #pragma unroll
   for (int e = 0; e < VEC; e += 4) {
@@ -210,15 +209,20 @@ __global__ __launch_bounds__(256) void rope_qk_kernel(bf16_t* __restrict__ qkv, 
       si[e + q] = s[q];
     }
   }
-  vec_t o1, o2;
+  vec_t o1, o2, p1, p2;
 #pragma unroll
   for (int e = 0; e < VEC; ++e) {
-    const float a = bf2f(x1[e]), b = bf2f(x2[e]);
+    const float a = bf2f(q1[e]), b = bf2f(q2[e]);
     o1[e] = f2bf(rot_first(a, b, co[e], si[e]));
     o2[e] = f2bf(rot_second(a, b, co[e], si[e]));
+    const float c = bf2f(k1[e]), g = bf2f(k2[e]);
+    p1[e] = f2bf(rot_first(c, g, co[e], si[e]));
+    p2[e] = f2bf(rot_second(c, g, co[e], si[e]));
   }
-  *(vec_t*)base = o1;
-  *(vec_t*)(base + half) = o2;
+  *(vec_t*)qb = o1;
+  *(vec_t*)(qb + half) = o2;
+  *(vec_t*)kb = p1;
+  *(vec_t*)(kb + half) = p2;
 }
 
 }  // namespace
@@ -352,14 +356,13 @@ extern "C" int cs_rope_qk(void* qkv, int64_t ld, const float* cos_sin, int32_t L
       ld < (int64_t)3 * heads * head_dim || (((uintptr_t)qkv | (uintptr_t)cos_sin) & 15))
     return CS_ERR_INVALID_ARG;
   if (L == 0) return CS_OK;
-  if (head_dim % 16 == 0) {
-    const int64_t total = (int64_t)L * 2 * heads * (head_dim / 16);
-    hipLaunchKernelGGL(rope_qk_kernel<8>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (bf16_t*)qkv, ld,
-                       cos_sin, L, heads, head_dim);
-  } else {  // d/2 is a multiple of 4 only (head dim 72): 8-byte vectors
-    const int64_t total = (int64_t)L * 2 * heads * (head_dim / 8);
-    hipLaunchKernelGGL(rope_qk_kernel<4>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, (bf16_t*)qkv, ld,
-                       cos_sin, L, heads, head_dim);
-  }
+  const int vec = head_dim % 16 == 0 ? 8 : 4;   // d/2 is a multiple of 4 only for head dim 72: 8-byte vectors
+  const int64_t total = (int64_t)L * heads * (head_dim / 2 / vec);
+  if (total > 0x7fffff00) return CS_ERR_TOO_LARGE;   // the kernel numbers its work items with 32 bits
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  if (vec == 8)
+    hipLaunchKernelGGL(rope_qk_kernel<8>, grid, block, 0, stream, (bf16_t*)qkv, ld, cos_sin, L, heads, head_dim);
+  else
+    hipLaunchKernelGGL(rope_qk_kernel<4>, grid, block, 0, stream, (bf16_t*)qkv, ld, cos_sin, L, heads, head_dim);
   return cs_launch_status();
 }
