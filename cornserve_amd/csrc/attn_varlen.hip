@@ -668,9 +668,12 @@ struct AttnDirectShape {
   static_assert(2 * LDS <= 160 * 1024, "two workgroups per CU");
 };
 
-template <int D>
+// ROPE_Q: the keys were rotated in place beforehand; the query rows are rotated here while they are staged (a
+// query block is staged once, whereas every query block of a segment would rotate the segment's keys again).
+template <int D, bool ROPE_Q = false>
 __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs a) {
   constexpr int NT = 256, BQ = 128;
+  static_assert(!ROPE_Q || D % 16 == 0, "rotary needs an even number of 16-byte chunks per half");
   using Shape = AttnDirectShape<D>;
   constexpr int KS = Shape::KS, DT = (D + 31) / 32, DC = Shape::DC, DKC = Shape::DKC;
   constexpr int RS = Shape::RS, K_SLOTS = Shape::K_SLOTS, V_SLOTS = Shape::V_SLOTS;
@@ -767,11 +770,38 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
   // ---- prologue: tile 0 requested, Q -> LDS -> fragments, then the Q region becomes buffers 1 and 2
   issue_tile(0, 0);
   init_padding(0);
-  for (int i = tid; i < BQ * DKC; i += NT) {
-    const int r = i / DKC, c = i - r * DKC;
-    bf16x8_t x = zero8;
-    if (r < nq && c < DC) x = *(const bf16x8_t*)(a.q + (int64_t)(q0 + r) * a.ld + hoff + c * 8);
-    *(bf16x8_t*)(q_lds + r * RS + c * 16) = x;
+  if constexpr (ROPE_Q) {
+    constexpr int HC = DC / 2;   // chunks per half; D % 16 == 0, so there are no padding chunks (DKC == DC)
+    for (int i = tid; i < BQ * HC; i += NT) {
+      const int r = i / HC, jc = i - r * HC;
+      bf16x8_t o1 = zero8, o2 = zero8;
+      if (r < nq) {
+        const int64_t g = q0 + r;
+        const bf16_t* p = a.q + g * a.ld + hoff + jc * 8;
+        const bf16x8_t x1 = *(const bf16x8_t*)p;
+        const bf16x8_t x2 = *(const bf16x8_t*)(p + D / 2);
+        const float* cs = a.cos_sin + g * D + jc * 8;
+        const f32x4_t c0 = *(const f32x4_t*)cs, c1 = *(const f32x4_t*)(cs + 4);
+        const f32x4_t s0 = *(const f32x4_t*)(cs + D / 2), s1 = *(const f32x4_t*)(cs + D / 2 + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float co = e < 4 ? c0[e] : c1[e - 4];
+          const float si = e < 4 ? s0[e] : s1[e - 4];
+          const float xa = bf2f(x1[e]), xb = bf2f(x2[e]);
+          o1[e] = f2bf(rot_first(xa, xb, co, si));
+          o2[e] = f2bf(rot_second(xa, xb, co, si));
+        }
+      }
+      *(bf16x8_t*)(q_lds + r * RS + jc * 16) = o1;
+      *(bf16x8_t*)(q_lds + r * RS + (jc + HC) * 16) = o2;
+    }
+  } else {
+    for (int i = tid; i < BQ * DKC; i += NT) {
+      const int r = i / DKC, c = i - r * DKC;
+      bf16x8_t x = zero8;
+      if (r < nq && c < DC) x = *(const bf16x8_t*)(a.q + (int64_t)(q0 + r) * a.ld + hoff + c * 8);
+      *(bf16x8_t*)(q_lds + r * RS + c * 16) = x;
+    }
   }
   __syncthreads();
   bf16x8_t qf[KS];
@@ -838,11 +868,11 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
 }
 
 
-template <int D>
+template <int D, bool ROPE_Q = false>
 int launch_attn_full_direct(const AttnArgs& a, dim3 grid, hipStream_t stream) {
   constexpr int lds = AttnDirectShape<D>::LDS;
   static bool attr_set = false;
-  auto kern = attn_full_direct_kernel<D>;
+  auto kern = attn_full_direct_kernel<D, ROPE_Q>;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return CS_ERR_LAUNCH;
@@ -853,7 +883,8 @@ int launch_attn_full_direct(const AttnArgs& a, dim3 grid, hipStream_t stream) {
 }
 
 template <int D>
-int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, bool rope, hipStream_t stream) {
+int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, bool rope, bool keys_rotated,
+                hipStream_t stream) {
   const dim3 grid(n_work, heads);
   a.n_work = n_work;
   a.heads = heads;
@@ -861,6 +892,14 @@ int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, 
   a.n_chunks_x = (n_work + a.chunk - 1) / a.chunk;
   const int n_chunks = a.n_chunks_x * heads;
   const dim3 grid_full(((n_chunks + 7) / 8) * 8 * a.chunk);
+  if (keys_rotated) {
+    // only the long-segment kernel has this form (short segments rotate q and k while staging, one workgroup each)
+    if constexpr (D % 16 == 0) {
+      if (block_q != 64 && rope && (int64_t)max_seqlen * a.ld * 2 < (int64_t)1 << 31)
+        return launch_attn_full_direct<D, true>(a, grid_full, stream);
+    }
+    return CS_ERR_UNSUPPORTED;
+  }
   if (block_q == 64) {
     if (rope) {
       // two heads per workgroup when that still leaves several workgroups per CU
@@ -913,10 +952,11 @@ extern "C" int cs_attn_work_host(const int32_t* cu_seqlens_host, int32_t n_seg, 
   return CS_OK;
 }
 
-extern "C" int cs_attn_varlen(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
-                              const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
-                              const float* cos_sin, int32_t max_seqlen, void* stream_) {
+static int attn_varlen_entry(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
+                             const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
+                             const float* cos_sin, int32_t max_seqlen, bool keys_rotated, void* stream_) {
   hipStream_t stream = (hipStream_t)stream_;
+  if (keys_rotated && !cos_sin) return CS_ERR_INVALID_ARG;
   if (!q || !k || !v || !out || !work || n_work < 0 || heads <= 0 || heads > 65535 || head_dim <= 0 ||
       max_seqlen <= 0)
     return CS_ERR_INVALID_ARG;
@@ -937,10 +977,23 @@ extern "C" int cs_attn_varlen(const void* q, const void* k, const void* v, int64
   const int bq = cs_attn_block_q(max_seqlen);
   const bool rope = cos_sin != nullptr;
   switch (head_dim) {
-    case 64: return launch_attn<64>(a, n_work, heads, bq, max_seqlen, rope, stream);
-    case 72: return launch_attn<72>(a, n_work, heads, bq, max_seqlen, rope, stream);
-    case 80: return launch_attn<80>(a, n_work, heads, bq, max_seqlen, rope, stream);
-    case 96: return launch_attn<96>(a, n_work, heads, bq, max_seqlen, rope, stream);
+    case 64: return launch_attn<64>(a, n_work, heads, bq, max_seqlen, rope, keys_rotated, stream);
+    case 72: return launch_attn<72>(a, n_work, heads, bq, max_seqlen, rope, keys_rotated, stream);
+    case 80: return launch_attn<80>(a, n_work, heads, bq, max_seqlen, rope, keys_rotated, stream);
+    case 96: return launch_attn<96>(a, n_work, heads, bq, max_seqlen, rope, keys_rotated, stream);
     default: return CS_ERR_UNSUPPORTED;
   }
+}
+
+extern "C" int cs_attn_varlen(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
+                              const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
+                              const float* cos_sin, int32_t max_seqlen, void* stream) {
+  return attn_varlen_entry(q, k, v, ld, out, ldo, work, n_work, heads, head_dim, scale, cos_sin, max_seqlen, false, stream);
+}
+
+extern "C" int cs_attn_varlen_keys_rotated(const void* q, const void* k, const void* v, int64_t ld, void* out,
+                                           int64_t ldo, const int32_t* work, int32_t n_work, int32_t heads,
+                                           int32_t head_dim, float scale, const float* cos_sin, int32_t max_seqlen,
+                                           void* stream) {
+  return attn_varlen_entry(q, k, v, ld, out, ldo, work, n_work, heads, head_dim, scale, cos_sin, max_seqlen, true, stream);
 }

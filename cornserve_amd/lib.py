@@ -83,6 +83,10 @@ _SIGNATURES: dict[str, list] = {
         c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
         c_void_p, c_int32, c_int32, c_int32, c_float, c_void_p, c_int32, c_void_p,
     ],
+    "cs_attn_varlen_keys_rotated": [
+        c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int64,
+        c_void_p, c_int32, c_int32, c_int32, c_float, c_void_p, c_int32, c_void_p,
+    ],
     "cs_attn_block_q": [c_int32],
     "cs_attn_work_host": [c_void_p, c_int32, c_int32, c_void_p, c_int32, POINTER(c_int32)],
     "cs_qwen_patchify_u8": [c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64,

@@ -422,8 +422,10 @@ def attn_plan(cu_seqlens_host: np.ndarray, device: torch.device) -> AttnPlan:
 
 
 def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPlan, heads: int, head_dim: int,
-                scale: float, cos_sin: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
-    """q/k/v: [L, >= heads*head_dim] views sharing one row stride (e.g. thirds of a packed QKV buffer)."""
+                scale: float, cos_sin: torch.Tensor | None = None, out: torch.Tensor | None = None,
+                keys_rotated: bool = False) -> torch.Tensor:
+    """q/k/v: [L, >= heads*head_dim] views sharing one row stride (e.g. thirds of a packed QKV buffer).
+    `keys_rotated`: k already carries the rotary of `cos_sin`; only q is rotated (long segments only)."""
     lib = _l.load()
     for name, t in (("q", q), ("k", k), ("v", v)):
         _req(t, torch.bfloat16, name)
@@ -436,11 +438,11 @@ def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPla
             raise ValueError("cos_sin must be contiguous [L, head_dim]")
     if out is None:
         out = torch.empty((L, heads * head_dim), dtype=torch.bfloat16, device=q.device)
+    entry = lib.cs_attn_varlen_keys_rotated if keys_rotated else lib.cs_attn_varlen
     _l.check(
-        lib.cs_attn_varlen(q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
-                           plan.work.data_ptr(), plan.n_work, heads, head_dim, scale, _ptr(cos_sin),
-                           plan.max_seqlen, _stream()),
-        "cs_attn_varlen",
+        entry(q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
+              plan.work.data_ptr(), plan.n_work, heads, head_dim, scale, _ptr(cos_sin), plan.max_seqlen, _stream()),
+        "cs_attn_varlen_keys_rotated" if keys_rotated else "cs_attn_varlen",
     )
     return out
 
@@ -448,19 +450,22 @@ def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPla
 def attn_varlen_rotary_(qkv: torch.Tensor, plan: AttnPlan, heads: int, head_dim: int, scale: float,
                         cos_sin: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """Rotary + attention over a packed [L, 3*heads*head_dim] buffer whose q and k the caller no longer needs.
-    Segments of at most 64 rows (window attention) take the kernel that rotates while it stages q and k; longer
-    segments rotate q and k in place once (every query block of a segment would otherwise rotate the segment's keys
-    again) and take the kernel that streams K/V tiles straight into LDS.  Both routes give the same bits."""
+    Segments of at most 64 rows (window attention) take the kernel that rotates while it stages q and k.  Longer
+    segments rotate the keys in place once (every query block of a segment would otherwise rotate the segment's keys
+    again) and take the kernel that streams K/V tiles straight into LDS and rotates its query rows while staging them;
+    head shapes that kernel does not take rotate q and k in place and run without a table.  All routes give the same
+    bits."""
     E = heads * head_dim
     q, k, v = qkv[:, :E], qkv[:, E : 2 * E], qkv[:, 2 * E :]
     if plan.max_seqlen <= 64:
         return attn_varlen(q, k, v, plan, heads, head_dim, scale, cos_sin=cos_sin, out=out)
+    if heads % 2 == 0 and head_dim % 16 == 0 and plan.max_seqlen * qkv.stride(0) * 2 < 2**31:
+        rope_qk_(qkv[:, E:], cos_sin, heads // 2, head_dim)   # the k block as two tensors of heads / 2 heads
+        return attn_varlen(q, k, v, plan, heads, head_dim, scale, cos_sin=cos_sin, out=out, keys_rotated=True)
     rope_qk_(qkv, cos_sin, heads, head_dim)
     return attn_varlen(q, k, v, plan, heads, head_dim, scale, out=out)
 
 
-
-# ------------------------------------------------------------------------------------------ SigLIP
 def qwen_patchify_u8(frames: torch.Tensor, table: torch.Tensor, patch: int, merge: int, temporal: int, *,
                      out: torch.Tensor | None = None, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """uint8 frames [T,H,W,3] -> normalised patch rows [ceil(T/temporal)*(H/patch)*(W/patch), 3*temporal*patch^2]

@@ -204,6 +204,15 @@ int cs_rows_bilinear(const void* src, int64_t lds, int32_t n_src_rows, const int
 int cs_attn_varlen(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
                    const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
                    const float* cos_sin, int32_t max_seqlen, void* stream);
+/* The same call for a caller that has ALREADY rotated the keys in place (cs_rope_qk on the k block, i.e. with the
+ * k block's address and heads / 2): only the query rows are rotated here, with cos_sin (required), while a query
+ * block is staged.  A segment's keys are then rotated once instead of once per query block, which is what the
+ * fused path of cs_attn_varlen costs on long segments (the rotary of qwen2_5_vl.py:26-33,104-108 in front of full
+ * attention).  Same bits as cs_attn_varlen with the same table.  Only for max_seqlen > 64 and head_dim % 16 == 0
+ * (CS_ERR_UNSUPPORTED otherwise: short segments take cs_attn_varlen, which rotates each row once anyway).        */
+int cs_attn_varlen_keys_rotated(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
+                                const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
+                                const float* cos_sin, int32_t max_seqlen, void* stream);
 /* Host routine: expand cu_seqlens_host[n_seg+1] into query-block work items of at most block_q rows
  * (block_q = cs_attn_block_q(max_seqlen)).  Writes n_work items of 4 int32 into work_host.      */
 int cs_attn_block_q(int32_t max_seqlen);

@@ -121,10 +121,11 @@ def test_qwen_patchify_u8_bit_exact(ops, dev, t, h, w, patch, merge, temporal):
         ops.qwen_patchify_u8(torch.zeros((1, 30, 28, 3), dtype=torch.uint8, device=dev), table.to(dev), 14, 2, 2)
 
 
-@pytest.mark.parametrize("heads,d", [(16, 80), (4, 64), (2, 96)])
+@pytest.mark.parametrize("heads,d", [(16, 80), (4, 64), (2, 96), (3, 80)])
 def test_attn_rotary_in_place_route_equals_fused_route(ops, dev, heads, d):
-    """Long segments: rotating q and k in place and running the kernel without rotary gives the bits of the kernel
-    that rotates while staging (ragged segment lengths either side of the tile sizes)."""
+    """Long segments: rotating the keys in place and the query rows while they are staged (or, for head shapes without
+    that kernel, q and k in place) gives the bits of the kernel that rotates everything while staging (ragged segment
+    lengths either side of the tile sizes)."""
     lens = [100, 1024, 65, 300, 128, 1, 777]
     cu = np.concatenate([[0], np.cumsum(lens)]).astype(np.int32)
     L, E = int(cu[-1]), heads * d
@@ -137,7 +138,12 @@ def test_attn_rotary_in_place_route_equals_fused_route(ops, dev, heads, d):
     buf = qkv.clone()
     got = ops.attn_varlen_rotary_(buf, plan, heads, d, d ** -0.5, cs)
     assert torch.equal(got, fused)
-    assert not torch.equal(buf[:, :E], qkv[:, :E]) and torch.equal(buf[:, 2 * E:], qkv[:, 2 * E:])   # q, k rotated; v untouched
+    # k rotated in place, v untouched; q only where the keys-rotated kernel does not apply (odd head count)
+    assert not torch.equal(buf[:, E:2 * E], qkv[:, E:2 * E]) and torch.equal(buf[:, 2 * E:], qkv[:, 2 * E:])
+    assert torch.equal(buf[:, :E], qkv[:, :E]) == (heads % 2 == 0)
+    rot = qkv.clone()
+    ops.rope_qk_(rot, cs, heads, d)
+    assert torch.equal(buf[:, E:2 * E], rot[:, E:2 * E])   # the k block rotated as two half-size tensors = rotated as one
     short = ops.attn_plan(np.arange(0, 64 * 5 + 1, 64, dtype=np.int32), dev)   # window route: the buffer stays as it is
     buf = qkv[:320].clone()
     got = ops.attn_varlen_rotary_(buf, short, heads, d, d ** -0.5, cs[:320].contiguous())
