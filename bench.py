@@ -340,6 +340,9 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-power-probe", action="store_true",
+                    help="skip roofline.power_limit_probe (its 600 extra launches of the dominant GEMM, a third of them "
+                         "on zero weights, would blur that kernel's average in a profile)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (counter calibration for rocprofv3 --pmc runs)")
     ap.add_argument("--cpu-sample-images", type=int, default=8)
@@ -456,7 +459,7 @@ def main() -> None:
             model.forward_device(one_px, one_grid)
         torch.cuda.synchronize()
         one_ms = (time.perf_counter() - t0) / 10 * 1e3
-        probe = power_limit_probe(torch, ops, model, L) if model.fold_norm else None
+        probe = power_limit_probe(torch, ops, model, L) if model.fold_norm and not args.no_power_probe else None
     stage_ms = {k: sum(v) / 3 for k, v in full.durations_ms().items()}
     mfma_keys = [k for k in stage_ms if k.startswith("gemm_") or k.startswith("attn_") or k == "patch_embed"]
     # The instrumented pass records an event between stages, which costs a little device time per mark: its
