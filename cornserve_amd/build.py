@@ -87,6 +87,8 @@ def _check_source(hipcc: str, src: Path) -> None:
     offenders = check_hand_managed_acc_registers(asm.read_text())
     asm.unlink()
     if offenders:
+        # the object of a source that fails this check must not survive for a later incremental build to link
+        (OBJ_DIR / (src.stem + ".o")).unlink(missing_ok=True)
         raise RuntimeError(f"{src.name}: the compiler used accumulation registers that inline assembly owns:\n  "
                            + "\n  ".join(offenders))
 

@@ -15,6 +15,7 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(int)))) int i32x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
 
 #define CS_DEVICE __device__ __forceinline__
 
@@ -23,6 +24,40 @@ CS_DEVICE float bf2f(bf16_t x) { return (float)x; }
 CS_DEVICE bf16_t f2bf(float x) { return (bf16_t)x; }
 // Round an fp32 value to bf16 precision and return it as fp32 (a "rounding point").
 CS_DEVICE float rbf(float x) { return (float)(bf16_t)x; }
+
+// Residual stream with 16 significant bits: a value is kept as a bf16 "hi" plane, which is what the next GEMM reads
+// as its operand, and a byte "lo" plane holding the next 8 mantissa bits as a signed correction:
+//   value = bits(hi) << 16  +  (int8)lo << 8     (as an fp32 bit pattern: sign-magnitude, so the sum is monotone)
+// split24 rounds an fp32 value to 24 bits (nearest, at bit 8), then rounds those 24 bits half-up in magnitude to hi;
+// lo is what is left.  A zero lo plane means "the value is hi exactly", so a plain bf16 tensor next to a zero-filled
+// byte plane is a valid pair.  The residual additions of an encoder then lose 2^-17 per addition instead of the 2^-9
+// of a bf16 stream, for 3 bytes per element instead of the 6 of an fp32 stream plus its bf16 copy.
+CS_DEVICE float join24(uint32_t hi_bits, uint32_t lo_byte) {
+  const int32_t corr = (int32_t)(int8_t)lo_byte;
+  return __builtin_bit_cast(float, (uint32_t)((int32_t)(hi_bits << 16) + (corr << 8)));
+}
+CS_DEVICE void split24(float v, uint32_t& hi_bits, uint32_t& lo_byte) {
+  const uint32_t b = __builtin_bit_cast(uint32_t, v) + 0x80u;
+  lo_byte = (b >> 8) & 0xFFu;
+  hi_bits = (b + 0x8000u) >> 16;
+}
+
+// Four values at once: the addend's planes as raw words (two bf16 per word, four bytes in one word) joined with four
+// fp32 increments, and the sums split again.
+CS_DEVICE void add_split24(const float (&delta)[4], u32x2_t hi_in, uint32_t lo_in, u32x2_t& hi_out, uint32_t& lo_out) {
+  uint32_t h[2] = {0u, 0u}, l = 0u;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const uint32_t hi_r = (hi_in[r >> 1] >> (16 * (r & 1))) & 0xFFFFu;
+    const uint32_t lo_r = (lo_in >> (8 * r)) & 0xFFu;
+    uint32_t ho, lo;
+    split24(delta[r] + join24(hi_r, lo_r), ho, lo);
+    h[r >> 1] |= (ho & 0xFFFFu) << (16 * (r & 1));
+    l |= lo << (8 * r);
+  }
+  hi_out = u32x2_t{h[0], h[1]};
+  lo_out = l;
+}
 
 // One rotary pair in fp32 with every product and sum rounded on its own (no fused multiply-add), as the
 // reference's tensor program computes it (x1*cos - x2*sin, x1*sin + x2*cos): every kernel that rotates gives

@@ -240,6 +240,9 @@ extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
   if (a.w_fp8 ? (a.ldw % 16 || a.K % 16 || !a.w_scale) : (a.ldw % 8)) return CS_ERR_INVALID_ARG;
   if (a.epilogue == CS_EPI_RESIDUAL && (!a.residual || a.ldr % 4)) return CS_ERR_INVALID_ARG;
   if (a.epilogue != CS_EPI_SWIGLU && a.ldc % 4) return CS_ERR_INVALID_ARG;
+  // the byte planes of a 16-bit residual stream: only with the residual epilogue, 4-byte accesses along N
+  if ((a.c_lo || a.residual_lo) && (a.epilogue != CS_EPI_RESIDUAL || a.pos || !a.c_lo)) return CS_ERR_INVALID_ARG;
+  if (((uintptr_t)a.c_lo | (uintptr_t)a.residual_lo) & 7) return CS_ERR_INVALID_ARG;
   if (a.pos && (a.pos_period <= 0 || a.ldpos % 4 || a.epilogue == CS_EPI_SWIGLU)) return CS_ERR_INVALID_ARG;
   if (((uintptr_t)a.A | (uintptr_t)a.W) & 15) return CS_ERR_INVALID_ARG;
   if (((uintptr_t)a.C | (uintptr_t)a.bias | (uintptr_t)a.residual | (uintptr_t)a.pos) & 7) return CS_ERR_INVALID_ARG;

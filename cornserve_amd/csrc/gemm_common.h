@@ -80,6 +80,16 @@ CS_DEVICE void epilogue(const CsGemmArgs& p, const f32x16_t (&acc)[MT][NT], int 
             for (int q = 0; q < 4; ++q) v[q] = quick_gelu(rbf(v[q]));
           } else if (EPI == CS_EPI_RESIDUAL) {
             const bf16x4_t r = *(const bf16x4_t*)(pRes + (int64_t)m * p.ldr + n);
+            if (p.c_lo) {  // residual stream with 16 significant bits: join, add unrounded, split
+              const uint32_t lo4 = p.residual_lo ? *(const uint32_t*)(p.residual_lo + (int64_t)m * p.ldr + n) : 0u;
+              u32x2_t hi_words;
+              uint32_t packed_lo;
+              add_split24(v, __builtin_bit_cast(u32x2_t, r), lo4, hi_words, packed_lo);
+              const bf16x4_t o = __builtin_bit_cast(bf16x4_t, hi_words);
+              *(bf16x4_t*)(pC + crow * p.ldc + n) = o;
+              *(uint32_t*)(p.c_lo + crow * p.ldc + n) = packed_lo;
+              continue;
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q) v[q] = rbf(v[q]) + bf2f(r[q]);
           }

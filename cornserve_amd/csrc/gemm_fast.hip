@@ -91,6 +91,8 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
       if (a.w_scale) hi.w_scale = a.w_scale + n1;
       if (a.bias) hi.bias = (const char*)a.bias + (int64_t)n1 * 2;
       if (a.residual) hi.residual = (const char*)a.residual + (int64_t)n1 * 2;
+      if (a.residual_lo) hi.residual_lo = a.residual_lo + n1;
+      if (a.c_lo) hi.c_lo = a.c_lo + n1;
       if (a.pos) hi.pos = (const char*)a.pos + (int64_t)n1 * 2;
       hi.C = (char*)a.C + (int64_t)(a.epilogue == CS_EPI_SWIGLU ? n1 / 2 : n1) * 2;
       const int st = cs_gemm_fast_tile_256x256(lo, stream);

@@ -136,7 +136,7 @@ struct RingShape {
 // rstd * (acc - mean * w_col_sum[n]) + bias[n] with mean and rstd from the two sets of parts (the norm's weight is
 // folded into W, its bias into the GEMM bias, and w_col_sum[n] = sum_k W'[n,k] carries the mean term).
 constexpr int FUSE_NORM_A = 1, FUSE_SUMSQ_C = 2, FUSE_LN_A = 3, FUSE_STATS_C = 4;
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE, bool SPLIT_RES>
 __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   static_assert(WAVES_M * WAVES_N == NW, "four waves, one per SIMD");
@@ -203,10 +203,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   //      lane lands in slot lane%8 of row 8rb + lane/8 and fetches chunk (lane%8) ^ key(row).  Buffer
   //      loads: a 32-bit per-lane byte offset plus a scalar K offset on a scalar descriptor, so an address
   //      costs one register and no vector arithmetic.
-  const int l_row = lane >> 3, l_slot = lane & 7;
   uint32_t a_src[A_LD];
   uint32_t w_src[W_LD];
   auto setup_sources = [&](int m0, int n0) {
+    // (an opaque copy of the lane number: the swizzled chunk offsets are recomputed at every call instead of being
+    // kept in registers across the main loop)
+    int lane_s = lane;
+    asm volatile("" : "+v"(lane_s));
+    const int l_row = lane_s >> 3, l_slot = lane_s & 7;
 #pragma unroll
     for (int j = 0; j < A_LD; ++j) {
       const int row = (j * NW + wave) * 8 + l_row;  // tile-local
@@ -218,10 +222,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     for (int j = 0; j < W_LD; ++j) {
       const int blk = min(j * NW + wave, W_BLK - 1);
       if constexpr (W_FP8) {  // 64-byte rows: the lane lands in slot lane%4 of row 16 blk + lane/4
-        const int row = blk * 16 + (lane >> 2);
+        const int row = blk * 16 + (lane_s >> 2);
         const int key = ((row % (16 * G)) / (4 * G)) & 3;
         const int r = min(n0 + row, p.N - 1);
-        w_src[j] = (uint32_t)((int64_t)r * p.ldw + (((lane & 3) ^ key) << 4));
+        w_src[j] = (uint32_t)((int64_t)r * p.ldw + (((lane_s & 3) ^ key) << 4));
       } else {
         const int row = blk * 8 + l_row;
         const int key = ((((row % (16 * G)) / (4 * G)) & 3) << 1) | ((row >> 1) & 1);
@@ -460,6 +464,12 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     {
       const bf16_t* const pBias = (const bf16_t*)p.bias;
       bf16_t* const pC = (bf16_t*)p.C;
+      // The lane's column and row are re-derived behind an opaque copy of the lane number: otherwise the compiler
+      // hoists the lane-dependent halves of the epilogue's addresses out of the tile loop and keeps them in registers
+      // across the main loop, which has none to spare.
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
+      const int fa = lane_e & 15, kq = lane_e >> 4;
       const int n_lane = n0 + wn * WTN + kq * (4 * G);
       int mrow[MT];
       int crow[MT];  // 32-bit row numbers; the 64-bit address is formed at the store
@@ -513,7 +523,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         for (int j = 0; j < NT; ++j) scale_v[j] = *(const f32x4_t*)(p.w_scale + min(n_lane + piece_col(j), p.N - 4));
       }
       constexpr bool ADDEND = (EPI == CS_EPI_RESIDUAL) || (EPI == CS_EPI_BIAS_POS);
+      // SPLIT: the residual stream is carried with 16 significant bits (bf16 plane + byte plane, see split24)
+      constexpr bool SPLIT = SPLIT_RES && EPI == CS_EPI_RESIDUAL;
       bf16x4_t addend[ADDEND ? MT : 1][ADDEND ? NT : 1];
+      uint32_t addend_lo[SPLIT ? MT : 1][SPLIT ? NT : 1];   // the four bytes of a piece
       auto load_addend = [&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
         const int mc = min(mrow[i], p.M - 1);
@@ -523,15 +536,25 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
 #pragma unroll
         for (int j = 0; j < NT; ++j)
           addend[ADDEND ? i : 0][ADDEND ? j : 0] = *(const bf16x4_t*)(row + min(n_lane + piece_col(j), p.N - 4));
+        if constexpr (SPLIT) {
+          const uint8_t* row_lo = p.residual_lo + (int64_t)mc * p.ldr;
+#pragma unroll
+          for (int j = 0; j < NT; ++j)
+            addend_lo[SPLIT ? i : 0][SPLIT ? j : 0] = p.residual_lo ? *(const uint32_t*)(row_lo + min(n_lane + piece_col(j), p.N - 4)) : 0u;
+        }
       };
       // The kernel must stay inside the architectural registers (the accumulation registers are not the
-      // compiler's to use), so the addend rows are fetched in two batches.
-      constexpr int ADD_BATCH = MT / 2;
-      if constexpr (ADDEND) static_for<ADD_BATCH>(load_addend);
+      // compiler's to use), so the addend rows are fetched in batches, the first ahead of the accumulator reads, every
+      // later one right before its rows: two batches normally, row by row where the split stream's three registers
+      // per piece meet the fp8 scales.
+      constexpr int ADD_BATCH = (SPLIT && W_FP8 && MT >= 8) ? 1 : MT / 2;
+      auto load_addend_batch = [&](auto b_c) {
+        static_for<ADD_BATCH>([&](auto k_c) { load_addend(ic<decltype(b_c)::value * ADD_BATCH + decltype(k_c)::value>{}); });
+      };
+      if constexpr (ADDEND) load_addend_batch(ic<0>{});
       static_for<MT>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
-        if constexpr (ADDEND && i == ADD_BATCH)
-          static_for<MT - ADD_BATCH>([&](auto k_c) { load_addend(ic<ADD_BATCH + decltype(k_c)::value>{}); });
+        if constexpr (ADDEND && i % ADD_BATCH == 0 && i > 0) load_addend_batch(ic<i / ADD_BATCH>{});
         const bool mok = mrow[i] < p.M;
         f32x4_t racc[NT];
         static_for<NT * 4>([&](auto e_c) {
@@ -541,6 +564,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           racc[E / 4][E % 4] = t;
         });
         bf16x4_t out[NT];
+        uint32_t out_lo[SPLIT ? NT : 1];
 #pragma unroll
         for (int j = 0; j < NT; ++j) {
           float v[4];
@@ -569,12 +593,19 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
             } else if (EPI == CS_EPI_QUICK_GELU) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] = quick_gelu(rbf(v[r]));
-            } else if (ADDEND) {
+            } else if (ADDEND && !SPLIT) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] = rbf(v[r]) + bf2f(addend[ADDEND ? i : 0][ADDEND ? j : 0][r]);
             }
+            if constexpr (SPLIT) {
+              u32x2_t hi_words;
+              add_split24(v, __builtin_bit_cast(u32x2_t, addend[ADDEND ? i : 0][ADDEND ? j : 0]),
+                          addend_lo[SPLIT ? i : 0][SPLIT ? j : 0], hi_words, out_lo[SPLIT ? j : 0]);
+              out[j] = __builtin_bit_cast(bf16x4_t, hi_words);
+            } else {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
+              for (int r = 0; r < 4; ++r) out[j][r] = f2bf(v[r]);
+            }
           }
         }
         if constexpr (FUSE == FUSE_SUMSQ_C || FUSE == FUSE_STATS_C) {
@@ -639,6 +670,22 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
             for (int j = 0; j < NT; ++j)
               if (mok && n_lane + piece_col(j) < p.N) *(bf16x4_t*)(dst + piece_col(j)) = out[j];
           }
+          if constexpr (SPLIT) {
+            uint8_t* dst_lo = p.c_lo + (int64_t)crow[i] * p.ldc + n_lane;
+            if constexpr (G == 2) {
+#pragma unroll
+              for (int j = 0; j < NT; j += 2) {
+                if (mok && n_lane + piece_col(j) < p.N) {
+                  u32x2_t o = {out_lo[SPLIT ? j : 0], out_lo[SPLIT ? j + 1 : 0]};
+                  *(u32x2_t*)(dst_lo + piece_col(j)) = o;
+                }
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < NT; ++j)
+                if (mok && n_lane + piece_col(j) < p.N) *(uint32_t*)(dst_lo + piece_col(j)) = out_lo[SPLIT ? j : 0];
+            }
+          }
         }
       });
     }
@@ -650,14 +697,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   }
 }
 
-template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE = 0>
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE = 0, bool SPLIT_RES = false>
 int launch(const CsGemmArgs& a, hipStream_t stream) {
   CsGemmArgs p = a;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   constexpr int lds = RingShape<BM, BN, W_FP8>::BYTES;
   static bool attr_set = false;
-  auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE>;
+  auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE, SPLIT_RES>;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return CS_ERR_LAUNCH;
@@ -690,7 +737,9 @@ int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
     if (a.c_row_sum) {   // ... and behind it: sums and sums of squares of the output rows
       if (!a.c_row_sumsq || a.pos) return CS_ERR_UNSUPPORTED;
       if constexpr (BN == 160 && WAVES_N == 1) {
-        if (a.epilogue == CS_EPI_RESIDUAL) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_STATS_C>(a, s);
+        if (a.epilogue == CS_EPI_RESIDUAL)
+          return a.c_lo ? launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_STATS_C, true>(a, s)
+                        : launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_STATS_C>(a, s);
       }
       return CS_ERR_UNSUPPORTED;
     }
@@ -702,7 +751,9 @@ int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
     }
     if (a.c_row_sumsq) {
       if constexpr (BN == 160 && WAVES_N == 1) {
-        if (a.epilogue == CS_EPI_RESIDUAL) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_SUMSQ_C>(a, s);
+        if (a.epilogue == CS_EPI_RESIDUAL)
+          return a.c_lo ? launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_SUMSQ_C, true>(a, s)
+                        : launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, false, FUSE_SUMSQ_C>(a, s);
         if (a.epilogue == CS_EPI_BIAS && !a.pos) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, false, FUSE_SUMSQ_C>(a, s);
       }
       return CS_ERR_UNSUPPORTED;
@@ -716,7 +767,9 @@ int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
         if (a.pos) return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS_POS, false>(a, s);
       }
       return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_BIAS, W_FP8>(a, s);
-    case CS_EPI_RESIDUAL: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, W_FP8>(a, s);
+    case CS_EPI_RESIDUAL:
+      return a.c_lo ? launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, W_FP8, 0, true>(a, s)
+                    : launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, W_FP8>(a, s);
     case CS_EPI_SWIGLU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_SWIGLU, W_FP8>(a, s);
     case CS_EPI_GELU_ERF:
       if constexpr (W_FP8 && BN == 160) return CS_ERR_UNSUPPORTED;  // never dispatched, see cs_gemm_fast

@@ -17,7 +17,7 @@ CS_ERR_INVALID_ARG = 1
 CS_ERR_UNSUPPORTED = 2
 CS_ERR_LAUNCH = 3
 CS_ERR_TOO_LARGE = 4
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH, EPI_QUICK_GELU = range(6)
 
@@ -54,6 +54,8 @@ class CsGemmArgs(ctypes.Structure):
         ("a_row_sum", c_void_p),
         ("c_row_sum", c_void_p),
         ("w_col_sum", c_void_p),
+        ("residual_lo", c_void_p),
+        ("c_lo", c_void_p),
     ]
 
 

@@ -94,8 +94,15 @@ def gemm(
     a_row_sum: torch.Tensor | None = None,
     c_row_sum: torch.Tensor | None = None,
     w_col_sum: torch.Tensor | None = None,
+    residual_lo: torch.Tensor | None = None,
+    out_lo: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`.
+
+    `out_lo` (uint8, shaped and strided like `out`; EPI_RESIDUAL only) carries the residual stream with 16
+    significant bits: the sum is not rounded to bf16 but split into `out` (the leading 16 bits) and `out_lo` (the
+    next 8 as a signed correction); `residual_lo` is the same plane of the addend (None: the addend is `residual`
+    exactly).  A zero-filled plane next to any bf16 tensor is a valid pair.
 
     `a_row_sumsq` (fp32 [M, SUMSQ_PARTS]) scales row m of the product by rsqrt(sum(parts)/K + norm_eps): an
     RMSNorm of `a` whose weight the caller has folded into the columns of `w`.  `c_row_sumsq` (same layout,
@@ -111,14 +118,59 @@ def gemm(
         _req(w, torch.bfloat16, "w")
     elif w_scale is None:
         raise ValueError("fp8 weights need w_scale")
+    for name, t in (("a_rows", a_rows), ("c_rows", c_rows)):
+        if t is not None:
+            _req(t, torch.int32, name)
+            if t.dim() != 1 or not t.is_contiguous():
+                raise ValueError(f"{name} must be a contiguous int32 vector")
     M = a.shape[0] if a_rows is None else a_rows.shape[0]
     K = a.shape[1] if k is None else k
     N = w.shape[0]
+    if K > a.shape[1] or K < 1:
+        raise ValueError(f"k={K} exceeds the {a.shape[1]} columns of a")
     if w.shape[1] < K:
         raise ValueError(f"w has {w.shape[1]} columns, need at least K={K}")
+    if c_rows is not None and c_rows.shape[0] < M:
+        raise ValueError(f"c_rows has {c_rows.shape[0]} entries for {M} output rows")
     n_out = N // 2 if epilogue == EPI_SWIGLU else N
-    if out is None:
+    if out is None:  # (with c_rows: a permutation of the M rows; anything else needs the caller's `out`)
         out = torch.empty((M, n_out), dtype=torch.bfloat16, device=a.device)
+    # Everything below reaches the kernel as a raw pointer: shapes, dtypes and devices are checked here, before
+    # anything is enqueued, because an undersized or mistyped buffer would be an out-of-bounds device access.
+    _req(out, torch.bfloat16, "out")
+    if out.dim() != 2 or out.shape[1] < n_out or (c_rows is None and out.shape[0] < M):
+        raise ValueError(f"out must be bf16 [>={M}, >={n_out}], got {tuple(out.shape)}")
+    if bias is not None:
+        _req(bias, torch.bfloat16, "bias")
+        if bias.dim() != 1 or bias.shape[0] < N:
+            raise ValueError(f"bias must be bf16 [{N}], got {tuple(bias.shape)}")
+    if epilogue == EPI_RESIDUAL and residual is None:
+        raise ValueError("EPI_RESIDUAL needs `residual`")
+    if residual is not None:
+        _req(residual, torch.bfloat16, "residual")
+        if residual.dim() != 2 or residual.shape[0] < M or residual.shape[1] < N:
+            raise ValueError(f"residual must be bf16 [>={M}, >={N}], got {tuple(residual.shape)}")
+    if pos is not None:
+        _req(pos, torch.bfloat16, "pos")
+        if pos.dim() != 2 or pos.shape[0] < 1 or pos.shape[1] < N:
+            raise ValueError(f"pos must be bf16 [period, >={N}], got {tuple(pos.shape)}")
+    if w_scale is not None:
+        _req(w_scale, torch.float32, "w_scale")
+        if w_scale.dim() != 1 or w_scale.shape[0] < N or not w_scale.is_contiguous():
+            raise ValueError(f"w_scale must be a contiguous fp32 [{N}] tensor")
+    if residual_lo is not None or out_lo is not None:
+        if epilogue != EPI_RESIDUAL or out_lo is None:
+            raise ValueError("residual_lo / out_lo belong to EPI_RESIDUAL, and residual_lo needs out_lo")
+        _req(out_lo, torch.uint8, "out_lo")
+        if out_lo.shape != out.shape or out_lo.stride() != out.stride():
+            raise ValueError("out_lo must have the shape and strides of out")
+        if residual_lo is not None:
+            _req(residual_lo, torch.uint8, "residual_lo")
+            if residual_lo.shape != residual.shape or residual_lo.stride() != residual.stride():
+                raise ValueError("residual_lo must have the shape and strides of residual")
+    on = {t.device for t in (a, w, out, bias, residual, pos, w_scale, a_rows, c_rows, residual_lo, out_lo) if t is not None}
+    if len(on) != 1:
+        raise ValueError(f"gemm operands live on different devices: {sorted(map(str, on))}")
     args = _l.CsGemmArgs()
     args.A, args.lda = a.data_ptr(), a.stride(0)
     args.W, args.ldw = w.data_ptr(), w.stride(0)
@@ -151,6 +203,8 @@ def gemm(
     args.a_row_sum = _ptr(a_row_sum)
     args.c_row_sum = _ptr(c_row_sum)
     args.w_col_sum = _ptr(w_col_sum)
+    args.residual_lo = _ptr(residual_lo)
+    args.c_lo = _ptr(out_lo)
     _l.check(lib.cs_gemm(ctypes.byref(args), _stream()), "cs_gemm")
     return out
 

@@ -36,7 +36,7 @@ extern "C" {
 #define CS_ERR_TOO_LARGE 4
 
 /* ABI version of this header; cs_abi_version() returns the value the library was built with. */
-#define CS_ABI_VERSION 3
+#define CS_ABI_VERSION 4
 int cs_abi_version(void);
 
 /* ------------------------------------------------------------------------------------------------
@@ -48,7 +48,8 @@ int cs_abi_version(void);
  * ---------------------------------------------------------------------------------------------- */
 enum CsEpilogue {
   CS_EPI_BIAS = 0,      /* y = acc (+ bias)                                                     */
-  CS_EPI_RESIDUAL = 1,  /* y = bf16(acc + bias) + residual[m,n]         qwen2_5_vl.py:175,177   */
+  CS_EPI_RESIDUAL = 1,  /* y = bf16(acc + bias) + residual[m,n]         qwen2_5_vl.py:175,177
+                           (with c_lo: y = acc + bias + residual, kept to 16 significant bits)  */
   CS_EPI_SWIGLU = 2,    /* W rows interleaved gate_j,up_j; y[m,j] = silu(g)*u; C is N/2 wide
                            qwen2_5_vl.py:143-148                                               */
   CS_EPI_GELU_ERF = 3,  /* y = gelu(acc + bias), erf form               qwen2_5_vl.py:220       */
@@ -101,6 +102,18 @@ typedef struct CsGemmArgs {
   const float* a_row_sum;
   float* c_row_sum;
   const float* w_col_sum;
+  /* Residual stream with 16 significant bits (CS_EPI_RESIDUAL only).  The residual additions at qwen2_5_vl.py:175,177
+   * (siglip.py:178,188) are the one place where a bf16 encoder accumulates rounding error with depth: 64 roundings of
+   * the stream to 8 bits.  With these planes the stream is carried as a bf16 "hi" tensor (C / residual, which is what
+   * every other kernel reads) plus a byte "lo" tensor with the next 8 mantissa bits as a signed correction:
+   *   value = fp32 from bits  (hi << 16) + ((int8)lo << 8)
+   * residual_lo: optional uint8 [M,N], leading dimension ldr; the addend is the joined value instead of bf16 residual.
+   * c_lo:        optional uint8 [M,N], leading dimension ldc (rows scattered like C's); the sum acc + bias + addend is
+   *              not rounded to bf16 on the way (neither is acc + bias) but split: 24 bits to nearest, the upper 16 of
+   *              them rounded half-up to C, the rest to c_lo.  A zero-filled plane next to a bf16 tensor is a valid
+   *              pair, so the stream can start from any bf16 tensor.  May alias residual_lo when C aliases residual. */
+  const uint8_t* residual_lo;
+  uint8_t* c_lo;
 } CsGemmArgs;
 #define CS_SUMSQ_PARTS 8
 

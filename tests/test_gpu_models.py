@@ -171,8 +171,7 @@ def test_full_size_configs_through_properties(dev):
     """The benchmark configurations at their full size (32 blocks, full attention at 7/15/23/31), where the CPU oracle
     is too slow for the whole batch, through properties that do not depend on the size: an item's embedding is the
     same bits alone and in the batch, a permuted batch gives permuted outputs, equal items give equal outputs; and
-    one image of the batch against the oracle, with the distance of the reference's own bf16 arithmetic to the fp32
-    result as the yardstick (at 64 residual additions in bf16 that distance itself is about the 2e-2 bar)."""
+    config 2 -- all 8 images, 32 blocks -- against the fp32 oracle at the stated tolerance."""
     full = (7, 15, 23, 31)
     model, sd, ocfg = build_qwen(dev, 32, full, seed=21)
 
@@ -191,17 +190,20 @@ def test_full_size_configs_through_properties(dev):
     alone = run([px[5]], [grid[5]])[0]
     assert torch.equal(alone, out[5]), "an item alone equals the item in the batch"
     assert not torch.equal(out[0], out[1])
+    # the whole batch against the fp32 oracle on the same bf16-rounded weights and inputs, at the flat bar: the
+    # residual stream carries 16 significant bits, so 64 residual additions do not use up the tolerance (the
+    # reference's bf16 arithmetic, restated step by step, sits at about 2.3e-2 from the same fp32 result)
     sd16 = {k: v.bfloat16() for k, v in sd.items()}
     sd32 = {k: v.float() for k, v in sd16.items()}
-    px5 = px[5].bfloat16()
-    ref16 = oq.forward(sd16, ocfg, [px5], [grid[5]], dtype=torch.bfloat16)[0].float()
-    ref32 = oq.forward(sd32, ocfg, [px5.float()], [grid[5]], dtype=torch.float32)[0]
-    got = out[5].float().cpu()
+    ref32 = torch.cat(oq.forward(sd32, ocfg, [p.bfloat16().float() for p in px], grid, dtype=torch.float32))
+    got = torch.cat(out).float().cpu()
     dist = lambda a, b: ((a - b).abs().max() / b.abs().max()).item()
     cos = lambda a, b: F.cosine_similarity(a.flatten(), b.flatten(), dim=0).item()
-    assert cos(got, ref32) >= COS_MIN and cos(got, ref16) >= COS_MIN
-    yard = dist(ref16, ref32)
-    assert dist(got, ref32) <= max(REL_BF16, 1.25 * yard), (dist(got, ref32), yard)
+    assert cos(got, ref32) >= COS_MIN and dist(got, ref32) <= REL_BF16, (cos(got, ref32), dist(got, ref32))
+    for o, r in zip(out, ref32.split(256)):     # ... and every image on its own scale
+        assert dist(o.float().cpu(), r) <= REL_BF16
+    ref16 = oq.forward(sd16, ocfg, [px[5].bfloat16()], [grid[5]], dtype=torch.bfloat16)[0].float()
+    assert cos(out[5].float().cpu(), ref16) >= COS_MIN
 
     # config 4: 16 images with sides drawn from the multiples of 28 in [224, 1344]
     grids = synth.ragged_grids(16, seed=4)

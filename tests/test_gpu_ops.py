@@ -492,6 +492,105 @@ def test_gemm_rejects_bad_shapes(ops, dev):
         ops.gemm(a.float(), w, None)
 
 
+def test_gemm_rejects_mistyped_or_undersized_buffers(ops, dev):
+    """Every buffer reaches the kernel as a raw pointer, so the wrapper refuses what the kernel would read or write
+    out of bounds -- before anything is enqueued."""
+    M, N, K = 64, 128, 64
+    a, w, b = rnd((M, K), dev=dev), rnd((N, K), dev=dev), rnd((N,), dev=dev)
+    res = rnd((M, N), dev=dev)
+    rows64 = torch.arange(M, device=dev)                       # int64, as get_window_index returns it
+    bad = [
+        dict(a_rows=rows64),
+        dict(c_rows=rows64),
+        dict(c_rows=torch.arange(M - 1, device=dev, dtype=torch.int32)),
+        dict(out=torch.empty((M, N), dtype=torch.float16, device=dev)),
+        dict(out=torch.empty((M - 1, N), dtype=torch.bfloat16, device=dev)),
+        dict(out=torch.empty((M, N - 8), dtype=torch.bfloat16, device=dev)),
+        dict(out=torch.empty((M, N), dtype=torch.bfloat16)),   # host tensor
+        dict(k=K + 8),
+        dict(epilogue=ops.EPI_RESIDUAL),                          # no residual
+        dict(epilogue=ops.EPI_RESIDUAL, residual=res[:, : N - 8]),
+        dict(epilogue=ops.EPI_RESIDUAL, residual=res[: M - 1]),
+        dict(epilogue=ops.EPI_RESIDUAL, residual=res.float()),
+        dict(pos=rnd((4, N - 8), dev=dev)),
+        dict(pos=rnd((4, N), dev=dev).float()),
+        dict(out_lo=torch.zeros((M, N), dtype=torch.uint8, device=dev)),   # not the residual epilogue
+        dict(epilogue=ops.EPI_RESIDUAL, residual=res, residual_lo=torch.zeros((M, N), dtype=torch.uint8, device=dev)),
+        dict(epilogue=ops.EPI_RESIDUAL, residual=res, out=torch.empty_like(res),
+             out_lo=torch.zeros((M, N), dtype=torch.int8, device=dev)),
+        dict(epilogue=ops.EPI_RESIDUAL, residual=res, out=torch.empty_like(res),
+             out_lo=torch.zeros((M, N + 8), dtype=torch.uint8, device=dev)),
+    ]
+    for kw in bad:
+        with pytest.raises(ValueError):
+            ops.gemm(a, w, b, **kw)
+    for bias in (b.float(), b[: N - 8], b[None]):
+        with pytest.raises(ValueError):
+            ops.gemm(a, w, bias)
+    with pytest.raises(ValueError):
+        ops.gemm(a, w.to(torch.float8_e4m3fn), b, w_scale=torch.ones(N - 1, device=dev))
+    torch.cuda.synchronize()
+    assert torch.isfinite(ops.gemm(a, w, b).float()).all()    # the device is still healthy
+
+
+def _join24(hi: torch.Tensor, lo: torch.Tensor) -> torch.Tensor:
+    """The value a (bf16 plane, byte plane) pair stands for: fp32 from the bits (hi << 16) + (int8(lo) << 8)."""
+    h = hi.cpu().view(torch.int16).to(torch.int32) << 16
+    l = lo.cpu().view(torch.int8).to(torch.int32) << 8
+    return (h + l).view(torch.float32)
+
+
+# The residual stream with 16 significant bits, in every kernel that has the residual epilogue: the 160-column forms
+# that also emit row sums (as the encoder blocks call them), the plain fast forms, fp8 weights, the general kernel.
+@pytest.mark.parametrize("M,N,K,form", [
+    (8192, 1280, 192, "sumsq"), (1000, 1280, 320, "sumsq"), (300, 1152, 448, "stats"), (8192, 2304, 256, "plain"),
+    (300, 520, 448, "plain"), (777, 1280, 256, "fp8"), (515, 1280, 72, "general"),
+])
+def test_gemm_split_residual(ops, dev, M, N, K, form):
+    a, b = rnd((M, K), 1.0, 51, dev), rnd((N,), 0.02, 53, dev)
+    w = rnd((N, K), 0.05, 52, dev)
+    kw, wf = {}, w.float().cpu()
+    if form == "fp8":
+        q, s = w.to(torch.float8_e4m3fn), torch.full((N,), 0.5, device=dev)
+        wf, w, kw = q.float().cpu() * 0.5, q, dict(w_scale=s)
+    res = rnd((M, N), 3.0, 54, dev)
+    res_lo = torch.randint(0, 256, (M, N), generator=torch.Generator().manual_seed(55), dtype=torch.uint8).to(dev)
+    ss = torch.zeros((M, 8), dtype=torch.float32, device=dev)
+    sm = torch.zeros_like(ss)
+    if form == "sumsq":
+        kw["c_row_sumsq"] = ss
+    if form == "stats":
+        kw.update(c_row_sumsq=ss, c_row_sum=sm)
+    rows = torch.cat([torch.arange(0, M, max(1, M // 199)), torch.tensor([M - 1])])
+    exact = a.float().cpu()[rows] @ wf.t() + b.float().cpu()             # fp32, no rounding anywhere
+    for lo_in in (res_lo, None):
+        out, out_lo = torch.empty_like(res), torch.full((M, N), 0xAB, dtype=torch.uint8, device=dev)
+        ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res, residual_lo=lo_in, out=out, out_lo=out_lo, **kw)
+        addend = _join24(res, lo_in) if lo_in is not None else res.float().cpu()
+        want = exact + addend[rows]
+        got = _join24(out, out_lo)[rows]
+        # 2^-17 of the value from the split, plus the accumulation-order noise of an fp32 dot product
+        assert (got - want).abs().max().item() <= want.abs().max().item() * 2.0**-16, (form, (got - want).abs().max().item())
+        # the bf16 plane alone is the value rounded to bf16 (half an ulp; a bf16 ulp is at most 2^-7 of the value)
+        assert ((out.float().cpu()[rows] - got).abs() <= got.abs() * 2.0**-8 + 1e-30).all()
+        if form in ("sumsq", "stats"):
+            parts = (N + 159) // 160
+            torch.testing.assert_close(ss.cpu()[:, :parts], _sumsq_parts_ref(out)[:, :parts], rtol=1e-5, atol=1e-6)
+    # a zero byte plane is "the bf16 value exactly": the addend equals the plain residual
+    assert torch.equal(_join24(res, torch.zeros_like(res_lo)), res.float().cpu())
+    # in place, 64 times: the stream follows the exact sum to 16 bits where a bf16 stream drifts by 2^-9 per addition
+    x, x_lo = res.clone(), torch.zeros_like(res_lo)
+    xb = res.clone()
+    for _ in range(64):
+        ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=x, residual_lo=x_lo, out=x, out_lo=x_lo, **kw)
+        ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=xb, out=xb, **kw)
+    want = res.float().cpu()[rows] + 64.0 * exact
+    err_split = (_join24(x, x_lo)[rows] - want).abs().max().item()
+    err_bf16 = (xb.float().cpu()[rows] - want).abs().max().item()
+    top = want.abs().max().item()
+    assert err_split <= 64 * top * 2.0**-16 and err_split < err_bf16 / 16, (err_split, err_bf16, top)
+
+
 # --------------------------------------------------------------------------------------- attention
 def attn_ref(qkv, cu, nh, d, cos_sin=None):
     L = qkv.shape[0]
