@@ -154,6 +154,8 @@ class SiglipEncoderBase(EricModel):
     """What the encoders built on the SigLIP tower share: the packed weights and the tower's launch sequence.
     A subclass sets `self.config` (with `.vision_config`), `self.vision_tower` (a SiglipVisionModel) and calls
     `_init_tower(fold_norm)`."""
+    # the residual stream (siglip.py:178,188) is carried with 16 significant bits, as in Qwen2_5_VisionTransformer
+    split_residual: bool = True
 
     def _init_tower(self, fold_norm: bool) -> None:
         vc = self.config.vision_config
@@ -258,6 +260,9 @@ class SiglipEncoderBase(EricModel):
             raise NotImplementedError(f"Activation function {act!r} is not implemented.")
         fold = self.fold_norm
         stats_out = {}
+        if self.split_residual:   # the byte plane of the residual stream (see Qwen2_5_VisionTransformer); zero = "x is exact"
+            lo = torch.zeros(x.shape, dtype=torch.uint8, device=x.device)
+            stats_out = {"residual_lo": lo, "out_lo": lo}
         if fold:
             if M * max(3 * H, pk["ip"]) * 2 >= 2**32:
                 raise ValueError(f"{M} tokens in one forward exceed what the folded-norm GEMMs address; split the batch "
@@ -265,7 +270,7 @@ class SiglipEncoderBase(EricModel):
             ss = torch.zeros((M, ops.SUMSQ_PARTS), dtype=torch.float32, device=x.device)
             sm = torch.zeros_like(ss)
             ops.row_stats(x, ss, sm)
-            stats_out = {"c_row_sumsq": ss, "c_row_sum": sm}
+            stats_out.update(c_row_sumsq=ss, c_row_sum=sm)
         for lyr in pk["layers"]:
             if fold:
                 ops.gemm(x, lyr["qkv_w"], lyr["qkv_b"], out=qkv, a_row_sumsq=ss, a_row_sum=sm,

@@ -118,6 +118,8 @@ class QwenVisionBase(EricModel):
 
     # what the checkpoint's image processor normalises with (preprocessor_config.json): CLIP statistics for
     # Qwen2-VL and Qwen2.5-VL; subclasses override
+    # carry the residual stream with 16 significant bits (see Qwen2_5_VisionTransformer.__init__)
+    split_residual: bool = True
     image_mean: tuple = frame_ops.CLIP_MEAN
     image_std: tuple = frame_ops.CLIP_STD
 

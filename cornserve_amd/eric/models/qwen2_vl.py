@@ -157,6 +157,10 @@ class Qwen2VisionTransformer(QwenVisionBase):
         hmid = torch.empty((L, self.mlp_hidden), dtype=torch.bfloat16, device=dev)
         scale = d**-0.5
         fold = self.fold_norm
+        res = {}
+        if self.split_residual:   # the byte plane of the residual stream; zero = "x is exact"
+            lo = torch.zeros(x.shape, dtype=torch.uint8, device=dev)
+            res = {"residual_lo": lo, "out_lo": lo}
         if fold:
             if L * max(3 * E, self.mlp_hidden) * 2 >= 2**32:
                 raise ValueError(f"{L} patches in one forward exceed what the folded-norm GEMMs address; split the batch "
@@ -179,7 +183,7 @@ class Qwen2VisionTransformer(QwenVisionBase):
             mark("attn_full")
             ops.attn_varlen_rotary_(qkv, plan, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")
-            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **(stats_out if fold else {}))
+            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **res, **(stats_out if fold else {}))
             if fold:
                 mark("gemm_fc1")
                 ops.gemm(x, b["fc1"]["w"], b["fc1"]["b"], epilogue=ops.EPI_QUICK_GELU, out=hmid, **stats_in(b["fc1"]))
@@ -189,7 +193,7 @@ class Qwen2VisionTransformer(QwenVisionBase):
                 mark("gemm_fc1")
                 self._g(n, b["fc1"], epilogue=ops.EPI_QUICK_GELU, out=hmid)
             mark("gemm_fc2")
-            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **(stats_out if fold else {}))
+            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **res, **(stats_out if fold else {}))
         mark("norm")
         ops.layernorm(x, *pk["ln_q"], eps, out=n)
         mark("gemm_merger")

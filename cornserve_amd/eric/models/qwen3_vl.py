@@ -229,6 +229,9 @@ class Qwen3_VisionTransformer(QwenVisionBase):
             stats_out = {"c_row_sumsq": ss, "c_row_sum": sm}
         else:
             stats_out = {}
+        if self.split_residual:   # the byte plane of the residual stream; zero = "x is exact".  It is updated in place
+            lo = torch.zeros(x.shape, dtype=torch.uint8, device=dev)   # even when the bf16 plane moves to a new buffer
+            stats_out = dict(stats_out, residual_lo=lo, out_lo=lo)
         for i, b in enumerate(pk["blocks"]):
             if fold:
                 mark("gemm_qkv")

@@ -521,8 +521,8 @@ def test_gemma3_real_resolution_and_crops(dev):
 
 def test_gemma3_full_size_through_properties(dev):
     """Config 3 at its full size (27 layers, four 896 x 896 images): a permuted batch gives permuted outputs, an
-    image alone equals the image in the batch (bit for bit), and one image against the oracle with the distance of
-    the bf16 oracle to the fp32 oracle as the yardstick."""
+    image alone equals the image in the batch (bit for bit), and every image against the fp32 oracle at the stated
+    tolerance."""
     model, sd, ocfg = build_gemma(dev, 27, 896, 2560, 256, seed=31)
     px = [synth.uniform(31, f"img{i}", (1, 3, 896, 896), -1, 1) for i in range(4)]
     crops = [torch.tensor([0])] * 4
@@ -533,17 +533,18 @@ def test_gemma3_full_size_through_properties(dev):
     assert all(torch.equal(out_p[j], out[i]) for j, i in enumerate(perm))
     alone = model(Modality.IMAGE, "a", {"pixel_values": [px[2]], "num_crops": [crops[2]]})[0]
     assert torch.equal(alone, out[2])
+    # the whole batch against the fp32 oracle on the same bf16-rounded weights and inputs, at the flat bar (the residual
+    # stream carries 16 significant bits; a bf16 stream sits near the bar itself after 54 residual additions)
     sd16 = {k: v.bfloat16() for k, v in sd.items()}
     sd32 = {k: v.float() for k, v in sd16.items()}
-    p2 = px[2].bfloat16()
-    ref16 = og.forward(sd16, ocfg, [p2], [crops[2]], dtype=torch.bfloat16)[0].float()
-    ref32 = og.forward(sd32, ocfg, [p2.float()], [crops[2]], dtype=torch.float32)[0]
-    got = out[2].float().cpu()
+    ref32 = og.forward(sd32, ocfg, [p.bfloat16().float() for p in px], crops, dtype=torch.float32)
     dist = lambda a, b: ((a - b).abs().max() / b.abs().max()).item()
     cos = lambda a, b: F.cosine_similarity(a.flatten(), b.flatten(), dim=0).item()
-    assert cos(got, ref32) >= COS_MIN and cos(got, ref16) >= COS_MIN
-    yard = dist(ref16, ref32)
-    assert dist(got, ref32) <= max(REL_BF16, 1.25 * yard), (dist(got, ref32), yard)
+    for o, r in zip(out, ref32):
+        o = o.float().cpu()
+        assert cos(o, r) >= COS_MIN and dist(o, r) <= REL_BF16, (cos(o, r), dist(o, r))
+    ref16 = og.forward(sd16, ocfg, [px[2].bfloat16()], [crops[2]], dtype=torch.bfloat16)[0].float()
+    assert cos(out[2].float().cpu(), ref16) >= COS_MIN
 
 
 def test_layernorm_encoders_without_folded_norms(dev):
