@@ -63,6 +63,7 @@ class CsGemmArgs(ctypes.Structure):
 _SIGNATURES: dict[str, list] = {
     "cs_abi_version": [],
     "cs_gemm": [POINTER(CsGemmArgs), c_void_p],
+    "cs_gemm_rmsnorm_noalloc": [POINTER(CsGemmArgs), c_void_p],
     "cs_row_sumsq": [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p],
     "cs_row_stats": [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
     "cs_rmsnorm": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_float, c_int32, c_void_p],

@@ -120,6 +120,18 @@ typedef struct CsGemmArgs {
 /* Constraints: K % 8 == 0 (16 with fp8), lda/ldw % 8 == 0, N % 4 == 0, A and W 16-byte aligned. */
 int cs_gemm(const CsGemmArgs* args, void* stream);
 
+/* The RMSNorm-folded form of cs_gemm without a workspace: cs_row_sumsq on A followed by cs_gemm with a_row_sumsq, the
+ * [M][CS_SUMSQ_PARTS] row sums living in a static device array of the library instead of a buffer of the caller's.
+ * No counterpart in the reference (which allocates freely through torch): this entry point is for callers that cannot
+ * allocate device memory -- code under HIP graph capture, serving loops and harnesses that forbid hipMalloc.  It
+ * allocates and frees nothing.  args as for cs_gemm, with a_row_sumsq, a_row_sum and a_rows NULL and bf16 W; K is the
+ * normalised width (<= 160 * CS_SUMSQ_PARTS); norm_eps as for cs_gemm.  M above CS_NOALLOC_MAX_ROWS (or K above that
+ * width) returns CS_ERR_TOO_LARGE.  Every GPU the library is used on holds the array (CS_NOALLOC_MAX_ROWS *
+ * CS_SUMSQ_PARTS floats = 2 MiB) until the process ends; all calls on one GPU share it, so calls that overlap on one
+ * GPU (different streams, or threads) race -- serialise them on one stream.                                          */
+#define CS_NOALLOC_MAX_ROWS 65536
+int cs_gemm_rmsnorm_noalloc(const CsGemmArgs* args, void* stream);
+
 /* ------------------------------------------------------------------------------------------------
  * Normalisation (HBM-bound, one wavefront per row).
  * ---------------------------------------------------------------------------------------------- */
