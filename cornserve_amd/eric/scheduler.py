@@ -1,18 +1,26 @@
-"""Batching of embedding requests in front of the encoder (reference: eric/engine/scheduler.py:22-190 and the batch
+"""Batching of embedding requests in front of the encoder (the policy of eric/engine/scheduler.py:133-190 and the batch
 records of eric/schema.py:20-37,62-75,140-215, without the tracing spans and the msgpack transport, which belong to
 the engine around the path).
 
-Same policy as the reference: the queue is served in arrival order, and one batch takes the waiting items at its head
-that share the first item's modality and adapter, up to `max_batch_size` items.  One addition for the kernels behind
-`Worker.execute_model`: `max_batch_patches` bounds the batch by its total patch count, because their throughput is
-flat from about 8192 patches up (every GEMM launch then fills the 256 compute units for at least one full round) while
-activation memory and latency keep growing with the batch; a batch always takes at least one item.
+Policy, as observed from outside: items are served in arrival order; one batch takes the waiting items at the head of
+the line that share the first one's modality and adapter, up to `max_batch_size` items, and a request is reported
+finished when its last item is.  Two additions for the kernels behind `Worker.execute_model`:
+
+* `max_batch_patches` bounds a batch by its total patch count: throughput is flat from about 8192 patches up (every
+  GEMM launch then fills the 256 compute units for at least one full round) while activation memory and latency keep
+  growing with the batch; a batch always takes at least one item;
+* items handed out by `schedule()` are IN FLIGHT until `process_batch_result` reports them, and a second
+  `schedule()` before that skips them: the caller can take batch k+1 (and start its upload, `Worker.upload`) while
+  batch k is still running.
+
+The book-keeping is one flat line of item slots (arrival order) plus a count of unfinished items per request.
 """
 
 from __future__ import annotations
 
-from collections import defaultdict
-from collections.abc import Callable, Generator
+from collections import deque
+from collections.abc import Callable
+from enum import Enum
 from dataclasses import dataclass, field
 
 import torch
@@ -45,9 +53,13 @@ class SchedulerBatch(WorkerBatch):
     """Items that run in one forward pass (reference: schema.py:140-215)."""
 
     def to_worker_batch(self) -> WorkerBatch:
+        """The same batch as a plain WorkerBatch.  Everything travels, including the upload event of a batch whose
+        host tensors `Worker.upload` has already sent ahead (without it the compute stream would not wait for the
+        copies).  `Worker.execute_model` and `Worker.upload` also take the SchedulerBatch itself."""
         return WorkerBatch(modality=self.modality, adapter_name=self.adapter_name, request_ids=self.request_ids,
                            data_ids=self.data_ids, chunk_ids=self.chunk_ids, num_chunks=self.num_chunks,
-                           receiver_ranks=self.receiver_ranks, data=self.data, _dump_prefix=self._dump_prefix)
+                           receiver_ranks=self.receiver_ranks, data=self.data, _dump_prefix=self._dump_prefix,
+                           _uploaded=self._uploaded)
 
     def add_data(self, request_id: str, data: list[ProcessedEmbeddingData], chunk_ids: list[int],
                  num_chunks: list[int]) -> None:
@@ -81,103 +93,101 @@ def patch_count(item: ProcessedEmbeddingData) -> int:
     return int(first.shape[0]) if first.dim() else 1
 
 
-class RequestQueue:
-    """Requests in arrival order with a done flag per item (reference: scheduler.py:22-130)."""
+class _State(Enum):
+    WAITING = 0
+    IN_FLIGHT = 1
 
-    def __init__(self) -> None:
-        self.request_id_to_request: dict[str, EngineEnqueueRequest] = {}
-        self.request_id_to_data_done: dict[str, dict[str, bool]] = defaultdict(dict)
 
-    def __len__(self) -> int:
-        return len(self.request_id_to_request)
-
-    def enqueue(self, request: EngineEnqueueRequest) -> None:
-        self.request_id_to_request[request.request_id] = request
-        for data in request.data:
-            self.request_id_to_data_done[request.request_id][data.id] = False
-
-    def mark_done(self, request_ids: list[str], data_ids: list[str]) -> list[str]:
-        """Flag the items as done; returns (and forgets) the requests whose items are all done."""
-        assert len(request_ids) == len(data_ids)
-        for request_id, data_id in zip(request_ids, data_ids):
-            self.request_id_to_data_done[request_id][data_id] = True
-        finished = []
-        for request_id in dict.fromkeys(request_ids):
-            if all(self.request_id_to_data_done[request_id].values()):
-                finished.append(request_id)
-                del self.request_id_to_request[request_id]
-                del self.request_id_to_data_done[request_id]
-        return finished
-
-    def is_done(self, request_id: str, data_id: str | None = None) -> bool:
-        if request_id not in self.request_id_to_request:
-            return True
-        if data_id is None:
-            return False
-        return self.request_id_to_data_done[request_id][data_id]
-
-    def peek_request(self) -> EngineEnqueueRequest:
-        assert self.request_id_to_request, "Queue is empty"
-        return next(iter(self.request_id_to_request.values()))
-
-    def peek_data(self) -> ProcessedEmbeddingData:
-        request = self.peek_request()
-        assert request.data, "Request has no data"
-        for data in request.data:
-            if not self.is_done(request.request_id, data.id):
-                return data
-        raise ValueError("No waiting data in a waiting request")
-
-    def iter_waiting(self, modality: Modality, model_id: str, max_items: int | None = None,
-                     ) -> Generator[tuple[EngineEnqueueRequest, ProcessedEmbeddingData], None, None]:
-        """Waiting items from the head of the queue until the modality or the adapter changes."""
-        count = 0
-        for request in self.request_id_to_request.values():
-            for data in request.data:
-                if self.is_done(request.request_id, data.id):
-                    continue
-                if data.modality != modality or data.model_id != model_id:
-                    return
-                yield request, data
-                count += 1
-                if count == max_items:
-                    return
+@dataclass
+class _Slot:
+    request_id: str
+    item: ProcessedEmbeddingData
+    state: _State = _State.WAITING
 
 
 class Scheduler:
-    """Reference: scheduler.py:133-190."""
+    """Arrival-order batching with a patch budget and in-flight tracking (policy of scheduler.py:133-190)."""
 
     def __init__(self, max_batch_size: int | None = None, max_batch_patches: int | None = None,
                  count_patches: Callable[[ProcessedEmbeddingData], int] = patch_count) -> None:
         if max_batch_patches is not None and max_batch_patches < 1:
             raise ValueError("max_batch_patches must be positive")
+        if max_batch_size is not None and max_batch_size < 1:
+            raise ValueError("max_batch_size must be positive")
         self.max_batch_size = max_batch_size
         self.max_batch_patches = max_batch_patches
         self.count_patches = count_patches
-        self.queue = RequestQueue()
+        self._line: deque[_Slot] = deque()            # unfinished items, arrival order
+        self._open: dict[str, int] = {}               # request id -> items not yet reported done
+        self._slot_of: dict[tuple[str, str], _Slot] = {}
 
+    # ------------------------------------------------------------------ intake
     def enqueue(self, request: EngineEnqueueRequest) -> None:
-        self.queue.enqueue(request)
+        if request.request_id in self._open:
+            raise ValueError(f"request {request.request_id} is already queued")
+        if not request.data:
+            raise ValueError(f"request {request.request_id} has no data")
+        seen = set()
+        for item in request.data:
+            if item.id in seen:
+                raise ValueError(f"request {request.request_id} lists data id {item.id} twice")
+            seen.add(item.id)
+        self._open[request.request_id] = len(request.data)
+        for item in request.data:
+            slot = _Slot(request.request_id, item)
+            self._line.append(slot)
+            self._slot_of[(request.request_id, item.id)] = slot
 
     def has_waiting_requests(self) -> bool:
-        return len(self.queue) > 0
+        """Requests that are not finished yet (waiting or in flight), as the reference's method counts them."""
+        return bool(self._open)
 
+    def has_schedulable_items(self) -> bool:
+        """Items that a `schedule()` call could take right now (everything else is in flight)."""
+        return any(slot.state is _State.WAITING for slot in self._line)
+
+    # ------------------------------------------------------------------ batching
     def schedule(self) -> SchedulerBatch:
-        """The next batch; only called while requests are waiting."""
-        head = self.queue.peek_data()
-        batch = SchedulerBatch(modality=head.modality, adapter_name=head.model_id)
+        """The next batch; its items are in flight until `process_batch_result` names them."""
+        batch: SchedulerBatch | None = None
         patches = 0
-        for req, data in self.queue.iter_waiting(modality=head.modality, model_id=head.model_id,
-                                                 max_items=self.max_batch_size):
+        for slot in self._line:
+            if slot.state is not _State.WAITING:
+                continue
+            item = slot.item
+            if batch is None:
+                batch = SchedulerBatch(modality=item.modality, adapter_name=item.model_id)
+            elif item.modality != batch.modality or item.model_id != batch.adapter_name:
+                break                                   # the line is served in order: no overtaking
             if self.max_batch_patches is not None:
-                n = self.count_patches(data)
+                n = self.count_patches(item)
                 if len(batch) > 0 and patches + n > self.max_batch_patches:
                     break
                 patches += n
-            batch.add_data(request_id=req.request_id, data=[data], chunk_ids=[0], num_chunks=[1])
-        assert batch.request_ids, "Batch should not be empty"
+            batch.add_data(request_id=slot.request_id, data=[item], chunk_ids=[0], num_chunks=[1])
+            slot.state = _State.IN_FLIGHT
+            if self.max_batch_size is not None and len(batch) == self.max_batch_size:
+                break
+        if batch is None:
+            raise RuntimeError("nothing to schedule: the queue is empty or every item is in flight")
         return batch
 
     def process_batch_result(self, request_ids: list[str], data_ids: list[str]) -> list[str]:
-        """Returns the requests that are completely done."""
-        return self.queue.mark_done(request_ids, data_ids)
+        """Report items as done.  Returns the requests whose last item this was, in the order given."""
+        if len(request_ids) != len(data_ids):
+            raise ValueError("request_ids and data_ids must have one entry per item")
+        finished: list[str] = []
+        for key in zip(request_ids, data_ids):
+            slot = self._slot_of.pop(key, None)
+            if slot is None:
+                raise KeyError(f"item {key[1]} of request {key[0]} is not queued (reported twice?)")
+            slot.state = None                          # finished: dropped from the line below
+            self._open[key[0]] -= 1
+            if self._open[key[0]] == 0:
+                del self._open[key[0]]
+                finished.append(key[0])
+        while self._line and self._line[0].state is None:
+            self._line.popleft()
+        if len(self._line) > 4 * len(self._slot_of) + 16:   # finished items stuck behind an unfinished head
+            self._line = deque(slot for slot in self._line if slot.state is not None)
+        return finished

@@ -227,6 +227,39 @@ def test_full_size_configs_through_properties(dev):
     assert torch.equal(twice[0], twice[1]) and torch.equal(twice[0], out[1]), "equal clips give equal embeddings"
 
 
+def test_scheduler_upload_ahead_pipeline(dev):
+    """The pipelined loop: batch k+1 is taken from the scheduler and its host tensors sent ahead on the side stream
+    while batch k is still queued on the device; the upload event survives `to_worker_batch`, and every embedding
+    equals the one from a direct call."""
+    from cornserve_amd.eric import scheduler as sc
+    from cornserve_amd.eric.worker import Worker
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=15)
+    grids = [(1, 16, 16), (1, 8, 12), (2, 4, 4), (1, 12, 8), (1, 16, 20), (1, 4, 6)]
+    px, grid = synth.qwen_inputs(grids, seed=15)
+    direct = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    worker = Worker(model)
+    s = sc.Scheduler(max_batch_size=2)
+    for r in range(3):
+        s.enqueue(sc.EngineEnqueueRequest(f"r{r}", [
+            sc.ProcessedEmbeddingData(id=f"d{i}", modality=Modality.IMAGE, model_id="",
+                                      data={"pixel_values": px[i], "image_grid_thw": grid[i]}) for i in (2 * r, 2 * r + 1)]))
+    seen, finished = [], []
+    ahead = worker.upload(s.schedule())
+    assert ahead._uploaded is not None
+    while ahead is not None:
+        cur = ahead
+        ahead = worker.upload(s.schedule()) if s.has_schedulable_items() else None   # before batch k runs
+        wb = cur.to_worker_batch()
+        assert wb._uploaded is cur._uploaded and all(t.is_cuda for t in wb.data["pixel_values"])
+        out = worker.execute_model(wb)
+        for data_id, emb in zip(cur.data_ids, out):
+            assert torch.equal(emb, direct[int(data_id[1:])])
+            seen.append(data_id)
+        finished += s.process_batch_result(cur.request_ids, cur.data_ids)
+    assert seen == [f"d{i}" for i in range(6)] and finished == ["r0", "r1", "r2"] and not s.has_waiting_requests()
+
+
 def test_worker_hand_off_of_real_embeddings(dev, tmp_path):
     """Embeddings of a real forward pass through the worker's hand-off to the mock sidecar: contiguous device
     tensors (what the reference's sender exports by IPC handle), saved and reloaded bit-exactly."""

@@ -411,5 +411,31 @@ def test_scheduler_batches_like_the_reference_and_bounds_patches():
     assert s.schedule().data_ids == ["d3"]
     with pytest.raises(ValueError):
         sc.Scheduler(max_batch_patches=0)
+    # items handed out are in flight: a second schedule() before the result is reported takes the NEXT items, so a
+    # caller can prepare batch k+1 (upload it) while batch k runs; nothing is handed out twice
+    s = sc.Scheduler(max_batch_size=2)
+    s.enqueue(sc.EngineEnqueueRequest("r0", [item(i) for i in range(3)]))
+    s.enqueue(sc.EngineEnqueueRequest("r1", [item(3, Modality.VIDEO), item(4)]))
+    b0, b1 = s.schedule(), s.schedule()
+    assert b0.data_ids == ["d0", "d1"] and b1.data_ids == ["d2"]          # d3 is another modality
+    b2 = s.schedule()
+    assert (b2.modality, b2.data_ids) == (Modality.VIDEO, ["d3"]) and s.has_schedulable_items()
+    assert s.schedule().data_ids == ["d4"] and not s.has_schedulable_items() and s.has_waiting_requests()
+    with pytest.raises(RuntimeError, match="nothing to schedule"):
+        s.schedule()
+    assert s.process_batch_result(b1.request_ids, b1.data_ids) == []       # results may come back in any order
+    assert s.process_batch_result(b0.request_ids, b0.data_ids) == ["r0"]
+    with pytest.raises(KeyError):
+        s.process_batch_result(["r0"], ["d0"])                             # reported twice
+    assert s.process_batch_result(["r1", "r1"], ["d4", "d3"]) == ["r1"] and not s.has_waiting_requests()
+    with pytest.raises(ValueError):
+        s.enqueue(sc.EngineEnqueueRequest("r5", []))
+    s.enqueue(sc.EngineEnqueueRequest("r6", [item(0)]))
+    with pytest.raises(ValueError, match="already queued"):
+        s.enqueue(sc.EngineEnqueueRequest("r6", [item(1)]))
+    # the upload event of a batch sent ahead travels with the conversion
+    b = s.schedule()
+    b._uploaded = marker = object()
+    assert b.to_worker_batch()._uploaded is marker
     tiles = sc.ProcessedEmbeddingData("t", Modality.IMAGE, "m", {"pixel_values": torch.zeros(3, 3, 28, 42)})
     assert sc.patch_count(tiles) == 3 * 2 * 3 and sc.patch_count(item(0, grid=(2, 4, 6))) == 48
