@@ -23,10 +23,11 @@ of its Qwen2-VL processors:
 Pinned by tests/test_oracle_preprocess.py: `smart_resize` and the "numpy" table + layout bit-for-bit against the
 installed package's PIL processor on images whose size needs no resampling; the layout also against an index formula
 written independently (brute force over every output element of small cases); videos through the identity "a video
-of repeated frames == the image".  PARITY UNPINNED: the "fused" table (its processor needs torchvision, which is not
-installed) — it is checked only against the "numpy" table (at most 2 units in the last place apart, equal after
-the cast to bfloat16 for all but a few byte values); resampling (bicubic resize) is not restated at all: it stays
-in the caller's CPU code.
+of repeated frames == the image"; the "fused" table entry by entry against an exact-rational evaluation of its four
+binary32 operations with IEEE round-to-nearest-even after each (what the standard fixes for that sequence; float64
+intermediates or the other order of operations fail it).  PARITY UNPINNED: that torchvision's normalize -- absent here
+-- is exactly "subtract, then divide" in float32 (taken from its published source), and resampling (bicubic resize),
+which is not restated at all: it stays in the caller's CPU code.
 """
 
 from __future__ import annotations

@@ -61,6 +61,48 @@ def test_tables():
     assert (ta != tb).sum().item() <= 3
 
 
+def _rn32(x):
+    """Round an exact rational to the nearest float32, ties to even -- what one IEEE-754 binary32 operation returns
+    for an exact result x -- by exact comparison with the two neighbouring float32 values."""
+    from fractions import Fraction
+
+    c = np.float32(float(x))                       # within one float32 ulp of x
+    cands = sorted({np.nextafter(c, np.float32(-np.inf)), c, np.nextafter(c, np.float32(np.inf))}, key=float)
+    best = min(cands, key=lambda f: (abs(Fraction(float(f)) - x), int(np.float32(f).view(np.uint32)) & 1))
+    return np.float32(best)
+
+
+def test_fused_table_is_the_ieee_evaluation_of_the_published_sequence():
+    """The "fused" arithmetic of the torch image processor is four binary32 operations per value -- mean * (1/scale),
+    std * (1/scale), u - mean', (.) / std' (transformers `_fuse_mean_std_and_rescale_factor` followed by torchvision's
+    normalize: subtract, then divide) -- and IEEE-754 fixes the result of each: the exact value rounded to nearest
+    even.  Evaluated with exact rationals and that rounding, every one of the 768 entries must come out bit for bit;
+    float64 intermediates, a multiply by the reciprocal or the "numpy" order of operations each change some entry."""
+    from fractions import Fraction
+
+    for mean, std in ((qp.OPENAI_CLIP_MEAN, qp.OPENAI_CLIP_STD), ((0.5, 0.5, 0.5), (0.5, 0.5, 0.5))):
+        table = qp.normalization_table(mean, std, arithmetic="fused")
+        inv = _rn32(Fraction(1.0 / (1 / 255)))     # the Python float 1/scale enters the float32 multiply as float32
+        assert inv == np.float32(255.0)
+        for c in range(3):
+            m = _rn32(Fraction(float(np.float32(mean[c]))) * Fraction(float(inv)))
+            s = _rn32(Fraction(float(np.float32(std[c]))) * Fraction(float(inv)))
+            for u in range(256):
+                d = _rn32(Fraction(u) - Fraction(float(m)))
+                want = _rn32(Fraction(float(d)) / Fraction(float(s)))
+                assert table[c, u].view(np.uint32) == want.view(np.uint32), (c, u, table[c, u], want)
+    # the near-misses this evaluation tells apart from the published sequence
+    clip = qp.normalization_table(arithmetic="fused")
+    u = np.arange(256, dtype=np.float64)[None, :]
+    m64, s64 = np.asarray(qp.OPENAI_CLIP_MEAN, np.float32).astype(np.float64)[:, None], np.asarray(qp.OPENAI_CLIP_STD, np.float32).astype(np.float64)[:, None]
+    assert (((u - m64 * 255.0) / (s64 * 255.0)).astype(np.float32) != clip).any()        # float64 intermediates
+    assert (qp.normalization_table(arithmetic="numpy") != clip).any()                     # the other order
+    # the library's own table (what the GPU kernel looks bytes up in) is the same array
+    from cornserve_amd.eric import frames
+    assert np.array_equal(frames.byte_table(arithmetic="fused").numpy(), clip)
+    assert np.array_equal(frames.byte_table(arithmetic="numpy").numpy(), qp.normalization_table(arithmetic="numpy"))
+
+
 def _brute_force(frames, table, patch, merge, temporal):
     """Every output element from its definition, with plain index arithmetic (no reshape / transpose)."""
     T, H, W, _ = frames.shape
