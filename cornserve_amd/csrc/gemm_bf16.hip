@@ -15,7 +15,7 @@
 // Epilogues (all optional-bias, fp32 accumulate, rounding points follow the reference's bf16 steps):
 //   EPI_BIAS       y = bf16(acc + b)
 //   EPI_RESIDUAL   y = bf16( bf16(acc + b) + r )                     (qwen2_5_vl.py:175,177)
-//   EPI_SWIGLU     y[j] = bf16( bf16(silu(bf16(acc[2j]+b[2j]))) * bf16(acc[2j+1]+b[2j+1]) )
+//   EPI_SWIGLU     y[j] = bf16( silu(bf16(acc[2j]+b[2j])) * bf16(acc[2j+1]+b[2j+1]) )
 //                                                                    (qwen2_5_vl.py:143-148)
 //   EPI_GELU_ERF   y = bf16(gelu_erf(bf16(acc + b)))                 (qwen2_5_vl.py:218-222)
 //   EPI_GELU_TANH  y = bf16(gelu_tanh(bf16(acc + b)))                (siglip.py:155-163)

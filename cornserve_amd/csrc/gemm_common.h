@@ -62,8 +62,10 @@ CS_DEVICE void epilogue(const CsGemmArgs& p, const f32x16_t (&acc)[MT][NT], int 
           for (int q = 0; q < 4; ++q) v[q] += bf2f(b[q]);
         }
         if (EPI == CS_EPI_SWIGLU) {
-          const float gate0 = rbf(silu(rbf(v[0]))), up0 = rbf(v[1]);
-          const float gate1 = rbf(silu(rbf(v[2]))), up1 = rbf(v[3]);
+          // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the product stay
+          // in fp32 until the single output rounding (the same rounding points as the direct-to-LDS kernel)
+          const float gate0 = silu(rbf(v[0])), up0 = rbf(v[1]);
+          const float gate1 = silu(rbf(v[2])), up1 = rbf(v[3]);
           bf16x2_t o;
           o[0] = f2bf(gate0 * up0);
           o[1] = f2bf(gate1 * up1);

@@ -41,9 +41,6 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   // 256x160 tile exists for N = 1280 (8 column tiles: 8192 rows give exactly 256 workgroups).
   const double c256 = rounds_cost(a.M, a.N, 256, 256);
   const double c160 = rounds_cost(a.M, a.N, 256, 160) * 1.15;  // narrower tiles: more LDS and L2 traffic per FLOP
-  static const char* force = getenv("CS_GEMM_TILE");        // benchmarking aid: "160" or "256"
-  // (the erf GELU epilogue with fp8 scales does not fit the architectural registers of the 256x160 form)
-  const bool fits160 = !(a.w_fp8 && a.epilogue == CS_EPI_GELU_ERF);
   // Few rows: 160-column tiles of 256 rows would leave half of the compute units or more without a tile (N = 1280
   // gives 8 column tiles, so 1024 rows are 32 workgroups).  The 128x160 form has the same waves-by-columns layout,
   // so every output element and every row-sum part is computed by the same sequence of operations: results do not
@@ -56,12 +53,12 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
     return narrow();
   }
   if (a.a_row_sum) return narrow();   // see dispatch_epi_w
-  if (fits160 && (force ? force[0] == '1' : c160 < c256)) return narrow();
+  if (c160 < c256) return narrow();
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller
   // tiles (256x128 or 128x192: more workgroups, each shorter).  The two launches write disjoint column
   // ranges of C.
-  if (!force) {
+  {
     const int tn = (a.N + 255) / 256;
     double best = c256;
     int best_cols = 0;

@@ -77,13 +77,6 @@ CS_DEVICE void wg_barrier() {
   asm volatile("" ::: "memory");
 }
 
-#ifdef CS_GEMM_TS
-__device__ long long* cs_ts_buf;  // [tiles][8]: 4 wall-clock stamps + 4 shader-clock stamps by wave 0 (profiling builds only)
-#define CS_TS(slot) do { if (tid == 0 && cs_ts_buf) { cs_ts_buf[vb * 8 + (slot)] = wall_clock64(); cs_ts_buf[vb * 8 + 4 + (slot)] = clock64(); } } while (0)
-#else
-#define CS_TS(slot) do { } while (0)
-#endif
-
 // every accumulation register, as an inline-asm clobber list
 #define CS_ALL_ACC_REGS \
   "a0", "a1", "a2", "a3", "a4", "a5", "a6", "a7", "a8", "a9", "a10", "a11", "a12", "a13", "a14", "a15", \
@@ -370,13 +363,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     const int vb_next = vb + gridDim.x;
     const bool has_next = vb_next < ntiles;
     int m0_next = 0, n0_next = 0;
-
-    CS_TS(0);
     // K tile 0 has landed once at most the loads issued after it are outstanding.  (Loads complete in
     // order; stores of the previous epilogue that are still in flight only make this wait longer.)
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(PENDING_AT_TILE_START));
     wg_barrier();
-    CS_TS(1);
     static_for<NFR>([&](auto n) { read_frag(a_base_of(0, ring), w_base_of(0, ring), 0, 0, n); });
 
     // One K iteration.  TAIL 0: steady state.  TAIL t > 0: t iterations before the end of the output tile,
@@ -453,7 +443,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     // inline-asm MFMAs are opaque to the compiler's hazard tracking: let the last results land before the
     // epilogue reads the accumulation registers
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-    CS_TS(2);
 
     // ---- epilogue.  Accumulator (i, j), element r = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
     //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
@@ -689,7 +678,6 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         }
       });
     }
-    CS_TS(3);
     if (!has_next) break;
     vb = vb_next;
     m0 = m0_next;
@@ -771,9 +759,7 @@ int dispatch_epi_w(const CsGemmArgs& a, hipStream_t s) {
       return a.c_lo ? launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, W_FP8, 0, true>(a, s)
                     : launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_RESIDUAL, W_FP8>(a, s);
     case CS_EPI_SWIGLU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_SWIGLU, W_FP8>(a, s);
-    case CS_EPI_GELU_ERF:
-      if constexpr (W_FP8 && BN == 160) return CS_ERR_UNSUPPORTED;  // never dispatched, see cs_gemm_fast
-      else return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_ERF, W_FP8>(a, s);
+    case CS_EPI_GELU_ERF: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_ERF, W_FP8>(a, s);
     case CS_EPI_GELU_TANH: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_GELU_TANH, W_FP8>(a, s);
     case CS_EPI_QUICK_GELU: return launch<BM, BN, WAVES_M, WAVES_N, CS_EPI_QUICK_GELU, W_FP8>(a, s);
     default: return CS_ERR_INVALID_ARG;

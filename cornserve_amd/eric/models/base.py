@@ -104,7 +104,7 @@ def fold_layernorm(w: torch.Tensor, b: torch.Tensor | None, ln_w: torch.Tensor, 
     normalisation itself (CsGemmArgs.a_row_sum):  LN(x) . W^T + b  ==  rstd * (x . W'^T - mean * colsum) + b'.
     Returns (W' = W * ln_w along the columns, b' = b + W . ln_b, colsum = row sums of the rounded W' in fp32)."""
     wf = (w.float() * ln_w.float()[None, :]).to(w.dtype)
-    bf = w.float() @ ln_b.float()
+    bf = (w.float() * ln_b.float()[None, :]).sum(dim=1)   # W . ln_b as an elementwise product and a row sum
     if b is not None:
         bf = bf + b.float()
     return wf.contiguous(), bf.to(w.dtype).contiguous(), wf.float().sum(dim=1).contiguous()

@@ -253,6 +253,33 @@ def test_gemm_epilogues(ops, dev):
     close(ops.gemm(a, w, b, pos=pos), base + pos.float().cpu()[idx], 2**-7, "pos")
 
 
+def test_both_gemm_kernels_round_their_epilogues_alike(ops, dev):
+    """The direct-to-LDS kernel and the general kernel accumulate in different orders, so on random data their fp32
+    sums differ in the last bits; on operands whose products and sums are exact (small integers over 8) the sums are
+    equal, and then every fused epilogue -- SwiGLU included -- must give the same bits in either kernel: same rounding
+    points, same activation code.  K = 192 takes the fast kernel; the same matrices with 8 zero columns appended
+    (K = 200, a K tail) take the general one."""
+    g = torch.Generator().manual_seed(5)
+    M, N, K = 300, 512, 192
+    a = torch.randint(-3, 4, (M, K), generator=g).bfloat16()
+    w = (torch.randint(-3, 4, (N, K), generator=g).float() / 8).bfloat16()
+    b = (torch.randint(-8, 9, (N,), generator=g).float() / 8).bfloat16().to(dev)
+    res = (torch.randint(-64, 65, (M, N), generator=g).float() / 8).bfloat16().to(dev)
+    pad = lambda t: torch.cat([t, torch.zeros((t.shape[0], 8), dtype=t.dtype)], dim=1).contiguous().to(dev)  # noqa: E731
+    a_f, w_f, a_g, w_g = a.to(dev), w.to(dev), pad(a), pad(w)
+    for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_SWIGLU, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU):
+        kw = dict(epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
+        fast, general = ops.gemm(a_f, w_f, b, **kw), ops.gemm(a_g, w_g, b, **kw)
+        assert torch.equal(fast, general), f"epilogue {epi}"
+    lo = torch.randint(0, 256, (M, N), generator=g, dtype=torch.uint8).to(dev)
+    outs = []
+    for aa, ww in ((a_f, w_f), (a_g, w_g)):
+        o, ol = torch.empty_like(res), torch.empty_like(lo)
+        ops.gemm(aa, ww, b, epilogue=ops.EPI_RESIDUAL, residual=res, residual_lo=lo, out=o, out_lo=ol)
+        outs.append((o, ol))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+
+
 def _epilogue_ref(ops, epi, base, res):
     """fp32 reference of one fused epilogue on `base` = bf16-rounded A.W^T + bias."""
     if epi == ops.EPI_BIAS:
