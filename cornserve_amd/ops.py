@@ -1,8 +1,13 @@
-"""Thin tensor-level wrappers over the C ABI: torch supplies device memory and the stream, nothing else.
+"""Thin PyTorch custom ops over the C ABI: torch supplies device memory and the stream, nothing else.
 
-Every function enqueues HIP kernels from libcornserve_amd.so on torch's current stream and returns
-torch tensors allocated by torch's caching allocator (so outputs stay IPC-exportable for the sidecar,
-reference: sidecar/api.py:198-242).  There is no eager-PyTorch fallback in this module.
+Every kernel entry point of libcornserve_amd.so is registered as an operator of the `cornserve_amd` namespace
+(`torch.ops.cornserve_amd.gemm_`, `.attn_varlen_`, `.rmsnorm_`, ...: schema, a fake implementation for shape
+propagation, and one implementation that validates its arguments and enqueues the HIP kernels on torch's current
+stream through ctypes).  The functions of this module are the keyword-argument front ends the encoders call: they
+allocate outputs with torch's caching allocator (so outputs stay IPC-exportable for the sidecar, reference:
+sidecar/api.py:198-242) and dispatch through `torch.ops`, so the launches are visible to the dispatcher, the
+profiler's operator records and tracing.  The operators that write into caller-provided tensors end in `_` and
+return nothing; `gemm` also exists in a functional form.  There is no eager-PyTorch fallback in this module.
 """
 
 from __future__ import annotations
@@ -99,16 +104,43 @@ def gemm(
 ) -> torch.Tensor:
     """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`.
 
+    `a_row_sumsq` (fp32 [M, SUMSQ_PARTS]) scales row m of the product by rsqrt(sum(parts)/K + norm_eps): an
+    RMSNorm of `a` whose weight the caller has folded into the columns of `w`.  `c_row_sumsq` (same layout,
+    indexed by output row) receives the sums of squares of the output rows.  With `a_row_sum` (and `w_col_sum`,
+    fp32 [N], the row sums of the folded weight) the fold is a LayerNorm's: rstd * (acc - mean * w_col_sum) + bias;
+    `c_row_sum` receives the plain sums of the output rows.
+
     `out_lo` (uint8, shaped and strided like `out`; EPI_RESIDUAL only) carries the residual stream with 16
     significant bits: the sum is not rounded to bf16 but split into `out` (the leading 16 bits) and `out_lo` (the
     next 8 as a signed correction); `residual_lo` is the same plane of the addend (None: the addend is `residual`
     exactly).  A zero-filled plane next to any bf16 tensor is a valid pair.
 
-    `a_row_sumsq` (fp32 [M, SUMSQ_PARTS]) scales row m of the product by rsqrt(sum(parts)/K + norm_eps): an
-    RMSNorm of `a` whose weight the caller has folded into the columns of `w`.  `c_row_sumsq` (same layout,
-    indexed by output row) receives the sums of squares of the output rows.  With `a_row_sum` (and `w_col_sum`,
-    fp32 [N], the row sums of the folded weight) the fold is a LayerNorm's: rstd * (acc - mean * w_col_sum) + bias;
-    `c_row_sum` receives the plain sums of the output rows."""
+    Dispatches to `torch.ops.cornserve_amd.gemm_` (or the functional `gemm` when nothing is written in place)."""
+    if out is None and c_row_sumsq is None and c_row_sum is None and out_lo is None and residual_lo is None:
+        return torch.ops.cornserve_amd.gemm(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k,
+                                            a_row_sumsq, norm_eps, a_row_sum, w_col_sum)
+    if out is None:  # (with c_rows: a permutation of the M rows; anything else needs the caller's `out`)
+        M = a.shape[0] if a_rows is None else a_rows.shape[0]
+        out = torch.empty((M, w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]), dtype=torch.bfloat16, device=a.device)
+    torch.ops.cornserve_amd.gemm_(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq,
+                                  c_row_sumsq, norm_eps, a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo)
+    return out
+
+
+def _gemm_functional(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, norm_eps, a_row_sum,
+                     w_col_sum):
+    if a.dim() != 2 or w.dim() != 2:
+        raise ValueError("gemm operands must be 2-D")
+    M = a.shape[0] if a_rows is None else a_rows.shape[0]
+    out = torch.empty((M, w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]), dtype=torch.bfloat16, device=a.device)
+    _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, None, norm_eps,
+               a_row_sum, None, w_col_sum, None, None)
+    return out
+
+
+def _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, c_row_sumsq, norm_eps,
+               a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo) -> None:
+    """Implementation of cornserve_amd::gemm_: argument checks, then cs_gemm on the current stream."""
     lib = _l.load()
     _req(a, torch.bfloat16, "a")
     if a.dim() != 2 or w.dim() != 2:
@@ -133,8 +165,6 @@ def gemm(
     if c_rows is not None and c_rows.shape[0] < M:
         raise ValueError(f"c_rows has {c_rows.shape[0]} entries for {M} output rows")
     n_out = N // 2 if epilogue == EPI_SWIGLU else N
-    if out is None:  # (with c_rows: a permutation of the M rows; anything else needs the caller's `out`)
-        out = torch.empty((M, n_out), dtype=torch.bfloat16, device=a.device)
     # Everything below reaches the kernel as a raw pointer: shapes, dtypes and devices are checked here, before
     # anything is enqueued, because an undersized or mistyped buffer would be an out-of-bounds device access.
     _req(out, torch.bfloat16, "out")
@@ -206,93 +236,129 @@ def gemm(
     args.residual_lo = _ptr(residual_lo)
     args.c_lo = _ptr(out_lo)
     _l.check(lib.cs_gemm(ctypes.byref(args), _stream()), "cs_gemm")
-    return out
 
 
 # -------------------------------------------------------------------------------------------- norms
 SUMSQ_PARTS = 8  # CS_SUMSQ_PARTS
 
 
+def _rows_2d(t: torch.Tensor, dtype: torch.dtype, name: str) -> None:
+    _req(t, dtype, name)
+    if t.dim() != 2:
+        raise ValueError(f"{name} must be 2-D")
+
+
+def _row_stats_impl(sumsq_out, sum_out, x) -> None:
+    lib = _l.load()
+    _rows_2d(x, torch.bfloat16, "x")
+    for name, t in (("sumsq_out", sumsq_out), ("sum_out", sum_out)):
+        if t is not None:
+            _req(t, torch.float32, name)
+            if tuple(t.shape) != (x.shape[0], SUMSQ_PARTS) or not t.is_contiguous() or t.device != x.device:
+                raise ValueError(f"{name} must be a contiguous fp32 [rows, {SUMSQ_PARTS}] tensor on x's device")
+    if sum_out is None:
+        _l.check(lib.cs_row_sumsq(x.data_ptr(), x.stride(0), x.shape[0], x.shape[1], sumsq_out.data_ptr(), _stream()),
+                 "cs_row_sumsq")
+    else:
+        _l.check(lib.cs_row_stats(x.data_ptr(), x.stride(0), x.shape[0], x.shape[1], sumsq_out.data_ptr(),
+                                  sum_out.data_ptr(), _stream()), "cs_row_stats")
+
+
 def row_stats(x: torch.Tensor, sumsq_out: torch.Tensor, sum_out: torch.Tensor) -> None:
     """Sums of squares and sums of the rows of `x`, each fp32 [rows, SUMSQ_PARTS] in parts of 160 columns."""
-    lib = _l.load()
-    _req(x, torch.bfloat16, "x")
-    _req(sumsq_out, torch.float32, "sumsq_out")
-    _req(sum_out, torch.float32, "sum_out")
-    if x.dim() != 2 or tuple(sumsq_out.shape) != (x.shape[0], SUMSQ_PARTS) or tuple(sum_out.shape) != (x.shape[0], SUMSQ_PARTS):
-        raise ValueError("row_stats takes a 2-D tensor and two [rows, SUMSQ_PARTS] outputs")
-    _l.check(lib.cs_row_stats(x.data_ptr(), x.stride(0), x.shape[0], x.shape[1], sumsq_out.data_ptr(), sum_out.data_ptr(),
-                              _stream()), "cs_row_stats")
+    torch.ops.cornserve_amd.row_stats_(sumsq_out, sum_out, x)
 
 
 def row_sumsq(x: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """fp32 [rows, SUMSQ_PARTS]: sums of squares of the rows of `x` in parts of 160 columns."""
-    lib = _l.load()
-    _req(x, torch.bfloat16, "x")
-    if x.dim() != 2:
-        raise ValueError("row_sumsq takes a 2-D tensor")
     if out is None:
+        if x.dim() != 2:
+            raise ValueError("row_sumsq takes a 2-D tensor")
         out = torch.empty((x.shape[0], SUMSQ_PARTS), dtype=torch.float32, device=x.device)
-    _l.check(lib.cs_row_sumsq(x.data_ptr(), x.stride(0), x.shape[0], x.shape[1], out.data_ptr(), _stream()), "cs_row_sumsq")
+    torch.ops.cornserve_amd.row_stats_(out, None, x)
     return out
+
+
+def _norm_args(out, x, w, b) -> None:
+    _rows_2d(x, torch.bfloat16, "x")
+    _rows_2d(out, torch.bfloat16, "out")
+    H = x.shape[1]
+    if out.shape[0] < x.shape[0] or out.shape[1] < H or out.device != x.device:
+        raise ValueError(f"out must be bf16 [>={x.shape[0]}, >={H}] on x's device")
+    for name, t in (("w", w), ("b", b)):
+        if t is not None:
+            _req(t, torch.bfloat16, name)
+            if t.dim() != 1 or t.shape[0] < H or t.device != x.device:
+                raise ValueError(f"{name} must be bf16 [{H}] on x's device")
+
+
+def _rmsnorm_impl(out, x, w, eps, gemma) -> None:
+    lib = _l.load()
+    _norm_args(out, x, w, None)
+    _l.check(lib.cs_rmsnorm(x.data_ptr(), x.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0), x.shape[0],
+                            x.shape[1], eps, int(gemma), _stream()), "cs_rmsnorm")
+
+
+def _layernorm_impl(out, x, w, b, eps) -> None:
+    lib = _l.load()
+    _norm_args(out, x, w, b)
+    _l.check(lib.cs_layernorm(x.data_ptr(), x.stride(0), w.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
+                              x.shape[0], x.shape[1], eps, _stream()), "cs_layernorm")
 
 
 def rmsnorm(x: torch.Tensor, w: torch.Tensor, eps: float, *, gemma: bool = False,
             out: torch.Tensor | None = None) -> torch.Tensor:
-    lib = _l.load()
-    _req(x, torch.bfloat16, "x")
-    _req(w, torch.bfloat16, "w")
     x2 = x.reshape(-1, x.shape[-1])
     if out is None:
         out = torch.empty_like(x2)
-    _l.check(
-        lib.cs_rmsnorm(x2.data_ptr(), x2.stride(0), w.data_ptr(), out.data_ptr(), out.stride(0),
-                       x2.shape[0], x2.shape[1], eps, int(gemma), _stream()),
-        "cs_rmsnorm",
-    )
+    torch.ops.cornserve_amd.rmsnorm_(out, x2, w, eps, gemma)
     return out.view(x.shape)
 
 
 def layernorm(x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float,
               out: torch.Tensor | None = None) -> torch.Tensor:
-    lib = _l.load()
-    _req(x, torch.bfloat16, "x")
-    _req(w, torch.bfloat16, "w")
-    _req(b, torch.bfloat16, "b")
     x2 = x.reshape(-1, x.shape[-1])
     if out is None:
         out = torch.empty_like(x2)
-    _l.check(
-        lib.cs_layernorm(x2.data_ptr(), x2.stride(0), w.data_ptr(), b.data_ptr(), out.data_ptr(), out.stride(0),
-                         x2.shape[0], x2.shape[1], eps, _stream()),
-        "cs_layernorm",
-    )
+    torch.ops.cornserve_amd.layernorm_(out, x2, w, b, eps)
     return out.view(x.shape)
+
+
+def _avgpool_gemma_rmsnorm_impl(out, x, w, side, k, eps) -> None:
+    lib = _l.load()
+    _req(x, torch.bfloat16, "x")
+    _req(w, torch.bfloat16, "w")
+    _req(out, torch.bfloat16, "out")
+    if x.dim() != 3 or x.shape[1] != side * side or not x.is_contiguous() or k < 1 or side % k:
+        raise ValueError("x must be contiguous [B, side*side, H] with side a multiple of k")
+    B, _, H = x.shape
+    if tuple(out.shape) != (B, (side // k) ** 2, H) or not out.is_contiguous() or w.dim() != 1 or w.shape[0] < H:
+        raise ValueError("out must be contiguous [B, (side/k)^2, H] and w [H]")
+    _l.check(lib.cs_avgpool_gemma_rmsnorm(x.data_ptr(), w.data_ptr(), out.data_ptr(), B, side, k, H, eps, _stream()),
+             "cs_avgpool_gemma_rmsnorm")
 
 
 def avgpool_gemma_rmsnorm(x: torch.Tensor, w: torch.Tensor, side: int, k: int, eps: float) -> torch.Tensor:
     """x [B, side*side, H] -> [B, (side/k)^2, H]: AvgPool2d(k) over the token grid, then GemmaRMSNorm."""
-    lib = _l.load()
-    _req(x, torch.bfloat16, "x")
-    _req(w, torch.bfloat16, "w")
-    if x.dim() != 3 or x.shape[1] != side * side or not x.is_contiguous():
+    if x.dim() != 3 or k < 1:
         raise ValueError("x must be contiguous [B, side*side, H]")
-    B, _, H = x.shape
-    out = torch.empty((B, (side // k) ** 2, H), dtype=torch.bfloat16, device=x.device)
-    _l.check(
-        lib.cs_avgpool_gemma_rmsnorm(x.data_ptr(), w.data_ptr(), out.data_ptr(), B, side, k, H, eps, _stream()),
-        "cs_avgpool_gemma_rmsnorm",
-    )
+    out = torch.empty((x.shape[0], (side // k) ** 2, x.shape[2]), dtype=torch.bfloat16, device=x.device)
+    torch.ops.cornserve_amd.avgpool_gemma_rmsnorm_(out, x, w, side, k, eps)
     return out
 
 
-def cast_f32_bf16(x: torch.Tensor) -> torch.Tensor:
+def _cast_impl(out, x) -> None:
     lib = _l.load()
     _req(x, torch.float32, "x")
-    if not x.is_contiguous():
-        raise ValueError("x must be contiguous")
-    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    _req(out, torch.bfloat16, "out")
+    if not x.is_contiguous() or not out.is_contiguous() or out.shape != x.shape or out.device != x.device:
+        raise ValueError("x and out must be contiguous tensors of one shape on one device")
     _l.check(lib.cs_cast_f32_bf16(x.data_ptr(), out.data_ptr(), x.numel(), _stream()), "cs_cast_f32_bf16")
+
+
+def cast_f32_bf16(x: torch.Tensor) -> torch.Tensor:
+    out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+    torch.ops.cornserve_amd.cast_f32_bf16_(out, x)
     return out
 
 
@@ -346,7 +412,6 @@ class VitIndex:
 
 def vit_index(item_meta: torch.Tensor, total_patches: int, max_units_per_item: int, merge: int, win: int,
               inv_freq: torch.Tensor, *, want_pos_ids: bool = False) -> VitIndex:
-    lib = _l.load()
     _req(item_meta, torch.int32, "item_meta")
     _req(inv_freq, torch.float32, "inv_freq")
     dev = item_meta.device
@@ -358,36 +423,76 @@ def vit_index(item_meta: torch.Tensor, total_patches: int, max_units_per_item: i
     src_rows = torch.empty(L, dtype=torch.int32, device=dev)
     pos_ids = torch.empty((L, 2), dtype=torch.int32, device=dev) if want_pos_ids else None
     cos_sin = torch.empty((L, 2 * rot_dim), dtype=torch.float32, device=dev)
+    torch.ops.cornserve_amd.vit_index_(window_index, reverse_index, src_rows, pos_ids, cos_sin, item_meta,
+                                       max_units_per_item, merge, win, inv_freq)
+    return VitIndex(window_index, reverse_index, src_rows, pos_ids, cos_sin)
+
+
+def _vit_index_impl(window_index, reverse_index, src_rows, pos_ids, cos_sin, item_meta, max_units_per_item, merge, win,
+                    inv_freq) -> None:
+    lib = _l.load()
+    _req(item_meta, torch.int32, "item_meta")
+    _req(inv_freq, torch.float32, "inv_freq")
+    if item_meta.dim() != 2 or item_meta.shape[1] != 8 or not item_meta.is_contiguous() or not inv_freq.is_contiguous():
+        raise ValueError("item_meta must be contiguous int32 [n_items, 8] and inv_freq contiguous")
+    rot_dim = 2 * inv_freq.numel()
+    L, U = src_rows.shape[0], window_index.shape[0]
+    for name, t, dt, shape in (("window_index", window_index, torch.int32, (U,)), ("reverse_index", reverse_index, torch.int32, (U,)),
+                               ("src_rows", src_rows, torch.int32, (L,)), ("pos_ids", pos_ids, torch.int32, (L, 2)),
+                               ("cos_sin", cos_sin, torch.float32, (L, 2 * rot_dim))):
+        if t is not None:
+            _req(t, dt, name)
+            if tuple(t.shape) != shape or not t.is_contiguous() or t.device != item_meta.device:
+                raise ValueError(f"{name} must be a contiguous {dt} {shape} tensor on item_meta's device")
+    if U * merge * merge != L:
+        raise ValueError("window_index and src_rows disagree about the number of patches")
     _l.check(
         lib.cs_vit_index(item_meta.data_ptr(), item_meta.shape[0], max_units_per_item, merge, win,
                          inv_freq.data_ptr(), rot_dim, window_index.data_ptr(), reverse_index.data_ptr(),
                          src_rows.data_ptr(), _ptr(pos_ids), cos_sin.data_ptr(), _stream()),
         "cs_vit_index",
     )
-    return VitIndex(window_index, reverse_index, src_rows, pos_ids, cos_sin)
 
 
 def pos_embed_interp(table: torch.Tensor, item_meta: torch.Tensor, total_patches: int, max_units_per_item: int,
                      merge: int) -> torch.Tensor:
     """Qwen3-VL position rows [total_patches, E] (bf16, patch order) interpolated from the learned side x side table."""
+    if table.dim() != 2:
+        raise ValueError("table must be a contiguous [side*side, E] tensor")
+    out = torch.empty((total_patches, table.shape[1]), dtype=torch.bfloat16, device=table.device)
+    torch.ops.cornserve_amd.pos_embed_interp_(out, table, item_meta, max_units_per_item, merge)
+    return out
+
+
+def _pos_embed_interp_impl(out, table, item_meta, max_units_per_item, merge) -> None:
     lib = _l.load()
     _req(table, torch.bfloat16, "table")
     _req(item_meta, torch.int32, "item_meta")
+    _rows_2d(out, torch.bfloat16, "out")
     side = int(round(table.shape[0] ** 0.5))
     if table.dim() != 2 or side * side != table.shape[0] or not table.is_contiguous():
         raise ValueError("table must be a contiguous [side*side, E] tensor")
-    out = torch.empty((total_patches, table.shape[1]), dtype=torch.bfloat16, device=table.device)
+    if out.shape[1] < table.shape[1] or item_meta.dim() != 2 or item_meta.shape[1] != 8 or not item_meta.is_contiguous():
+        raise ValueError("out must have the table's width and item_meta must be contiguous int32 [n_items, 8]")
     _l.check(
         lib.cs_pos_embed_interp(table.data_ptr(), side, table.shape[1], item_meta.data_ptr(), item_meta.shape[0],
                                 max_units_per_item, merge, out.data_ptr(), out.stride(0), _stream()),
         "cs_pos_embed_interp",
     )
-    return out
 
 
 def rows_bilinear(src: torch.Tensor, taps: torch.Tensor, frac: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
     """out[r] = bilinear mix of the four rows taps[r] of src with the fractions frac[r] = (ly, lx); (0, 0) copies
     row taps[r, 0].  src: bf16 [n, E] with contiguous rows, taps: int32 [R, 4], frac: fp32 [R, 2] (device tensors)."""
+    if out is None:
+        if src.dim() != 2 or taps.dim() != 2:
+            raise ValueError("src must be 2-D with contiguous rows and taps [R, 4]")
+        out = torch.empty((taps.shape[0], src.shape[1]), dtype=torch.bfloat16, device=src.device)
+    torch.ops.cornserve_amd.rows_bilinear_(out, src, taps, frac)
+    return out
+
+
+def _rows_bilinear_impl(out, src, taps, frac) -> None:
     lib = _l.load()
     _req(src, torch.bfloat16, "src")
     _req(taps, torch.int32, "taps")
@@ -398,48 +503,59 @@ def rows_bilinear(src: torch.Tensor, taps: torch.Tensor, frac: torch.Tensor, out
     if taps.shape != (R, 4) or frac.shape != (R, 2) or not taps.is_contiguous() or not frac.is_contiguous():
         raise ValueError("taps must be contiguous [R, 4] and frac contiguous [R, 2]")
     E = src.shape[1]
-    if out is None:
-        out = torch.empty((R, E), dtype=torch.bfloat16, device=src.device)
-    else:
-        _req(out, torch.bfloat16, "out")
-        if out.shape != (R, E) or out.stride(1) != 1:
-            raise ValueError("out must be [R, E] with contiguous rows")
+    _req(out, torch.bfloat16, "out")
+    if out.shape != (R, E) or out.stride(1) != 1:
+        raise ValueError("out must be [R, E] with contiguous rows")
     _l.check(
         lib.cs_rows_bilinear(src.data_ptr(), src.stride(0), src.shape[0], taps.data_ptr(), frac.data_ptr(), R, E,
                              out.data_ptr(), out.stride(0), _stream()),
         "cs_rows_bilinear",
     )
-    return out
 
 
 def row_gather(x: torch.Tensor, rows: torch.Tensor) -> torch.Tensor:
     """out[i] = x[rows[i]] for a 2-D tensor with contiguous rows."""
+    if x.dim() != 2 or rows.dim() != 1:
+        raise ValueError("x must be a 2-D device tensor with contiguous rows and rows a vector")
+    out = torch.empty((rows.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    torch.ops.cornserve_amd.row_gather_(out, x, rows)
+    return out
+
+
+def _row_gather_impl(out, x, rows) -> None:
     lib = _l.load()
     _req(rows, torch.int32, "rows")
     if not x.is_cuda or x.dim() != 2 or x.stride(1) != 1:
         raise ValueError("x must be a 2-D device tensor with contiguous rows")
     es = x.element_size()
-    out = torch.empty((rows.shape[0], x.shape[1]), dtype=x.dtype, device=x.device)
+    if (not rows.is_contiguous() or out.dtype != x.dtype or out.device != x.device or out.dim() != 2 or out.stride(1) != 1
+            or tuple(out.shape) != (rows.shape[0], x.shape[1]) or (x.shape[1] * es) % 4):
+        raise ValueError("out must be [len(rows), x.shape[1]] of x's dtype on x's device, rows of whole 4-byte words")
     _l.check(
         lib.cs_row_gather(x.data_ptr(), x.stride(0) * es, rows.data_ptr(), out.data_ptr(), out.stride(0) * es,
                           rows.shape[0], x.shape[1] * es, _stream()),
         "cs_row_gather",
     )
-    return out
 
 
 def rope_qk_(qkv: torch.Tensor, cos_sin: torch.Tensor, heads: int, head_dim: int) -> torch.Tensor:
     """In-place rotary on the q and k blocks of a packed [L, 3*heads*head_dim] buffer."""
+    torch.ops.cornserve_amd.rope_qk_(qkv, cos_sin, heads, head_dim)
+    return qkv
+
+
+def _rope_qk_impl(qkv, cos_sin, heads, head_dim) -> None:
     lib = _l.load()
-    _req(qkv, torch.bfloat16, "qkv")
+    _rows_2d(qkv, torch.bfloat16, "qkv")
     _req(cos_sin, torch.float32, "cos_sin")
-    if cos_sin.shape != (qkv.shape[0], head_dim) or not cos_sin.is_contiguous():
-        raise ValueError("cos_sin must be contiguous [L, head_dim]")
+    if cos_sin.shape != (qkv.shape[0], head_dim) or not cos_sin.is_contiguous() or cos_sin.device != qkv.device:
+        raise ValueError("cos_sin must be contiguous [L, head_dim] on qkv's device")
+    if heads < 1 or qkv.shape[1] < 2 * heads * head_dim:
+        raise ValueError(f"qkv rows hold {qkv.shape[1]} values, fewer than the q and k blocks of {heads} heads")
     _l.check(
         lib.cs_rope_qk(qkv.data_ptr(), qkv.stride(0), cos_sin.data_ptr(), qkv.shape[0], heads, head_dim, _stream()),
         "cs_rope_qk",
     )
-    return qkv
 
 
 # --------------------------------------------------------------------------------------- attention
@@ -480,25 +596,37 @@ def attn_varlen(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, plan: AttnPla
                 keys_rotated: bool = False) -> torch.Tensor:
     """q/k/v: [L, >= heads*head_dim] views sharing one row stride (e.g. thirds of a packed QKV buffer).
     `keys_rotated`: k already carries the rotary of `cos_sin`; only q is rotated (long segments only)."""
+    if out is None:
+        out = torch.empty((q.shape[0], heads * head_dim), dtype=torch.bfloat16, device=q.device)
+    torch.ops.cornserve_amd.attn_varlen_(out, q, k, v, plan.work, plan.n_work, plan.max_seqlen, heads, head_dim, scale,
+                                         cos_sin, keys_rotated)
+    return out
+
+
+def _attn_varlen_impl(out, q, k, v, work, n_work, max_seqlen, heads, head_dim, scale, cos_sin, keys_rotated) -> None:
     lib = _l.load()
-    for name, t in (("q", q), ("k", k), ("v", v)):
-        _req(t, torch.bfloat16, name)
+    for name, t in (("q", q), ("k", k), ("v", v), ("out", out)):
+        _rows_2d(t, torch.bfloat16, name)
+        if t.shape[1] < heads * head_dim or t.device != q.device:
+            raise ValueError(f"{name} must hold {heads} heads of {head_dim} values per row on q's device")
     if not (q.stride(0) == k.stride(0) == v.stride(0)):
         raise ValueError("q, k, v must share a row stride")
     L = q.shape[0]
+    if k.shape[0] != L or v.shape[0] != L or out.shape[0] < L:
+        raise ValueError("q, k, v and out must have one row per token")
+    _req(work, torch.int32, "work")
+    if work.dim() != 2 or work.shape[1] != 4 or not work.is_contiguous() or work.shape[0] < n_work or work.device != q.device:
+        raise ValueError("work must be a contiguous int32 [>=n_work, 4] tensor on q's device")
     if cos_sin is not None:
         _req(cos_sin, torch.float32, "cos_sin")
-        if cos_sin.shape != (L, head_dim) or not cos_sin.is_contiguous():
-            raise ValueError("cos_sin must be contiguous [L, head_dim]")
-    if out is None:
-        out = torch.empty((L, heads * head_dim), dtype=torch.bfloat16, device=q.device)
+        if cos_sin.shape != (L, head_dim) or not cos_sin.is_contiguous() or cos_sin.device != q.device:
+            raise ValueError("cos_sin must be contiguous [L, head_dim] on q's device")
     entry = lib.cs_attn_varlen_keys_rotated if keys_rotated else lib.cs_attn_varlen
     _l.check(
         entry(q.data_ptr(), k.data_ptr(), v.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0),
-              plan.work.data_ptr(), plan.n_work, heads, head_dim, scale, _ptr(cos_sin), plan.max_seqlen, _stream()),
+              work.data_ptr(), n_work, heads, head_dim, scale, _ptr(cos_sin), max_seqlen, _stream()),
         "cs_attn_varlen_keys_rotated" if keys_rotated else "cs_attn_varlen",
     )
-    return out
 
 
 def attn_varlen_rotary_(qkv: torch.Tensor, plan: AttnPlan, heads: int, head_dim: int, scale: float,
@@ -525,6 +653,17 @@ def qwen_patchify_u8(frames: torch.Tensor, table: torch.Tensor, patch: int, merg
     """uint8 frames [T,H,W,3] -> normalised patch rows [ceil(T/temporal)*(H/patch)*(W/patch), 3*temporal*patch^2]
     in the Qwen2-VL processor's layout; `table` is the fp32 [3,256] byte table.  `out` may be a row slice of a
     larger buffer."""
+    if out is None:
+        if frames.dim() != 4:
+            raise ValueError("frames must be contiguous uint8 [T,H,W,3]")
+        T, H, W, _ = frames.shape
+        out = torch.empty((-(-T // temporal) * (H // patch) * (W // patch), 3 * temporal * patch * patch), dtype=dtype,
+                          device=frames.device)
+    torch.ops.cornserve_amd.qwen_patchify_u8_(out, frames, table, patch, merge, temporal)
+    return out
+
+
+def _qwen_patchify_u8_impl(out, frames, table, patch, merge, temporal) -> None:
     lib = _l.load()
     _req(frames, torch.uint8, "frames")
     _req(table, torch.float32, "table")
@@ -536,25 +675,85 @@ def qwen_patchify_u8(frames: torch.Tensor, table: torch.Tensor, patch: int, merg
     if H % (patch * merge) or W % (patch * merge):
         raise ValueError(f"frame size {H}x{W} is not a multiple of patch*merge = {patch * merge}")
     rows, cols = -(-T // temporal) * (H // patch) * (W // patch), 3 * temporal * patch * patch
-    if out is None:
-        out = torch.empty((rows, cols), dtype=dtype, device=frames.device)
-    elif out.dtype not in (torch.bfloat16, torch.float32) or tuple(out.shape) != (rows, cols) or out.stride(1) != 1:
-        raise ValueError(f"out must be bf16 or fp32 [{rows},{cols}]")
+    if (not out.is_cuda or out.dtype not in (torch.bfloat16, torch.float32) or tuple(out.shape) != (rows, cols)
+            or out.stride(1) != 1 or out.device != frames.device or table.device != frames.device):
+        raise ValueError(f"out must be bf16 or fp32 [{rows},{cols}] on the frames' device")
     _l.check(lib.cs_qwen_patchify_u8(frames.data_ptr(), T, H, W, patch, merge, temporal, table.data_ptr(),
                                      out.data_ptr(), out.stride(0), int(out.dtype == torch.float32), _stream()),
              "cs_qwen_patchify_u8")
-    return out
 
 
 def patchify_nchw(pixels: torch.Tensor, patch: int, ldo: int) -> torch.Tensor:
     """[B,C,H,W] bf16 -> [B*(H//p)*(W//p), ldo] rows of (c,ky,kx)-ordered patch values, zero padded.  Pixels past the
     last whole patch are dropped, as a convolution with stride = kernel and no padding drops them."""
-    lib = _l.load()
-    _req(pixels, torch.bfloat16, "pixels")
-    if pixels.dim() != 4 or not pixels.is_contiguous():
+    if pixels.dim() != 4 or patch < 1:
         raise ValueError("pixels must be contiguous [B,C,H,W]")
     B, C, H, W = pixels.shape
     out = torch.empty((B * (H // patch) * (W // patch), ldo), dtype=torch.bfloat16, device=pixels.device)
-    _l.check(lib.cs_patchify_nchw(pixels.data_ptr(), B, C, H, W, patch, out.data_ptr(), ldo, _stream()),
-             "cs_patchify_nchw")
+    torch.ops.cornserve_amd.patchify_nchw_(out, pixels, patch)
     return out
+
+
+def _patchify_nchw_impl(out, pixels, patch) -> None:
+    lib = _l.load()
+    _req(pixels, torch.bfloat16, "pixels")
+    _rows_2d(out, torch.bfloat16, "out")
+    if pixels.dim() != 4 or not pixels.is_contiguous() or patch < 1:
+        raise ValueError("pixels must be contiguous [B,C,H,W]")
+    B, C, H, W = pixels.shape
+    if (out.shape[0] != B * (H // patch) * (W // patch) or out.shape[1] < C * patch * patch or not out.is_contiguous()
+            or out.device != pixels.device):
+        raise ValueError("out must be contiguous [B*(H//patch)*(W//patch), >= C*patch*patch] on the pixels' device")
+    _l.check(lib.cs_patchify_nchw(pixels.data_ptr(), B, C, H, W, patch, out.data_ptr(), out.shape[1], _stream()),
+             "cs_patchify_nchw")
+
+
+# ------------------------------------------------------------------------------- operator registration
+# One operator per kernel entry point, in the `cornserve_amd` namespace.  Operators ending in `_` write into their
+# leading tensor argument(s) and return nothing; every argument that reaches a kernel as a pointer is a Tensor of the
+# schema, so the dispatcher sees it.  The implementation is registered for every backend key: it validates devices and
+# dtypes itself and raises ValueError, the reference model API's error for bad input.
+_LIBRARY = torch.library.Library("cornserve_amd", "DEF")
+_OPERATORS: dict[str, tuple[str, object]] = {
+    "gemm": ("(Tensor a, Tensor w, Tensor? bias, int epilogue, Tensor? residual, Tensor? w_scale, Tensor? pos, "
+             "Tensor? a_rows, Tensor? c_rows, int? k, Tensor? a_row_sumsq, float norm_eps, Tensor? a_row_sum, "
+             "Tensor? w_col_sum) -> Tensor", _gemm_functional),
+    "gemm_": ("(Tensor(a!) out, Tensor a, Tensor w, Tensor? bias, int epilogue, Tensor? residual, Tensor? w_scale, "
+              "Tensor? pos, Tensor? a_rows, Tensor? c_rows, int? k, Tensor? a_row_sumsq, Tensor(b!)? c_row_sumsq, "
+              "float norm_eps, Tensor? a_row_sum, Tensor(c!)? c_row_sum, Tensor? w_col_sum, Tensor? residual_lo, "
+              "Tensor(d!)? out_lo) -> ()", _gemm_impl),
+    "row_stats_": ("(Tensor(a!) sumsq_out, Tensor(b!)? sum_out, Tensor x) -> ()", _row_stats_impl),
+    "rmsnorm_": ("(Tensor(a!) out, Tensor x, Tensor w, float eps, bool gemma) -> ()", _rmsnorm_impl),
+    "layernorm_": ("(Tensor(a!) out, Tensor x, Tensor w, Tensor b, float eps) -> ()", _layernorm_impl),
+    "avgpool_gemma_rmsnorm_": ("(Tensor(a!) out, Tensor x, Tensor w, int side, int k, float eps) -> ()",
+                               _avgpool_gemma_rmsnorm_impl),
+    "cast_f32_bf16_": ("(Tensor(a!) out, Tensor x) -> ()", _cast_impl),
+    "vit_index_": ("(Tensor(a!) window_index, Tensor(b!) reverse_index, Tensor(c!) src_rows, Tensor(d!)? pos_ids, "
+                   "Tensor(e!) cos_sin, Tensor item_meta, int max_units_per_item, int merge, int win, Tensor inv_freq) -> ()",
+                   _vit_index_impl),
+    "pos_embed_interp_": ("(Tensor(a!) out, Tensor table, Tensor item_meta, int max_units_per_item, int merge) -> ()",
+                          _pos_embed_interp_impl),
+    "rows_bilinear_": ("(Tensor(a!) out, Tensor src, Tensor taps, Tensor frac) -> ()", _rows_bilinear_impl),
+    "row_gather_": ("(Tensor(a!) out, Tensor x, Tensor rows) -> ()", _row_gather_impl),
+    "rope_qk_": ("(Tensor(a!) qkv, Tensor cos_sin, int heads, int head_dim) -> ()", _rope_qk_impl),
+    "attn_varlen_": ("(Tensor(a!) out, Tensor q, Tensor k, Tensor v, Tensor work, int n_work, int max_seqlen, int heads, "
+                     "int head_dim, float scale, Tensor? cos_sin, bool keys_rotated) -> ()", _attn_varlen_impl),
+    "qwen_patchify_u8_": ("(Tensor(a!) out, Tensor frames, Tensor table, int patch, int merge, int temporal) -> ()",
+                          _qwen_patchify_u8_impl),
+    "patchify_nchw_": ("(Tensor(a!) out, Tensor pixels, int patch) -> ()", _patchify_nchw_impl),
+}
+
+
+def _fake_gemm(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, norm_eps, a_row_sum, w_col_sum):
+    M = a.shape[0] if a_rows is None else a_rows.shape[0]
+    return a.new_empty((M, w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]), dtype=torch.bfloat16)
+
+
+def _fake_nothing(*args, **kwargs) -> None:   # the in-place operators return nothing: shapes are their arguments'
+    return None
+
+
+for _name, (_schema, _impl) in _OPERATORS.items():
+    _LIBRARY.define(_name + _schema)
+    _LIBRARY.impl(_name, _impl, "CompositeExplicitAutograd")
+    torch.library.register_fake(f"cornserve_amd::{_name}", _fake_gemm if _name == "gemm" else _fake_nothing, lib=_LIBRARY)

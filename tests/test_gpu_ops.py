@@ -280,6 +280,44 @@ def test_both_gemm_kernels_round_their_epilogues_alike(ops, dev):
     assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
 
 
+def test_kernels_are_registered_torch_operators(ops, dev):
+    """Every kernel entry point is an operator of the `cornserve_amd` namespace with a schema that names what it
+    mutates and a fake implementation (shape propagation without running a kernel); `torch.library.opcheck` checks both
+    against real launches.  The front ends of `cornserve_amd.ops` dispatch through these operators."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+
+    M, N, K, heads, d = 130, 256, 192, 2, 64
+    a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
+    res = rnd((M, N), 1.0, 4, dev)
+    none14 = (None,) * 5
+    functional = (a, w, b, ops.EPI_SWIGLU, None, None, None, None, None, None, None, 0.0, None, None)
+    assert torch.equal(torch.ops.cornserve_amd.gemm(*functional), ops.gemm(a, w, b, epilogue=ops.EPI_SWIGLU))
+    tests = ("test_schema", "test_faketensor")
+    torch.library.opcheck(torch.ops.cornserve_amd.gemm.default, functional, test_utils=tests)
+    ss = torch.zeros((M, 8), dtype=torch.float32, device=dev)
+    lo = torch.zeros((M, N), dtype=torch.uint8, device=dev)
+    inplace = (torch.empty_like(res), a, w, b, ops.EPI_RESIDUAL, res, None, None, None, None, None, None, ss, 0.0, None,
+               None, None, lo.clone(), lo)
+    torch.library.opcheck(torch.ops.cornserve_amd.gemm_.default, inplace, test_utils=tests)
+    torch.library.opcheck(torch.ops.cornserve_amd.rmsnorm_.default, (torch.empty_like(a), a, rnd((K,), 1.0, 5, dev), 1e-6, False),
+                          test_utils=tests)
+    qkv = rnd((M, 3 * heads * d), 1.0, 6, dev)
+    plan = ops.attn_plan(np.array([0, 70, M], np.int32), dev)
+    E = heads * d
+    torch.library.opcheck(torch.ops.cornserve_amd.attn_varlen_.default,
+                          (torch.empty((M, E), dtype=torch.bfloat16, device=dev), qkv[:, :E], qkv[:, E:2 * E], qkv[:, 2 * E:],
+                           plan.work, plan.n_work, plan.max_seqlen, heads, d, d ** -0.5, None, False), test_utils=tests)
+    with FakeTensorMode():     # shapes propagate without a device launch
+        fa = torch.empty((M, K), dtype=torch.bfloat16, device=dev)
+        fw = torch.empty((N, K), dtype=torch.bfloat16, device=dev)
+        out = torch.ops.cornserve_amd.gemm(fa, fw, None, ops.EPI_SWIGLU, *none14, None, None, 0.0, None, None)
+        assert tuple(out.shape) == (M, N // 2) and out.dtype == torch.bfloat16
+    for name in ("gemm", "gemm_", "attn_varlen_", "rmsnorm_", "layernorm_", "rope_qk_", "row_stats_", "vit_index_",
+                 "row_gather_", "patchify_nchw_", "qwen_patchify_u8_", "avgpool_gemma_rmsnorm_", "rows_bilinear_",
+                 "pos_embed_interp_", "cast_f32_bf16_"):
+        assert hasattr(torch.ops.cornserve_amd, name), name
+
+
 def _epilogue_ref(ops, epi, base, res):
     """fp32 reference of one fused epilogue on `base` = bf16-rounded A.W^T + bias."""
     if epi == ops.EPI_BIAS:
