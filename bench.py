@@ -19,6 +19,7 @@ with the merged [2048, 3584] embeddings in HBM.  Prints ONE JSON line:
   host_inputs           the same step with the batch handed over as fp32 host tensors (PCIe-inclusive)
   host_inputs_uint8_frames  the same step from resized uint8 frames on the host (PCIe-inclusive; GPU patch layout)
   host_inputs_upload_ahead  the same two host formats with the next batch's copy started ahead on a side stream
+  host_outputs_download_overlap  upload-ahead plus the embeddings copied to pinned host memory on a side stream
   single_image          latency of a batch of one image of the same size (inputs resident in HBM)
   (--workload cfg3 | cfg4 | cfg5 | qwen2_vl | qwen3_vl | llava_ov prints a shorter line -- throughput only -- for the
   other configurations, --workload hbm_kernels the achieved GB/s of the HBM-bound kernels; the default, cfg2, is the
@@ -448,6 +449,34 @@ def main() -> None:
 
         ahead_ms = pipelined_ms(host_batch)
         ahead_frames_ms = pipelined_ms(frame_batch)
+
+        # both directions: upload-ahead as above, and the embeddings of batch k copied to pinned host memory on a
+        # side stream (Worker.download, the copy the reference's sidecar server performs) while batch k+1 computes;
+        # the host waits for download k-1 only after batch k has been enqueued
+        def full_duplex_ms(data: dict, n: int = 6) -> float:
+            mk = lambda: WorkerBatch(modality=Modality.IMAGE, adapter_name="", request_ids=["r"] * N_IMAGES,
+                                     data_ids=[str(i) for i in range(N_IMAGES)], chunk_ids=[0] * N_IMAGES,
+                                     num_chunks=[1] * N_IMAGES, receiver_ranks=[None] * N_IMAGES, data=dict(data))
+            pending = worker.upload(mk())
+            for _ in range(2):                           # warm-up of both pinned output buffers
+                worker.download(worker.execute_model(worker.upload(mk()))).wait()
+            torch.cuda.synchronize()
+            in_flight = None
+            t0 = time.perf_counter()
+            for _ in range(n):
+                nxt = worker.upload(mk())
+                started = worker.download(worker.execute_model(pending))
+                if in_flight is not None:
+                    in_flight.wait()
+                in_flight, pending = started, nxt
+            in_flight.wait()
+            torch.cuda.synchronize()
+            ms = (time.perf_counter() - t0) / n * 1e3
+            worker.execute_model(pending)
+            torch.cuda.synchronize()
+            return ms
+
+        duplex_ms = full_duplex_ms(host_batch)
         # latency of a batch of one: a single image of the same size, resident in HBM (the serving case when the
         # queue is short; the N = 1280 GEMMs then run on a quarter of the compute units)
         one_px, one_grid = pixel_values[: GRID[1] * GRID[2]], grid_np[:1]
@@ -525,6 +554,11 @@ def main() -> None:
         "fp32_pixel_values_ms_per_step": ahead_ms, "uint8_frames_ms_per_step": ahead_frames_ms,
         "note": "steady state of Worker.upload(batch k+1) issued before Worker.execute_model(batch k): pinned staging "
                 "and the PCIe copy on a side stream overlap the encoder's work on the previous batch",
+    }
+    result["host_outputs_download_overlap"] = {
+        "fp32_pixel_values_in_embeddings_out_ms_per_step": duplex_ms,
+        "note": "steady state with both copies off the critical path: Worker.upload(batch k+1) ahead of batch k, and "
+                "Worker.download of batch k's embeddings (14.7 MB, pinned host memory, side stream) while batch k+1 computes",
     }
     result["single_image"] = {"ms": one_ms, "patches": GRID[1] * GRID[2],
                               "note": "one 448x448 image alone (1024 patches), inputs resident in HBM"}

@@ -14,6 +14,13 @@ reference's executor test harness without a running sidecar.
 `Worker.upload` is this build's addition on the inbound side: it starts the host-to-device copy of a batch's
 pixel tensors (floating point or uint8) on a side stream through pinned staging buffers, so that the copy of batch k+1 runs while the encoder works
 on batch k; `execute_model` then makes the compute stream wait for that copy only.
+
+`Worker.download` is the outbound counterpart for the copy the reference's sidecar SERVER performs after it has opened
+the IPC handle: device-to-host into its shared-memory slot on a stream of its own (services/sidecar/sender.py:498-529,
+`buffer.data.copy_(data, non_blocking=True)` under `torch.cuda.stream(stream)`).  Here the copy of batch k's
+embeddings goes into pinned host memory on a side stream while batch k+1 computes.  The embeddings themselves stay
+exportable the way the reference's client exports them (`reduce_tensor`, sidecar/serde.py:89-95): contiguous row
+slices of one allocation of torch's caching allocator.
 """
 
 from __future__ import annotations
@@ -73,6 +80,22 @@ class MockSidecar:
             path.write_text(json.dumps(data))
 
 
+class Download:
+    """Embeddings on their way to pinned host memory (see Worker.download)."""
+
+    def __init__(self, host: list[torch.Tensor], done: "torch.cuda.Event") -> None:
+        self._host, self._done = host, done
+
+    def ready(self) -> bool:
+        return self._done.query()
+
+    def wait(self) -> list[torch.Tensor]:
+        """Block until the copies have landed; the host tensors (views of one pinned buffer) stay valid until the
+        second `Worker.download` call after the one that returned this object."""
+        self._done.synchronize()
+        return self._host
+
+
 class Worker:
     """Runs batches through one encoder and forwards the embeddings (reference: Worker.execute_model)."""
 
@@ -82,6 +105,45 @@ class Worker:
             sender_sidecar_client = MockSidecar()
         self.sender_sidecar_client = sender_sidecar_client
         self._copy_stream: torch.cuda.Stream | None = None
+        self._d2h_stream: torch.cuda.Stream | None = None
+        self._d2h_slots: list[torch.Tensor | None] = [None, None]   # two pinned buffers, used alternately
+        self._d2h_turn = 0
+
+    def download(self, embeddings: list[torch.Tensor]) -> Download:
+        """Start copying a batch's embeddings to pinned host memory on a side stream (default priority) and return at
+        once: the copy waits for the kernels that produce the embeddings (an event on the compute stream) and runs
+        while the next batch computes.  Two pinned buffers are used alternately and grown on demand, so the steady
+        state allocates nothing."""
+        device = self.model.device
+        if device.type != "cuda":
+            raise RuntimeError("download needs the model on a GPU")
+        if self._d2h_stream is None:
+            self._d2h_stream = torch.cuda.Stream(device=device)
+        for e in embeddings:
+            if not (isinstance(e, torch.Tensor) and e.is_cuda and e.is_contiguous()):
+                raise ValueError("download takes contiguous device tensors")
+        sizes = [(e.numel() * e.element_size() + 255) // 256 * 256 for e in embeddings]
+        total = max(sum(sizes), 256)
+        turn = self._d2h_turn
+        self._d2h_turn ^= 1
+        slot = self._d2h_slots[turn]
+        if slot is None or slot.numel() < total:
+            slot = self._d2h_slots[turn] = torch.empty((total,), dtype=torch.uint8, pin_memory=True)
+        compute = torch.cuda.current_stream(device)
+        produced = torch.cuda.Event()
+        produced.record(compute)
+        host, offset = [], 0
+        with torch.cuda.stream(self._d2h_stream):
+            self._d2h_stream.wait_event(produced)
+            for e, size in zip(embeddings, sizes):
+                dst = slot[offset : offset + e.numel() * e.element_size()].view(e.dtype).view(e.shape)
+                dst.copy_(e, non_blocking=True)
+                e.record_stream(self._d2h_stream)
+                host.append(dst)
+                offset += size
+            done = torch.cuda.Event()
+            done.record(self._d2h_stream)
+        return Download(host, done)
 
     def upload(self, batch: WorkerBatch) -> WorkerBatch:
         """Start copying the batch's host tensors to the model's device and return at once.  Every host tensor is

@@ -260,6 +260,71 @@ def test_scheduler_upload_ahead_pipeline(dev):
     assert seen == [f"d{i}" for i in range(6)] and finished == ["r0", "r1", "r2"] and not s.has_waiting_requests()
 
 
+def test_embeddings_survive_ipc_export(dev):
+    """What the reference's sidecar client does with every embedding (sidecar/api.py:235-261, serde.py:89-95): make it
+    flat, export it with `reduce_tensor` (an IPC memory handle plus offset into the allocation) and let another
+    process open it.  The encoders return row slices of ONE output buffer, so every item shares an allocation at a
+    different offset; a fresh child process (spawned, no GPU use before) must read back exactly the parent's bytes."""
+    import multiprocessing as mp
+
+    from torch.multiprocessing.reductions import reduce_tensor
+
+    from tests.ipc_child import main as child_main
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=17)
+    px, grid = synth.qwen_inputs([(1, 16, 16), (1, 8, 12), (2, 4, 4)], seed=17)
+    out = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    flat = [o.view(-1) for o in out]                     # api.py:239-242
+    assert all(o.is_contiguous() for o in out)
+    torch.cuda.synchronize()
+    want = [f.cpu().view(torch.uint8).numpy().tobytes() for f in flat]
+    payload = [reduce_tensor(f) for f in flat]
+    assert len({f.untyped_storage().data_ptr() for f in flat}) == 1 and len({f.data_ptr() for f in flat}) == 3
+    ctx = mp.get_context("spawn")
+    parent_end, child_end = ctx.Pipe()
+    proc = ctx.Process(target=child_main, args=(child_end,), daemon=True)
+    proc.start()
+    try:
+        parent_end.send(payload)
+        assert parent_end.poll(100), "the child did not answer"
+        status, got = parent_end.recv()
+    finally:
+        proc.join(20)
+        if proc.is_alive():
+            proc.kill()
+    assert status == "ok", got
+    assert got == want
+    torch.cuda.ipc_collect()                             # api.py:260-261
+
+
+def test_worker_download_overlaps_and_matches(dev):
+    """Embeddings copied to pinned host memory on the side stream equal the device tensors, across alternating
+    buffers and batches of different sizes, with the next batch enqueued before the previous download is awaited."""
+    from cornserve_amd.eric.worker import Worker, WorkerBatch
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=18)
+    worker = Worker(model)
+    sets = [[(1, 16, 16), (1, 8, 12)], [(1, 32, 32)], [(2, 4, 4), (1, 4, 6), (1, 12, 8)], [(1, 8, 8)]]
+    pending, results = None, []
+    for i, grids in enumerate(sets):
+        px, grid = synth.qwen_inputs(grids, seed=30 + i)
+        out = worker.execute_model(WorkerBatch(modality=Modality.IMAGE, adapter_name="", request_ids=["r"] * len(grids),
+                                               data_ids=[f"d{j}" for j in range(len(grids))], chunk_ids=[0] * len(grids),
+                                               num_chunks=[1] * len(grids), receiver_ranks=[None] * len(grids),
+                                               data={"pixel_values": px, "image_grid_thw": grid}))
+        started = worker.download(out)
+        if pending is not None:
+            host = pending[0].wait()
+            results.append(all(h.is_pinned() and torch.equal(h, o.cpu()) for h, o in zip(host, pending[1])))
+        pending = (started, out)
+    host = pending[0].wait()
+    assert pending[0].ready()
+    results.append(all(torch.equal(h, o.cpu()) for h, o in zip(host, pending[1])))
+    assert results == [True] * len(sets)
+    with pytest.raises(ValueError):
+        worker.download([torch.zeros(3)])
+
+
 def test_worker_hand_off_of_real_embeddings(dev, tmp_path):
     """Embeddings of a real forward pass through the worker's hand-off to the mock sidecar: contiguous device
     tensors (what the reference's sender exports by IPC handle), saved and reloaded bit-exactly."""
