@@ -160,7 +160,8 @@ class SiglipEncoderBase(EricModel):
     def _init_tower(self, fold_norm: bool) -> None:
         vc = self.config.vision_config
         self.fold_norm = (bool(fold_norm) and vc.hidden_size % 64 == 0 and 192 <= vc.hidden_size <= 160 * ops.SUMSQ_PARTS
-                          and getattr(vc, "hidden_act", "gelu_pytorch_tanh") == "gelu_pytorch_tanh")
+                          and getattr(vc, "hidden_act", "gelu_pytorch_tanh") == "gelu_pytorch_tanh"
+                          and vc.intermediate_size > 128)   # fc2's K, padded to a multiple of 64, must be at least 192
         self._packed: dict | None = None
         self.register_load_state_dict_post_hook(lambda module, incompatible: setattr(module, "_packed", None))
 
@@ -242,6 +243,10 @@ class SiglipEncoderBase(EricModel):
         d = H // nh
         B = pixel_values.shape[0]
         tokens = (vc.image_size // vc.patch_size) ** 2
+        if self.fold_norm:   # 32-bit operand offsets in the folded-norm GEMMs: a batch beyond them runs as several
+            most = max(1, ((2**32 - 1) // (2 * max(3 * H, pk["ip"]))) // tokens)
+            if B > most:
+                return torch.cat([self.vision_tower_forward(pixel_values[i : i + most]) for i in range(0, B, most)])
         M = B * tokens
         patches = ops.patchify_nchw(pixel_values.contiguous(), vc.patch_size, pk["kp"])
         x = ops.gemm(patches, pk["pe_w"], pk["pe_b"], pos=pk["pos"])
@@ -264,9 +269,6 @@ class SiglipEncoderBase(EricModel):
             lo = torch.zeros(x.shape, dtype=torch.uint8, device=x.device)
             stats_out = {"residual_lo": lo, "out_lo": lo}
         if fold:
-            if M * max(3 * H, pk["ip"]) * 2 >= 2**32:
-                raise ValueError(f"{M} tokens in one forward exceed what the folded-norm GEMMs address; split the batch "
-                                 "or construct the model with fold_norm=False")
             ss = torch.zeros((M, ops.SUMSQ_PARTS), dtype=torch.float32, device=x.device)
             sm = torch.zeros_like(ss)
             ops.row_stats(x, ss, sm)

@@ -199,6 +199,34 @@ class QwenVisionBase(EricModel):
             row += gt * gh * gw
         return px, grid
 
+    @staticmethod
+    def _addressable_groups(grid_thw: np.ndarray, max_rows: int) -> list[tuple[int, int]]:
+        """Consecutive item ranges [first, last) of at most `max_rows` patches each (items are independent, so a batch
+        can run as several); one range when the whole batch fits.  An item above the limit on its own is refused."""
+        g = np.asarray(grid_thw, dtype=np.int64).reshape(-1, 3)
+        rows = g[:, 0] * g[:, 1] * g[:, 2]
+        if int(rows.sum()) <= max_rows:
+            return [(0, len(rows))]
+        groups, first, acc = [], 0, 0
+        for i, r in enumerate(rows.tolist()):
+            if r > max_rows:
+                raise ValueError(f"item {i} has {r} patches, more than the {max_rows} the folded-norm GEMMs address; "
+                                 "construct the model with fold_norm=False")
+            if acc + r > max_rows:
+                groups.append((first, i))
+                first, acc = i, 0
+            acc += r
+        groups.append((first, len(rows)))
+        return groups
+
+    def _forward_in_groups(self, pixel_values: torch.Tensor, grid_thw: np.ndarray, groups, mark) -> list[torch.Tensor]:
+        g = np.asarray(grid_thw, dtype=np.int64).reshape(-1, 3)
+        starts = np.concatenate([[0], np.cumsum(g[:, 0] * g[:, 1] * g[:, 2])])
+        out: list[torch.Tensor] = []
+        for first, last in groups:
+            out += self.forward_device(pixel_values[int(starts[first]):int(starts[last])], g[first:last], mark)
+        return out
+
     @torch.inference_mode()
     def forward(self, modality: Modality, adapter_name: str, batch: dict[str, list[torch.Tensor]]) -> list[torch.Tensor]:
         """See the reference docstring (:402-413): `pixel_values` + `image_grid_thw` for images,
@@ -255,7 +283,10 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
             raise NotImplementedError("only the SiLU-gated MLP of Qwen2.5-VL is implemented")
         self.head_dim = self.hidden_size // self.num_heads
         H = self.hidden_size
-        self.fold_norm = bool(fold_norm) and weight_format == "bf16" and H % 64 == 0 and 192 <= H <= 160 * ops.SUMSQ_PARTS
+        # (the folded forms exist in the direct-to-LDS GEMM only: bf16 weights, K a multiple of 64 and at least 192 for
+        # both the hidden and the padded intermediate size, hidden size within the row-sum parts)
+        self.fold_norm = (bool(fold_norm) and weight_format == "bf16" and H % 64 == 0 and 192 <= H <= 160 * ops.SUMSQ_PARTS
+                          and _round_up(self.intermediate_size, 64) >= 192)
 
         self.patch_embed = _PatchEmbed(self.in_channels, self.hidden_size, self.temporal_patch_size, self.patch_size)
         self.blocks = nn.ModuleList([_Block(self.hidden_size, self.intermediate_size) for _ in range(vc.depth)])
@@ -345,6 +376,11 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         win = self.window_size // merge // self.patch_size
         dev = self.device
 
+        # the folded-norm GEMMs address their operands with 32-bit byte offsets: a batch beyond that runs as several
+        if self.fold_norm:
+            groups = self._addressable_groups(grid_thw, (2**32 - 1) // (2 * max(3 * H, pk["Ip"])))
+            if len(groups) > 1:
+                return self._forward_in_groups(pixel_values, grid_thw, groups, mark)
         mark("index")
         ix, plan_win, plan_full, L = self._index(grid_thw)
         if pixel_values.shape[0] != L:
@@ -358,9 +394,6 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         n = torch.empty_like(x)
         # the folded-norm GEMMs exist in the fast kernel only, whose per-lane byte offsets are 32-bit
         fold = self.fold_norm
-        if fold and L * max(3 * H, pk["Ip"]) * 2 >= 2**32:
-            raise ValueError(f"{L} patches in one forward exceed what the folded-norm GEMMs address; split the batch "
-                             "or construct the model with fold_norm=False")
         eps = self.norm_eps
         if fold:
             mark("norm")

@@ -79,7 +79,10 @@ class Qwen2VisionTransformer(QwenVisionBase):
             raise ValueError(f"Unknown weight_format: {weight_format}")
         self.weight_format = weight_format
         E = vc.embed_dim
-        self.fold_norm = bool(fold_norm) and weight_format == "bf16" and E % 64 == 0 and 192 <= E <= 160 * ops.SUMSQ_PARTS
+        hidden = int(vc.embed_dim * vc.mlp_ratio)
+        # (the folded forms exist in the direct-to-LDS GEMM only: K a multiple of 64 and at least 192 on both sides)
+        self.fold_norm = (bool(fold_norm) and weight_format == "bf16" and E % 64 == 0 and 192 <= E <= 160 * ops.SUMSQ_PARTS
+                          and hidden % 64 == 0 and hidden >= 192)
         self.hidden_size = vc.hidden_size          # width of the merger's output (:307)
         self.embed_dim = vc.embed_dim
         self.num_heads = vc.num_heads
@@ -135,6 +138,10 @@ class Qwen2VisionTransformer(QwenVisionBase):
         pk = self._ensure_packed()
         E, nh, d, unit, dev = self.embed_dim, self.num_heads, self.head_dim, self.spatial_merge_unit, self.device
         eps = self.norm_eps
+        if self.fold_norm:   # 32-bit operand offsets in the folded-norm GEMMs: a batch beyond them runs as several
+            groups = self._addressable_groups(grid_thw, (2**32 - 1) // (2 * max(3 * E, self.mlp_hidden)))
+            if len(groups) > 1:
+                return self._forward_in_groups(pixel_values, grid_thw, groups, mark)
 
         # Rotary table (rot_pos_emb, :354-384) and one attention segment per frame (:423-426).  The index routines
         # are the Qwen2.5-VL ones with a window larger than any grid: one window per frame, i.e. no permutation.
@@ -162,9 +169,6 @@ class Qwen2VisionTransformer(QwenVisionBase):
             lo = torch.zeros(x.shape, dtype=torch.uint8, device=dev)
             res = {"residual_lo": lo, "out_lo": lo}
         if fold:
-            if L * max(3 * E, self.mlp_hidden) * 2 >= 2**32:
-                raise ValueError(f"{L} patches in one forward exceed what the folded-norm GEMMs address; split the batch "
-                                 "or construct the model with fold_norm=False")
             mark("norm")
             ss = torch.zeros((L, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev)
             sm = torch.zeros_like(ss)

@@ -104,7 +104,7 @@ class Qwen3_VisionTransformer(QwenVisionBase):
         self.weight_format = weight_format
         E = vc.hidden_size
         self.fold_norm = (bool(fold_norm) and weight_format == "bf16" and E % 64 == 0 and 192 <= E <= 160 * ops.SUMSQ_PARTS
-                          and vc.hidden_act in ("gelu_pytorch_tanh", "quick_gelu"))
+                          and vc.hidden_act in ("gelu_pytorch_tanh", "quick_gelu") and vc.intermediate_size > 128)
         self.in_channels = vc.in_channels
         self.embed_dim = vc.hidden_size
         self.num_heads = vc.num_heads
@@ -191,6 +191,10 @@ class Qwen3_VisionTransformer(QwenVisionBase):
         pk = self._ensure_packed()
         E, nh, d, unit, dev = self.embed_dim, self.num_heads, self.head_dim, self.spatial_merge_unit, self.device
         eps, O = self.norm_eps, self.out_hidden_size
+        if self.fold_norm:   # 32-bit operand offsets in the folded-norm GEMMs: a batch beyond them runs as several
+            groups = self._addressable_groups(grid_thw, (2**32 - 1) // (2 * max(3 * E, self.intermediate_size + self.mlp_pad)))
+            if len(groups) > 1:
+                return self._forward_in_groups(pixel_values, grid_thw, groups, mark)
 
         # rotary table (:320-362) and one attention segment per frame (:288-291): the Qwen2.5-VL index routines
         # with a window larger than any grid, i.e. without the window permutation
@@ -218,9 +222,6 @@ class Qwen3_VisionTransformer(QwenVisionBase):
         kept: list[torch.Tensor] = []
         fold = self.fold_norm
         if fold:
-            if L * max(3 * E, self.intermediate_size + self.mlp_pad) * 2 >= 2**32:
-                raise ValueError(f"{L} patches in one forward exceed what the folded-norm GEMMs address; split the batch "
-                                 "or construct the model with fold_norm=False")
             mark("norm")
             ss = torch.zeros((L, ops.SUMSQ_PARTS), dtype=torch.float32, device=dev)
             sm = torch.zeros_like(ss)

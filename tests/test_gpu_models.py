@@ -84,6 +84,40 @@ def test_qwen_without_folded_norms(dev, golden_dir):
     check(out_f, out, REL_BF16, "folded vs unfolded")
 
 
+def test_qwen_shapes_the_folded_gemms_cannot_take(dev):
+    """A batch beyond the folded-norm GEMMs' 32-bit operand offsets runs as several item groups with the same bits,
+    and a configuration whose MLP is too narrow for them runs with the norms as their own kernels, instead of
+    raising (the reference has neither limit)."""
+    from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=3)
+    grids = [(1, 8, 12), (1, 16, 16), (2, 4, 4), (1, 4, 6), (1, 12, 8)]
+    px, grid = synth.qwen_inputs(grids, seed=3)
+    whole = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    g = torch.cat(grid).numpy().astype(np.int64)
+    groups = model._addressable_groups(g, 300)                # 96 | 256 + 32 | 24 + 96
+    assert groups == [(0, 1), (1, 3), (3, 5)] and model._addressable_groups(g, 10**9) == [(0, 5)]
+    dpx = torch.cat(px).to(device=dev, dtype=torch.bfloat16)
+    parts = model._forward_in_groups(dpx, g, groups, lambda name: None)
+    assert len(parts) == 5 and all(torch.equal(a, b) for a, b in zip(parts, whole))
+    with pytest.raises(ValueError, match="more than"):
+        model._addressable_groups(g, 200)
+    # intermediate size 96: padded to 128 < 192, which the direct-to-LDS GEMM (the one with the folded forms) refuses
+    cfg = synth.qwen_vision_config(depth=2, fullatt_block_indexes=(1,))
+    cfg.vision_config.intermediate_size = 96
+    sd = synth.qwen_state_dict(cfg, seed=4)
+    narrow = Qwen2_5_VisionTransformer(cfg)
+    narrow.load_state_dict(sd, strict=False)
+    narrow = narrow.to(device=dev, dtype=torch.bfloat16).eval()
+    assert not narrow.fold_norm
+    px, grid = synth.qwen_inputs([(1, 8, 12), (1, 4, 4)], seed=4)
+    out = narrow(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    ocfg = oq.QwenVisionConfig(depth=2, fullatt_block_indexes=[1], intermediate_size=96)
+    ref = oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
+    for o, r in zip(out, ref):
+        check(o, r, REL_BF16, "narrow MLP, unfolded")
+
+
 def test_qwen_uint8_frames_equal_float_pixel_values(dev):
     """The uint8-frame input format gives bit-identical embeddings to the reference's format fed with what the
     image processor makes of the same frames (oracle restatement of the processor)."""

@@ -505,6 +505,31 @@ def test_gemm_with_folded_layernorm(ops, dev, M, N, K):
         torch.testing.assert_close(m2.cpu(), pad.view(M, 8, 160).sum(-1), rtol=1e-5, atol=1e-4)
 
 
+@pytest.mark.parametrize("offset", [64.0, -100.0])
+def test_gemm_with_folded_layernorm_on_rows_with_a_large_common_offset(ops, dev, offset):
+    """The folded LayerNorm forms the variance as sumsq/K - mean^2 from fp32 sums, and the mean term as
+    acc - mean * colsum: both cancel when a row's mean is far larger than its spread (mean / std of 64 and 100 here,
+    where two thirds of the bits of sumsq/K cancel).  Checked against LayerNorm + linear on the same bf16 rows (the
+    reference's sequence, siglip.py:173-175 then F.linear) at the encoder tolerance."""
+    M, N, K, eps = 1000, 1280, 1152, 1e-6
+    a = (rnd((M, K), 1.0, 81).float() + offset).bfloat16().to(dev)
+    w, b = rnd((N, K), 0.05, 82, dev), rnd((N,), 0.02, 83, dev)
+    g, beta = (1.0 + rnd((K,), 0.1, 84)).bfloat16(), rnd((K,), 0.1, 85)
+    wf = (w.float().cpu() * g.float()[None, :]).bfloat16()
+    bf = (b.float().cpu() + (w.float().cpu() * beta.float()[None, :]).sum(1)).bfloat16()
+    csum = wf.float().sum(dim=1).contiguous()
+    ss = torch.empty((M, 8), dtype=torch.float32, device=dev)
+    sm = torch.empty_like(ss)
+    ops.row_stats(a, ss, sm)
+    af = a.float().cpu()
+    assert (af.mean(1).abs() / af.std(1)).min() > 50          # the case this test is about
+    ref = lin_ref(F.layer_norm(af, (K,), g.float(), beta.float(), eps).bfloat16(), w, b)
+    got = ops.gemm(a, wf.to(dev), bf.to(dev), a_row_sumsq=ss, a_row_sum=sm, w_col_sum=csum.to(dev), norm_eps=eps).float().cpu()
+    cos = F.cosine_similarity(got.flatten(), ref.flatten(), dim=0).item()
+    rel = ((got - ref).abs().max() / ref.abs().max()).item()
+    assert cos >= 0.999 and rel <= 2e-2, (cos, rel)
+
+
 def test_gemm_row_maps(ops, dev):
     M, N, K = 400, 512, 256
     a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
