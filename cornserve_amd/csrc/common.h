@@ -16,6 +16,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(int)))) int i32x2_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;
+typedef __attribute__((__vector_size__(4 * sizeof(uint32_t)))) uint32_t u32x4_t;
 
 #define CS_DEVICE __device__ __forceinline__
 

@@ -12,13 +12,13 @@
 // consecutive columns n: epilogues that pair adjacent columns (SwiGLU on interleaved gate|up) and
 // 8-byte packed stores fall out of that.
 //
-// Epilogues (all optional-bias, fp32 accumulate, rounding points follow the reference's bf16 steps):
+// Epilogues (all optional-bias, fp32 accumulate; an activation takes the fp32 sum and the result is rounded once,
+// where the reference, computing in bf16, also rounds the linear layer's output in between):
 //   EPI_BIAS       y = bf16(acc + b)
 //   EPI_RESIDUAL   y = bf16( bf16(acc + b) + r )                     (qwen2_5_vl.py:175,177)
-//   EPI_SWIGLU     y[j] = bf16( silu(bf16(acc[2j]+b[2j])) * bf16(acc[2j+1]+b[2j+1]) )
-//                                                                    (qwen2_5_vl.py:143-148)
-//   EPI_GELU_ERF   y = bf16(gelu_erf(bf16(acc + b)))                 (qwen2_5_vl.py:218-222)
-//   EPI_GELU_TANH  y = bf16(gelu_tanh(bf16(acc + b)))                (siglip.py:155-163)
+//   EPI_SWIGLU     y[j] = bf16( silu(acc[2j]+b[2j]) * (acc[2j+1]+b[2j+1]) )   (qwen2_5_vl.py:143-148)
+//   EPI_GELU_ERF   y = bf16(gelu_erf(acc + b))                       (qwen2_5_vl.py:218-222)
+//   EPI_GELU_TANH  y = bf16(gelu_tanh(acc + b))                      (siglip.py:155-163)
 // plus an optional fp32 per-output-channel scale applied to acc (fp8-e4m3 weights, W_FP8 = true), an
 // optional gather of A rows (a_rows) and scatter of C rows (c_rows) used to fuse the window permutation
 // (qwen2_5_vl.py:438-440) and its inverse (:478-479) into the neighbouring GEMMs, and an optional second

@@ -62,10 +62,9 @@ CS_DEVICE void epilogue(const CsGemmArgs& p, const f32x16_t (&acc)[MT][NT], int 
           for (int q = 0; q < 4; ++q) v[q] += bf2f(b[q]);
         }
         if (EPI == CS_EPI_SWIGLU) {
-          // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the product stay
-          // in fp32 until the single output rounding (the same rounding points as the direct-to-LDS kernel)
-          const float gate0 = silu(rbf(v[0])), up0 = rbf(v[1]);
-          const float gate1 = silu(rbf(v[2])), up1 = rbf(v[3]);
+          // SiLU(gate) * up on the fp32 sums with one rounding of the product (the same as the direct-to-LDS kernel)
+          const float gate0 = silu(v[0]), up0 = v[1];
+          const float gate1 = silu(v[2]), up1 = v[3];
           bf16x2_t o;
           o[0] = f2bf(gate0 * up0);
           o[1] = f2bf(gate1 * up1);
@@ -73,13 +72,13 @@ CS_DEVICE void epilogue(const CsGemmArgs& p, const f32x16_t (&acc)[MT][NT], int 
         } else {
           if (EPI == CS_EPI_GELU_ERF) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = gelu_erf(rbf(v[q]));
+            for (int q = 0; q < 4; ++q) v[q] = gelu_erf(v[q]);
           } else if (EPI == CS_EPI_GELU_TANH) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = gelu_tanh(rbf(v[q]));
+            for (int q = 0; q < 4; ++q) v[q] = gelu_tanh(v[q]);
           } else if (EPI == CS_EPI_QUICK_GELU) {
 #pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = quick_gelu(rbf(v[q]));
+            for (int q = 0; q < 4; ++q) v[q] = quick_gelu(v[q]);
           } else if (EPI == CS_EPI_RESIDUAL) {
             const bf16x4_t r = *(const bf16x4_t*)(pRes + (int64_t)m * p.ldr + n);
             if (p.c_lo) {  // residual stream with 16 significant bits: join, add unrounded, split

@@ -69,6 +69,16 @@ constexpr int WAITCNT_LGKM0 = 0xC07F;                                           
 
 typedef __attribute__((address_space(3))) void lds_void_t;
 
+// Buffer accesses: a scalar descriptor, one 32-bit byte offset per lane and an immediate, so that an address costs no
+// 64-bit vector arithmetic.  (Plain functions on purpose: the device-only builtins must not sit in generic lambdas.)
+CS_DEVICE u32x4_t buf_ld_u32x4(__amdgpu_buffer_rsrc_t r, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0); }
+CS_DEVICE u32x2_t buf_ld_u32x2(__amdgpu_buffer_rsrc_t r, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b64(r, off, 0, 0); }
+CS_DEVICE uint32_t buf_ld_u32(__amdgpu_buffer_rsrc_t r, uint32_t off) { return __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0); }
+CS_DEVICE f32x4_t buf_ld_f32x4(__amdgpu_buffer_rsrc_t r, uint32_t off) { return __builtin_bit_cast(f32x4_t, buf_ld_u32x4(r, off)); }
+CS_DEVICE void buf_st_u32x4(__amdgpu_buffer_rsrc_t r, uint32_t off, u32x4_t v) { __builtin_amdgcn_raw_buffer_store_b128(v, r, off, 0, 0); }
+CS_DEVICE void buf_st_u32x2(__amdgpu_buffer_rsrc_t r, uint32_t off, u32x2_t v) { __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, 0); }
+CS_DEVICE void buf_st_u32(__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t v) { __builtin_amdgcn_raw_buffer_store_b32(v, r, off, 0, 0); }
+
 // Workgroup barrier without the full memory fence of __syncthreads(): the callers order LDS traffic with
 // explicit waits, and the asm statements keep the compiler from moving memory operations across it.
 CS_DEVICE void wg_barrier() {
@@ -229,6 +239,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   };
   const __amdgpu_buffer_rsrc_t rsrc_a = __builtin_amdgcn_make_buffer_rsrc((void*)p.A, 0, -1, 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc((void*)p.W, 0, -1, 0x00020000);
+  // descriptors of what the epilogue's fast form reads and writes
+  const __amdgpu_buffer_rsrc_t rsrc_c = __builtin_amdgcn_make_buffer_rsrc((void*)p.C, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_clo = __builtin_amdgcn_make_buffer_rsrc((void*)p.c_lo, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_res = __builtin_amdgcn_make_buffer_rsrc((void*)p.residual, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_reslo = __builtin_amdgcn_make_buffer_rsrc((void*)p.residual_lo, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_bias = __builtin_amdgcn_make_buffer_rsrc((void*)p.bias, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_asumsq = __builtin_amdgcn_make_buffer_rsrc((void*)p.a_row_sumsq, 0, -1, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_asum = __builtin_amdgcn_make_buffer_rsrc((void*)p.a_row_sum, 0, -1, 0x00020000);
   // (The builtin is called from non-generic lambdas on purpose: inside a generic lambda the host pass of the
   // compiler rejects the device-only builtin, silently drops the kernel and leaves its launch stub undefined.)
   auto load_a = [&](int kt, char* lds_dst, uint32_t off) {
@@ -446,11 +464,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
 
     // ---- epilogue.  Accumulator (i, j), element r = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
     //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
-    //      The loads the epilogue needs (row map, bias, residual / position rows) are issued ahead of the
-    //      stores that follow them, from clamped addresses so that no branch guards a load: a load inside the
-    //      store loop would make the compiler wait for ALL outstanding memory operations (vmcnt counts stores
-    //      too), i.e. for every store issued so far and for the next tile's prefetch, once per row block.
-    {
+    //      With one wave per SIMD nothing overlaps the epilogue and it is bound by instruction issue (a vector
+    //      instruction every four to five clocks), so it comes in two forms.  FAST: the tile lies inside the matrix
+    //      and rows are not scattered -- no guards, no clamps, and every access is a buffer instruction (scalar
+    //      descriptor + one 32-bit lane offset + an immediate), so an address costs no vector arithmetic.  General:
+    //      edge tiles and scattered rows, with guards and 64-bit addresses.  In both, the loads the epilogue needs
+    //      (row map, bias, residual / position rows) are issued ahead of the stores that follow them: a load inside the
+    //      store loop would make the compiler wait for ALL outstanding memory operations (vmcnt counts stores too),
+    //      i.e. for every store issued so far and for the next tile's prefetch, once per row block.
+    auto epilogue = [&](auto fast_c) {
+      constexpr bool FAST = decltype(fast_c)::value;
       const bf16_t* const pBias = (const bf16_t*)p.bias;
       bf16_t* const pC = (bf16_t*)p.C;
       // The lane's column and row are re-derived behind an opaque copy of the lane number: otherwise the compiler
@@ -460,27 +483,41 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       asm volatile("" : "+v"(lane_e));
       const int fa = lane_e & 15, kq = lane_e >> 4;
       const int n_lane = n0 + wn * WTN + kq * (4 * G);
+      const int m_lane = m0 + wm * WTM + fa;   // the lane's row of row block 0; block i is 16 i rows further
       int mrow[MT];
       int crow[MT];  // 32-bit row numbers; the 64-bit address is formed at the store
 #pragma unroll
       for (int i = 0; i < MT; ++i) {
-        mrow[i] = m0 + wm * WTM + i * 16 + fa;
-        const int mc = min(mrow[i], p.M - 1);
-        crow[i] = p.c_rows ? p.c_rows[mc] : mc;
+        mrow[i] = m_lane + i * 16;
+        if constexpr (FAST) {
+          crow[i] = mrow[i];
+        } else {
+          const int mc = min(mrow[i], p.M - 1);
+          crow[i] = p.c_rows ? p.c_rows[mc] : mc;
+        }
       }
+      auto clamp_m = [&](int m) { return FAST ? m : min(m, p.M - 1); };
+      auto clamp_n = [&](int n) { return FAST ? n : min(n, p.N - 4); };
       constexpr bool NORM_A = FUSE == FUSE_NORM_A || FUSE == FUSE_LN_A;
       float rstd[NORM_A ? MT : 1];
       float nmean_rstd[FUSE == FUSE_LN_A ? MT : 1];   // -mean * rstd
+      auto total8 = [&](const float* base, const __amdgpu_buffer_rsrc_t rs, int row) {
+        f32x4_t s0, s1;
+        if constexpr (FAST) {
+          s0 = buf_ld_f32x4(rs, (uint32_t)row * (CS_SUMSQ_PARTS * 4));
+          s1 = buf_ld_f32x4(rs, (uint32_t)row * (CS_SUMSQ_PARTS * 4) + 16);
+        } else {
+          const float* parts = base + (int64_t)row * CS_SUMSQ_PARTS;
+          s0 = *(const f32x4_t*)parts;
+          s1 = *(const f32x4_t*)(parts + 4);
+        }
+        return ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
+      };
       if constexpr (FUSE == FUSE_LN_A) {
-        auto total = [](const float* parts) {
-          const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
-          return ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
-        };
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-          const int64_t row = (int64_t)min(mrow[i], p.M - 1) * CS_SUMSQ_PARTS;
-          const float mean = total(p.a_row_sum + row) / (float)p.K;
-          const float var = fmaxf(total(p.a_row_sumsq + row) / (float)p.K - mean * mean, 0.f);
+          const float mean = total8(p.a_row_sum, rsrc_asum, clamp_m(mrow[i])) / (float)p.K;
+          const float var = fmaxf(total8(p.a_row_sumsq, rsrc_asumsq, clamp_m(mrow[i])) / (float)p.K - mean * mean, 0.f);
           rstd[i] = rsqrtf(var + p.norm_eps);
           nmean_rstd[i] = -mean * rstd[i];
         }
@@ -488,28 +525,29 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       if constexpr (FUSE == FUSE_NORM_A) {
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
-          const float* parts = p.a_row_sumsq + (int64_t)min(mrow[i], p.M - 1) * CS_SUMSQ_PARTS;
-          const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
-          const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
+          const float ss = total8(p.a_row_sumsq, rsrc_asumsq, clamp_m(mrow[i]));
           rstd[i] = rsqrtf(ss / (float)p.K + p.norm_eps);
         }
       }
       f32x4_t csum_v[FUSE == FUSE_LN_A ? NT : 1];
       if constexpr (FUSE == FUSE_LN_A) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) csum_v[j] = *(const f32x4_t*)(p.w_col_sum + min(n_lane + piece_col(j), p.N - 4));
+        for (int j = 0; j < NT; ++j) csum_v[j] = *(const f32x4_t*)(p.w_col_sum + clamp_n(n_lane + piece_col(j)));
       }
       bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
 #pragma unroll
       for (int j = 0; j < NT; ++j) {
-        const int nc = min(n_lane + piece_col(j), p.N - 4);
         bias_v[j] = bf16x4_t{0, 0, 0, 0};
-        if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + nc);
+        if constexpr (FAST) {
+          if (pBias) bias_v[j] = __builtin_bit_cast(bf16x4_t, buf_ld_u32x2(rsrc_bias, (uint32_t)(n_lane + piece_col(j)) * 2));
+        } else {
+          if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + clamp_n(n_lane + piece_col(j)));
+        }
       }
       f32x4_t scale_v[W_FP8 ? NT : 1];
       if constexpr (W_FP8) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j) scale_v[j] = *(const f32x4_t*)(p.w_scale + min(n_lane + piece_col(j), p.N - 4));
+        for (int j = 0; j < NT; ++j) scale_v[j] = *(const f32x4_t*)(p.w_scale + clamp_n(n_lane + piece_col(j)));
       }
       constexpr bool ADDEND = (EPI == CS_EPI_RESIDUAL) || (EPI == CS_EPI_BIAS_POS);
       // SPLIT: the residual stream is carried with 16 significant bits (bf16 plane + byte plane, see split24)
@@ -518,18 +556,50 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       uint32_t addend_lo[SPLIT ? MT : 1][SPLIT ? NT : 1];   // the four bytes of a piece
       auto load_addend = [&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
-        const int mc = min(mrow[i], p.M - 1);
-        const bf16_t* row = (EPI == CS_EPI_RESIDUAL)
-                                ? (const bf16_t*)p.residual + (int64_t)mc * p.ldr
-                                : (const bf16_t*)p.pos + (int64_t)(mc % p.pos_period) * p.ldpos;
+        if constexpr (FAST && EPI == CS_EPI_RESIDUAL) {
+          // lane offset of the row inside the residual matrix; the piece's column is an immediate of the instruction
+          const uint32_t off = (uint32_t)mrow[i] * (uint32_t)p.ldr + (uint32_t)n_lane;
+          if constexpr (G == 2) {
 #pragma unroll
-        for (int j = 0; j < NT; ++j)
-          addend[ADDEND ? i : 0][ADDEND ? j : 0] = *(const bf16x4_t*)(row + min(n_lane + piece_col(j), p.N - 4));
-        if constexpr (SPLIT) {
-          const uint8_t* row_lo = p.residual_lo + (int64_t)mc * p.ldr;
+            for (int j = 0; j < NT; j += 2) {
+              const u32x4_t w = buf_ld_u32x4(rsrc_res, (off + piece_col(j)) * 2);
+              addend[ADDEND ? i : 0][ADDEND ? j : 0] = __builtin_bit_cast(bf16x4_t, u32x2_t{w[0], w[1]});
+              addend[ADDEND ? i : 0][ADDEND ? j + 1 : 0] = __builtin_bit_cast(bf16x4_t, u32x2_t{w[2], w[3]});
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+              addend[ADDEND ? i : 0][ADDEND ? j : 0] = __builtin_bit_cast(bf16x4_t, buf_ld_u32x2(rsrc_res, (off + piece_col(j)) * 2));
+          }
+          if constexpr (SPLIT) {
+            if constexpr (G == 2) {
+#pragma unroll
+              for (int j = 0; j < NT; j += 2) {
+                u32x2_t w = {0u, 0u};
+                if (p.residual_lo) w = buf_ld_u32x2(rsrc_reslo, off + piece_col(j));
+                addend_lo[SPLIT ? i : 0][SPLIT ? j : 0] = w[0];
+                addend_lo[SPLIT ? i : 0][SPLIT ? j + 1 : 0] = w[1];
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < NT; ++j)
+                addend_lo[SPLIT ? i : 0][SPLIT ? j : 0] = p.residual_lo ? buf_ld_u32(rsrc_reslo, off + piece_col(j)) : 0u;
+            }
+          }
+        } else {
+          const int mc = clamp_m(mrow[i]);
+          const bf16_t* row = (EPI == CS_EPI_RESIDUAL)
+                                  ? (const bf16_t*)p.residual + (int64_t)mc * p.ldr
+                                  : (const bf16_t*)p.pos + (int64_t)(mc % p.pos_period) * p.ldpos;
 #pragma unroll
           for (int j = 0; j < NT; ++j)
-            addend_lo[SPLIT ? i : 0][SPLIT ? j : 0] = p.residual_lo ? *(const uint32_t*)(row_lo + min(n_lane + piece_col(j), p.N - 4)) : 0u;
+            addend[ADDEND ? i : 0][ADDEND ? j : 0] = *(const bf16x4_t*)(row + clamp_n(n_lane + piece_col(j)));
+          if constexpr (SPLIT) {
+            const uint8_t* row_lo = p.residual_lo + (int64_t)mc * p.ldr;
+#pragma unroll
+            for (int j = 0; j < NT; ++j)
+              addend_lo[SPLIT ? i : 0][SPLIT ? j : 0] = p.residual_lo ? *(const uint32_t*)(row_lo + clamp_n(n_lane + piece_col(j))) : 0u;
+          }
         }
       };
       // The kernel must stay inside the architectural registers (the accumulation registers are not the
@@ -544,7 +614,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       static_for<MT>([&](auto i_c) {
         constexpr int i = decltype(i_c)::value;
         if constexpr (ADDEND && i % ADD_BATCH == 0 && i > 0) load_addend_batch(ic<i / ADD_BATCH>{});
-        const bool mok = mrow[i] < p.M;
+        const bool mok = FAST || mrow[i] < p.M;
         f32x4_t racc[NT];
         static_for<NT * 4>([&](auto e_c) {
           constexpr int E = decltype(e_c)::value;
@@ -566,22 +636,21 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
             v[r] = t + bf2f(bias_v[j][r]);
           }
           if (EPI == CS_EPI_SWIGLU) {
-            // gate and up are rounded to bf16 like the reference's two F.linear outputs; SiLU and the
-            // product stay in fp32 until the single output rounding
-            const float g0 = silu(rbf(v[0])), u0 = rbf(v[1]);
-            const float g1 = silu(rbf(v[2])), u1 = rbf(v[3]);
-            out[j][0] = f2bf(g0 * u0);
-            out[j][1] = f2bf(g1 * u1);
+            // SiLU(gate) * up on the fp32 sums, one rounding of the product (the reference rounds gate, SiLU(gate)
+            // and up to bf16 on the way, qwen2_5_vl.py:143-148: three roundings this epilogue does not spend
+            // instructions on)
+            out[j][0] = f2bf(silu(v[0]) * v[1]);
+            out[j][1] = f2bf(silu(v[2]) * v[3]);
           } else {
             if (EPI == CS_EPI_GELU_ERF) {
 #pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = gelu_erf(rbf(v[r]));
+              for (int r = 0; r < 4; ++r) v[r] = gelu_erf(v[r]);
             } else if (EPI == CS_EPI_GELU_TANH) {
 #pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(rbf(v[r]));
+              for (int r = 0; r < 4; ++r) v[r] = gelu_tanh(v[r]);
             } else if (EPI == CS_EPI_QUICK_GELU) {
 #pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] = quick_gelu(rbf(v[r]));
+              for (int r = 0; r < 4; ++r) v[r] = quick_gelu(v[r]);
             } else if (ADDEND && !SPLIT) {
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] = rbf(v[r]) + bf2f(addend[ADDEND ? i : 0][ADDEND ? j : 0][r]);
@@ -599,12 +668,13 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         }
         if constexpr (FUSE == FUSE_SUMSQ_C || FUSE == FUSE_STATS_C) {
           // Sum of squares of the row's ROUNDED outputs over this wave's columns: lane-local over the lane's
-          // pieces, then over the four lanes of the row (fixed order: the result does not depend on timing).
+          // pieces, then over the four lanes of the row (fixed order: the result does not depend on timing, and
+          // neither form of the epilogue changes it: a piece outside the matrix adds exact zeros).
           static_assert(WAVES_N == 1 && EPI != CS_EPI_SWIGLU, "one wave spans the tile's columns: one part per tile");
           float ss = 0.f, sm = 0.f;
 #pragma unroll
           for (int j = 0; j < NT; ++j) {
-            const bool nok = n_lane + piece_col(j) < p.N;
+            const bool nok = FAST || n_lane + piece_col(j) < p.N;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const float o = nok ? bf2f(out[j][r]) : 0.f;
@@ -623,7 +693,46 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         }
         // With G == 2 the pieces of fragments 2g and 2g+1 are adjacent: one 16-byte store per lane, and the
         // four lanes of an output row write 64 consecutive bytes (32 with the halved SwiGLU output).
-        if (EPI == CS_EPI_SWIGLU) {
+        if constexpr (FAST) {
+          if (EPI == CS_EPI_SWIGLU) {
+            const uint32_t off = ((uint32_t)mrow[i] * (uint32_t)p.ldc + (uint32_t)(n_lane >> 1)) * 2;
+            if constexpr (G == 2) {
+#pragma unroll
+              for (int j = 0; j < NT; j += 2) {
+                const bf16x4_t o = {out[j][0], out[j][1], out[j + 1][0], out[j + 1][1]};
+                buf_st_u32x2(rsrc_c, off + (piece_col(j) >> 1) * 2, __builtin_bit_cast(u32x2_t, o));
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < NT; ++j) {
+                const bf16x2_t o = {out[j][0], out[j][1]};
+                buf_st_u32(rsrc_c, off + (piece_col(j) >> 1) * 2, __builtin_bit_cast(uint32_t, o));
+              }
+            }
+          } else {
+            const uint32_t off = (uint32_t)mrow[i] * (uint32_t)p.ldc + (uint32_t)n_lane;   // in elements
+            if constexpr (G == 2) {
+#pragma unroll
+              for (int j = 0; j < NT; j += 2) {
+                const u32x2_t a0 = __builtin_bit_cast(u32x2_t, out[j]), a1 = __builtin_bit_cast(u32x2_t, out[j + 1]);
+                buf_st_u32x4(rsrc_c, (off + piece_col(j)) * 2, u32x4_t{a0[0], a0[1], a1[0], a1[1]});
+              }
+            } else {
+#pragma unroll
+              for (int j = 0; j < NT; ++j) buf_st_u32x2(rsrc_c, (off + piece_col(j)) * 2, __builtin_bit_cast(u32x2_t, out[j]));
+            }
+            if constexpr (SPLIT) {
+              if constexpr (G == 2) {
+#pragma unroll
+                for (int j = 0; j < NT; j += 2)
+                  buf_st_u32x2(rsrc_clo, off + piece_col(j), u32x2_t{out_lo[SPLIT ? j : 0], out_lo[SPLIT ? j + 1 : 0]});
+              } else {
+#pragma unroll
+                for (int j = 0; j < NT; ++j) buf_st_u32(rsrc_clo, off + piece_col(j), out_lo[SPLIT ? j : 0]);
+              }
+            }
+          }
+        } else if (EPI == CS_EPI_SWIGLU) {
           bf16_t* dst = pC + (int64_t)crow[i] * p.ldc + (n_lane >> 1);
           if constexpr (G == 2) {
 #pragma unroll
@@ -677,7 +786,10 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           }
         }
       });
-    }
+    };
+    // (p.fast_epilogue: the host has checked that every matrix the epilogue touches lies within 32-bit byte offsets)
+    if (p.fast_epilogue && m0 + BM <= p.M && n0 + BN <= p.N) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
     if (!has_next) break;
     vb = vb_next;
     m0 = m0_next;
@@ -690,6 +802,10 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   CsGemmArgs p = a;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
+  // The epilogue's fast form addresses C, the residual and their byte planes with 32-bit byte offsets from the
+  // matrix bases, and takes output row m for accumulator row m.
+  const int64_t lim = (int64_t)UINT32_MAX - 64;
+  p.fast_epilogue = !p.c_rows && (int64_t)p.M * p.ldc * 2 < lim && (!p.residual || (int64_t)p.M * p.ldr * 2 < lim);
   constexpr int lds = RingShape<BM, BN, W_FP8>::BYTES;
   static bool attr_set = false;
   auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE, SPLIT_RES>;

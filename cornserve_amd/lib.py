@@ -48,6 +48,7 @@ class CsGemmArgs(ctypes.Structure):
         ("w_fp8", c_int32),
         ("tiles_m", c_int32),
         ("tiles_n", c_int32),
+        ("fast_epilogue", c_int32),
         ("a_row_sumsq", c_void_p),
         ("c_row_sumsq", c_void_p),
         ("norm_eps", ctypes.c_float),

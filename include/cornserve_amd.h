@@ -78,6 +78,7 @@ typedef struct CsGemmArgs {
   int32_t epilogue;      /* enum CsEpilogue                                                      */
   int32_t w_fp8;
   int32_t tiles_m, tiles_n; /* filled in by the library                                          */
+  int32_t fast_epilogue;    /* filled in by the library                                          */
   /* RMSNorm folded into the neighbouring GEMMs (qwen2_5_vl.py:173-177: norm1 -> qkv, norm2 -> gate|up).
    * rsqrt(mean(x^2) + eps) is a per-row scalar, so  bf16(x*rstd) * w_norm . W^T  ==  rstd * (x . (W*w_norm)^T)
    * up to the rounding of the normalised activations: the caller folds w_norm into W's columns, passes the

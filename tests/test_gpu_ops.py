@@ -233,17 +233,18 @@ def test_gemm_epilogues(ops, dev):
     M, N, K = 515, 1280, 1280
     a, w, b = rnd((M, K), 1.0, 1, dev), rnd((N, K), 0.05, 2, dev), rnd((N,), 0.02, 3, dev)
     res = rnd((M, N), 1.0, 4, dev)
-    base = lin_ref(a, w, b).bfloat16().float()
+    exact = lin_ref(a, w, b)
+    base = exact.bfloat16().float()
     close(ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res), base + res.float().cpu(), 2**-7, "residual")
-    close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_ERF), F.gelu(base), 2**-7, "gelu erf")
-    close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_TANH), F.gelu(base, approximate="tanh"), 2**-7, "gelu tanh")
-    close(ops.gemm(a, w, b, epilogue=ops.EPI_QUICK_GELU), base * torch.sigmoid(1.702 * base), 2**-7, "quick gelu")
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_ERF), F.gelu(exact), 2**-7, "gelu erf")
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_GELU_TANH), F.gelu(exact, approximate="tanh"), 2**-7, "gelu tanh")
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_QUICK_GELU), exact * torch.sigmoid(1.702 * exact), 2**-7, "quick gelu")
     # the general kernel's copy of the same epilogue (K = 72 is not a shape the fast kernel takes)
     a72, w72 = a[:, :72].contiguous(), w[:, :72].contiguous()
-    base72 = lin_ref(a72, w72, b).bfloat16().float()
+    base72 = lin_ref(a72, w72, b)
     close(ops.gemm(a72, w72, b, epilogue=ops.EPI_QUICK_GELU), base72 * torch.sigmoid(1.702 * base72), 2**-7, "quick gelu, general kernel")
-    gate, up = base[:, 0::2], base[:, 1::2]
-    close(ops.gemm(a, w, b, epilogue=ops.EPI_SWIGLU), F.silu(gate).bfloat16().float() * up, 2**-7, "swiglu")
+    gate, up = exact[:, 0::2], exact[:, 1::2]
+    close(ops.gemm(a, w, b, epilogue=ops.EPI_SWIGLU), F.silu(gate) * up, 2**-7, "swiglu")
     # in-place residual (out aliases residual), as the model uses it
     x = res.clone()
     ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=x, out=x)
@@ -319,11 +320,12 @@ def test_kernels_are_registered_torch_operators(ops, dev):
 
 
 def _epilogue_ref(ops, epi, base, res):
-    """fp32 reference of one fused epilogue on `base` = bf16-rounded A.W^T + bias."""
+    """fp32 reference of one fused epilogue on `base` = A.W^T + bias in fp32.  The residual epilogue rounds the linear
+    layer's output before the addition (the reference's two bf16 operations); an activation takes the fp32 sum."""
     if epi == ops.EPI_BIAS:
         return base
     if epi == ops.EPI_RESIDUAL:
-        return base + res.float().cpu()
+        return base.bfloat16().float() + res.float().cpu()
     if epi == ops.EPI_GELU_ERF:
         return F.gelu(base)
     if epi == ops.EPI_GELU_TANH:
@@ -331,7 +333,7 @@ def _epilogue_ref(ops, epi, base, res):
     if epi == ops.EPI_QUICK_GELU:
         return base * torch.sigmoid(1.702 * base)
     gate, up = base[:, 0::2], base[:, 1::2]
-    return F.silu(gate).bfloat16().float() * up
+    return F.silu(gate) * up
 
 
 # Shapes that reach every tile form and every schedule of the fast kernel: the 256x256 five-unit ring, the
@@ -349,7 +351,7 @@ def test_gemm_fast_path_forms(ops, dev, M, N, K):
     res = rnd((M, N), 1.0, 14, dev)
     rows = torch.arange(0, M, max(1, M // 257))  # a sample of rows: the fp32 reference runs on the host
     rows = torch.cat([rows, torch.tensor([M - 1])])
-    base = lin_ref(a[rows], w, b).bfloat16().float()
+    base = lin_ref(a[rows], w, b)
     for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU, ops.EPI_SWIGLU):
         got = ops.gemm(a, w, b, epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
         close(got[rows], _epilogue_ref(ops, epi, base, res[rows]), 2**-7, f"{M}x{N}x{K} epilogue {epi}")
@@ -379,7 +381,7 @@ def test_gemm_fast_path_forms_fp8_weights(ops, dev, M, N, K):
     q = (w / scale[:, None]).to(torch.float8_e4m3fn)
     wd = q.float() * scale[:, None]          # de-quantised fp32 weights: the comparator of the fp8 path
     rows = torch.cat([torch.arange(0, M, max(1, M // 257)), torch.tensor([M - 1])])
-    base = (a[rows].float().cpu() @ wd.t() + b.float().cpu()).bfloat16().float()
+    base = a[rows].float().cpu() @ wd.t() + b.float().cpu()
     qd, sd = q.to(dev), scale.to(dev)
     for epi in (ops.EPI_BIAS, ops.EPI_RESIDUAL, ops.EPI_GELU_ERF, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU, ops.EPI_SWIGLU):
         got = ops.gemm(a, qd, b, w_scale=sd, epilogue=epi, residual=res if epi == ops.EPI_RESIDUAL else None)
@@ -444,10 +446,10 @@ def test_gemm_with_folded_rmsnorm(ops, dev, M, N, K):
     af = a[rows].float().cpu()
     rstd = torch.rsqrt((af * af).mean(-1, keepdim=True) + eps)
     # closed form of the fused op in fp32 ...
-    base = ((af @ wf.float().cpu().t()) * rstd + b.float().cpu()).bfloat16().float()
+    base = (af @ wf.float().cpu().t()) * rstd + b.float().cpu()
     # ... and the unfused reference sequence (norm.py:35-70 then F.linear): cast, multiply by the weight, cast
     n_ref = ((af * rstd).bfloat16().float() * g.float()).bfloat16()
-    base_unfused = lin_ref(n_ref, w, b).bfloat16().float()
+    base_unfused = lin_ref(n_ref, w, b)
     for epi in (ops.EPI_BIAS, ops.EPI_SWIGLU):
         if epi == ops.EPI_SWIGLU and (N // 2) % 8:   # output rows the fast kernel's 16-byte stores cannot take
             with pytest.raises(RuntimeError):
@@ -482,7 +484,7 @@ def test_gemm_with_folded_layernorm(ops, dev, M, N, K):
     rows = torch.cat([torch.arange(0, M, max(1, M // 257)), torch.tensor([M - 1])])
     af = a[rows].float().cpu()
     n_ref = F.layer_norm(af, (K,), g.float(), beta.float(), eps).bfloat16()     # the unfused reference sequence
-    base = lin_ref(n_ref, w, b).bfloat16().float()
+    base = lin_ref(n_ref, w, b)
     for epi in (ops.EPI_BIAS, ops.EPI_GELU_TANH, ops.EPI_QUICK_GELU):
         got = ops.gemm(a, wf.to(dev), bf.to(dev), epilogue=epi, a_row_sumsq=ss, a_row_sum=sm, w_col_sum=csum.to(dev), norm_eps=eps)
         close(got[rows], _epilogue_ref(ops, epi, base, None), 2**-6, f"folded LayerNorm {M}x{N}x{K} epilogue {epi}")
