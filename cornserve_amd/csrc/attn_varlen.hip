@@ -620,8 +620,9 @@ __global__ __launch_bounds__(256, 2) void attn_full_kernel(const AttnArgs a) {
 }
 
 // Full attention without rotary (SigLIP): K and V tiles go global -> LDS directly (buffer_load ... lds: no
-// staging registers, no LDS store instructions, no address arithmetic per tile) into a ring of three tile
-// buffers, requested two tiles ahead.  A direct load fixes the LDS side -- the 64 lanes of a wave fill 1 KB of
+// staging registers, no LDS store instructions, no address arithmetic per tile) into a ring of NB tile buffers:
+// three buffers requested two tiles ahead with two workgroups per CU, or two buffers requested one tile ahead with
+// three workgroups per CU (what launch_attn selects).  A direct load fixes the LDS side -- the 64 lanes of a wave fill 1 KB of
 // consecutive LDS -- so the padded row layout is produced on the global side: a tile is the flat sequence of
 // 16-byte chunk slots (row, slot), lane l of load j owns slot j*64 + l and fetches chunk `slot % slots_per_row`
 // of row `slot / slots_per_row`; lanes that own padding slots are switched off for the load, which leaves the
@@ -655,7 +656,7 @@ CS_DEVICE void pv_block(f32x16_t& o, i32x2_t (&raw)[8], const bf16x8_t (&pf)[2][
   }
 }
 
-template <int D>
+template <int D, int NB = 3>
 struct AttnDirectShape {
   static constexpr int KS = (D + 15) / 16, DKC = KS * 2, DC = D / 8;
   static constexpr int K_SLOTS = DKC | 1, V_SLOTS = V_RS / 16;      // 16-byte slots per tile row
@@ -663,18 +664,19 @@ struct AttnDirectShape {
   static constexpr int K_BYTES = BKV * RS, V_BYTES = BKV * V_RS, TILE_BYTES = K_BYTES + V_BYTES;
   static constexpr int K_LOADS = BKV * K_SLOTS / 64, V_LOADS = BKV * V_SLOTS / 64;   // BKV == 64: one load per slot column
   static constexpr int LOADS = K_LOADS + V_LOADS, PER_WAVE = (LOADS + 3) / 4;
-  static constexpr int NBUF = 3, LDS = NBUF * TILE_BYTES;
-  static_assert(128 * RS <= 2 * TILE_BYTES, "the Q tile aliases buffers 1 and 2");
-  static_assert(2 * LDS <= 160 * 1024, "two workgroups per CU");
+  static constexpr int NBUF = NB, LDS = NBUF * TILE_BYTES;
+  static constexpr int WGS_PER_CU = NB == 2 ? 3 : 2;
+  static_assert(128 * RS <= (NBUF - 1) * TILE_BYTES, "the Q tile aliases the buffers behind the first");
+  static_assert(WGS_PER_CU * LDS <= 160 * 1024, "workgroups per CU");
 };
 
 // ROPE_Q: the keys were rotated in place beforehand; the query rows are rotated here while they are staged (a
 // query block is staged once, whereas every query block of a segment would rotate the segment's keys again).
-template <int D, bool ROPE_Q = false>
-__global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs a) {
+template <int D, bool ROPE_Q = false, int NB = 3>
+__global__ __launch_bounds__(256, (NB == 2 ? 3 : 2)) void attn_full_direct_kernel(const AttnArgs a) {
   constexpr int NT = 256, BQ = 128;
   static_assert(!ROPE_Q || D % 16 == 0, "rotary needs an even number of 16-byte chunks per half");
-  using Shape = AttnDirectShape<D>;
+  using Shape = AttnDirectShape<D, NB>;
   constexpr int KS = Shape::KS, DT = (D + 31) / 32, DC = Shape::DC, DKC = Shape::DKC;
   constexpr int RS = Shape::RS, K_SLOTS = Shape::K_SLOTS, V_SLOTS = Shape::V_SLOTS;
   constexpr int K_BYTES = Shape::K_BYTES, TILE_BYTES = Shape::TILE_BYTES;
@@ -809,8 +811,10 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
   for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const bf16x8_t*)(q_lds + (wave * 32 + fr) * RS + (2 * ks + hf) * 16);
   __syncthreads();
   init_padding(1);
-  init_padding(2);
-  if (n_tiles > 1) issue_tile(1, 1);
+  if constexpr (NB == 3) {
+    init_padding(2);
+    if (n_tiles > 1) issue_tile(1, 1);
+  }
 
   f32x16_t oacc[DT];
 #pragma unroll
@@ -825,10 +829,16 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
   for (int t = 0; t < n_tiles; ++t) {
     // Tile t has landed when only the loads requested after it (tile t+1's) are in flight; the barrier then also
     // says that every wave is done with tile t-1, whose buffer the request for tile t+2 reuses.
-    if (t + 1 < n_tiles) wait_loads(std::integral_constant<int, PER>{});
-    else wait_loads(std::integral_constant<int, 0>{});
-    barrier();
-    if (t + 2 < n_tiles) issue_tile(t + 2, buf2);
+    if constexpr (NB == 3) {
+      if (t + 1 < n_tiles) wait_loads(std::integral_constant<int, PER>{});
+      else wait_loads(std::integral_constant<int, 0>{});
+      barrier();
+      if (t + 2 < n_tiles) issue_tile(t + 2, buf2);
+    } else {   // two buffers: tile t+1 travels while tile t is worked on (three workgroups per CU hide the rest)
+      wait_loads(std::integral_constant<int, 0>{});
+      barrier();
+      if (t + 1 < n_tiles) issue_tile(t + 1, buf ^ 1);
+    }
     const int nvalid = min(BKV, seg_len - t * BKV);
     if (wave_active) {
       const char* kd = k_buf(buf);
@@ -859,8 +869,12 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
         }
       }
     }
-    buf2 = buf;   // tile t+3 will reuse this iteration's buffer
-    buf = buf == 2 ? 0 : buf + 1;
+    if constexpr (NB == 3) {
+      buf2 = buf;   // tile t+3 will reuse this iteration's buffer
+      buf = buf == 2 ? 0 : buf + 1;
+    } else {
+      buf ^= 1;
+    }
   }
 
   const int qi = wave * 32 + fr;
@@ -868,11 +882,11 @@ __global__ __launch_bounds__(256, 2) void attn_full_direct_kernel(const AttnArgs
 }
 
 
-template <int D, bool ROPE_Q = false>
+template <int D, bool ROPE_Q = false, int NB = 3>
 int launch_attn_full_direct(const AttnArgs& a, dim3 grid, hipStream_t stream) {
-  constexpr int lds = AttnDirectShape<D>::LDS;
+  constexpr int lds = AttnDirectShape<D, NB>::LDS;
   static bool attr_set = false;
-  auto kern = attn_full_direct_kernel<D, ROPE_Q>;
+  auto kern = attn_full_direct_kernel<D, ROPE_Q, NB>;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return CS_ERR_LAUNCH;
@@ -892,11 +906,15 @@ int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, 
   a.n_chunks_x = (n_work + a.chunk - 1) / a.chunk;
   const int n_chunks = a.n_chunks_x * heads;
   const dim3 grid_full(((n_chunks + 7) / 8) * 8 * a.chunk);
+  // The direct-to-LDS kernel with two tile buffers and three workgroups per CU where its LDS allows (head dims up to
+  // 80): the softmax keeps the vector unit as busy as the matrix cores, so a third wave per SIMD buys more overlap
+  // than a third buffer of prefetch (measured: 4096 keys at d = 72 513 -> 444 us, 1024 keys at d = 80 87 -> 80 us).
+  constexpr int RING_DEPTH = D <= 80 ? 2 : 3;
   if (keys_rotated) {
     // only the long-segment kernel has this form (short segments rotate q and k while staging, one workgroup each)
     if constexpr (D % 16 == 0) {
       if (block_q != 64 && rope && (int64_t)max_seqlen * a.ld * 2 < (int64_t)1 << 31)
-        return launch_attn_full_direct<D, true>(a, grid_full, stream);
+        return launch_attn_full_direct<D, true, RING_DEPTH>(a, grid_full, stream);
     }
     return CS_ERR_UNSUPPORTED;
   }
@@ -919,7 +937,8 @@ int launch_attn(AttnArgs a, int n_work, int heads, int block_q, int max_seqlen, 
       else return CS_ERR_UNSUPPORTED;
     } else {
       // the direct-to-LDS kernel addresses a segment's K/V rows with 32-bit byte offsets
-      if ((int64_t)max_seqlen * a.ld * 2 < (int64_t)1 << 31) return launch_attn_full_direct<D>(a, grid_full, stream);
+      if ((int64_t)max_seqlen * a.ld * 2 < (int64_t)1 << 31)
+        return launch_attn_full_direct<D, false, RING_DEPTH>(a, grid_full, stream);
       hipLaunchKernelGGL((attn_full_kernel<D, false>), grid_full, dim3(256), 0, stream, a);
     }
   }
