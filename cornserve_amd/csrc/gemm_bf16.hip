@@ -53,7 +53,9 @@ CS_DEVICE void fp8x16_to_bf16(const i32x4_t& in, bf16x8_t& lo, bf16x8_t& hi) {
   }
 }
 
-template <int BM, int BN, int EPI, bool W_FP8>
+// CONV: the activation operand is gathered from NCHW pixels (a convolution with stride = kernel; see CsGemmArgs.conv_patch):
+// row m is a patch, its K elements are the patch's pixels in (c, ky, kx) order, fetched as 4-byte pixel pairs.
+template <int BM, int BN, int EPI, bool W_FP8, bool CONV = false>
 __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   const bf16_t* const pA = (const bf16_t*)p.A;
@@ -91,11 +93,19 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const CsGemmArgs p) {
   const int ld_c = tid & 7;
   const int ld_r = tid >> 3;
   const bf16_t* a_ptr[A_ITERS];
+  const int conv_pw = CONV ? p.conv_w / p.conv_patch : 1;                   // patches per image row
+  const int conv_pi = CONV ? (p.conv_h / p.conv_patch) * conv_pw : 1;       // patches per image
+  const int conv_kreal = CONV ? p.conv_c * p.conv_patch * p.conv_patch : 0;
 #pragma unroll
   for (int i = 0; i < A_ITERS; ++i) {
     int r = min(m0 + ld_r + 64 * i, p.M - 1);
-    if (p.a_rows) r = p.a_rows[r];
-    a_ptr[i] = pA + (int64_t)r * p.lda + ld_c * 8;
+    if constexpr (CONV) {   // first pixel of patch r: image b, patch row py, patch column px, channel 0
+      const int b = r / conv_pi, q = r - b * conv_pi, py = q / conv_pw, px = q - py * conv_pw;
+      a_ptr[i] = pA + ((int64_t)b * p.conv_c * p.conv_h + (int64_t)py * p.conv_patch) * p.conv_w + px * p.conv_patch;
+    } else {
+      if (p.a_rows) r = p.a_rows[r];
+      a_ptr[i] = pA + (int64_t)r * p.lda + ld_c * 8;
+    }
   }
   const char* w_ptr[W_ITERS];
   int w_lr[W_ITERS], w_lc[W_ITERS];
@@ -120,9 +130,36 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const CsGemmArgs p) {
 
   auto load_global = [&](int kt) {
     const int k0 = kt * BK;
+    if constexpr (CONV) {
+      // The thread's 8 consecutive k = four pixel pairs.  k is even and so is the patch size, so a pair never
+      // straddles a patch row; its offset from the patch's first pixel is (c*H + ky)*W + kx.
+      const int kk = k0 + ld_c * 8;
+      int off[4];
+      bool ok[4];
+      int c = kk / (p.conv_patch * p.conv_patch), rem = kk - c * p.conv_patch * p.conv_patch;
+      int ky = rem / p.conv_patch, kx = rem - ky * p.conv_patch;
 #pragma unroll
-    for (int i = 0; i < A_ITERS; ++i) {
-      ga[i] = (k0 + ld_c * 8 < p.K) ? *(const i32x4_t*)(a_ptr[i] + k0) : zero4;
+      for (int j = 0; j < 4; ++j) {
+        off[j] = (c * p.conv_h + ky) * p.conv_w + kx;
+        ok[j] = kk + 2 * j < conv_kreal;
+        kx += 2;
+        if (kx >= p.conv_patch) {
+          kx = 0;
+          if (++ky == p.conv_patch) {
+            ky = 0;
+            ++c;
+          }
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < A_ITERS; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) ga[i][j] = ok[j] ? *(const int*)(a_ptr[i] + off[j]) : 0;
+    } else {
+#pragma unroll
+      for (int i = 0; i < A_ITERS; ++i) {
+        ga[i] = (k0 + ld_c * 8 < p.K) ? *(const i32x4_t*)(a_ptr[i] + k0) : zero4;
+      }
     }
 #pragma unroll
     for (int i = 0; i < W_ITERS; ++i) {
@@ -196,14 +233,14 @@ __global__ __launch_bounds__(NTHREADS) void gemm_kernel(const CsGemmArgs p) {
   csgemm::epilogue<EPI, MT, NT>(p, acc, m0 + wm * WTM, n0 + wn * WTN, lane);
 }
 
-template <int BM, int BN, int EPI, bool W_FP8>
+template <int BM, int BN, int EPI, bool W_FP8, bool CONV = false>
 int launch(const CsGemmArgs& a, hipStream_t stream) {
   CsGemmArgs p = a;
   p.tiles_m = (p.M + BM - 1) / BM;
   p.tiles_n = (p.N + BN - 1) / BN;
   constexpr int lds = 2 * (BM + BN) * BK * 2;
   static bool attr_set = false;
-  auto kern = gemm_kernel<BM, BN, EPI, W_FP8>;
+  auto kern = gemm_kernel<BM, BN, EPI, W_FP8, CONV>;
   if (!attr_set) {
     if (hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return CS_ERR_LAUNCH;
@@ -236,7 +273,7 @@ extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
   if (a.M == 0 && a.W) return CS_OK;  // an empty batch may come with null activation buffers
   if (!a.A || !a.W || !a.C) return CS_ERR_INVALID_ARG;
   // 16-byte vector loads along K and 8-byte packed stores along N.
-  if (a.K % 8 || a.lda % 8 || a.N % 4 || a.ldc % 2) return CS_ERR_INVALID_ARG;
+  if (a.K % 8 || (a.lda % 8 && !a.conv_patch) || a.N % 4 || a.ldc % 2) return CS_ERR_INVALID_ARG;
   if (a.w_fp8 ? (a.ldw % 16 || a.K % 16 || !a.w_scale) : (a.ldw % 8)) return CS_ERR_INVALID_ARG;
   if (a.epilogue == CS_EPI_RESIDUAL && (!a.residual || a.ldr % 4)) return CS_ERR_INVALID_ARG;
   if (a.epilogue != CS_EPI_SWIGLU && a.ldc % 4) return CS_ERR_INVALID_ARG;
@@ -251,6 +288,18 @@ extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
        (uintptr_t)a.w_col_sum) & 15)
     return CS_ERR_INVALID_ARG;
 
+  if (a.conv_patch) {   // strided-gather form of the activation operand: general kernel only
+    if (a.conv_patch < 2 || a.conv_patch % 2 || a.conv_w % 2 || a.conv_c < 1 || a.conv_h < a.conv_patch ||
+        a.conv_w < a.conv_patch || a.epilogue != CS_EPI_BIAS || a.w_fp8 || a.a_rows || a.a_row_sumsq || a.c_row_sumsq ||
+        a.a_row_sum || a.c_row_sum)
+      return CS_ERR_INVALID_ARG;
+    const int64_t per_image = (int64_t)(a.conv_h / a.conv_patch) * (a.conv_w / a.conv_patch);
+    if (a.M % per_image || a.K < a.conv_c * a.conv_patch * a.conv_patch || a.K >= a.conv_c * a.conv_patch * a.conv_patch + 8 ||
+        (int64_t)a.conv_c * a.conv_h * a.conv_w >= ((int64_t)1 << 31))
+      return CS_ERR_INVALID_ARG;
+    const int64_t t256 = (int64_t)((a.M + 255) / 256) * ((a.N + 255) / 256);
+    return t256 < 192 ? launch<128, 128, CS_EPI_BIAS, false, true>(a, stream) : launch<256, 256, CS_EPI_BIAS, false, true>(a, stream);
+  }
   // Fast path (direct-to-LDS pipeline) when the shape allows it; otherwise the general kernel below.
   {
     bool handled = false;

@@ -183,7 +183,7 @@ class SiglipEncoderBase(EricModel):
         vc = self.config.vision_config
         H = vc.hidden_size
         kraw = vc.num_channels * vc.patch_size * vc.patch_size
-        kp = _round_up(kraw, 16)
+        kp = _round_up(kraw, 8)    # K of the strided-gather patch-embedding GEMM: a multiple of 8, zero columns behind kraw
         pe_w = torch.zeros((H, kp), dtype=self.dtype, device=self.device)
         pe_w[:, :kraw] = vm.embeddings.patch_embedding.weight.reshape(H, kraw)
         # The MLP intermediate size (4304 for SigLIP-so400m) is padded to a multiple of 64 so that fc2's K loop is
@@ -248,8 +248,9 @@ class SiglipEncoderBase(EricModel):
             if B > most:
                 return torch.cat([self.vision_tower_forward(pixel_values[i : i + most]) for i in range(0, B, most)])
         M = B * tokens
-        patches = ops.patchify_nchw(pixel_values.contiguous(), vc.patch_size, pk["kp"])
-        x = ops.gemm(patches, pk["pe_w"], pk["pe_b"], pos=pk["pos"])
+        # Conv2d(kernel = stride = patch) + position rows as ONE strided-gather GEMM: the patches are fetched from the
+        # NCHW image inside the kernel (siglip.py:30-36,94-101); no [tokens, C*patch*patch] buffer exists
+        x = ops.gemm(pixel_values.contiguous(), pk["pe_w"], pk["pe_b"], pos=pk["pos"], conv_patch=vc.patch_size)
         plan = ops.attn_plan(np.arange(0, M + 1, tokens, dtype=np.int32), x.device)
         n = torch.empty_like(x)
         qkv = torch.empty((M, 3 * H), dtype=torch.bfloat16, device=x.device)

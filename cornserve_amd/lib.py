@@ -57,6 +57,10 @@ class CsGemmArgs(ctypes.Structure):
         ("w_col_sum", c_void_p),
         ("residual_lo", c_void_p),
         ("c_lo", c_void_p),
+        ("conv_c", c_int32),
+        ("conv_h", c_int32),
+        ("conv_w", c_int32),
+        ("conv_patch", c_int32),
     ]
 
 

@@ -101,8 +101,14 @@ def gemm(
     w_col_sum: torch.Tensor | None = None,
     residual_lo: torch.Tensor | None = None,
     out_lo: torch.Tensor | None = None,
+    conv_patch: int = 0,
 ) -> torch.Tensor:
     """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`.
+
+    `conv_patch` > 0: `a` is NCHW pixels [B,C,H,W] (bf16, contiguous) and the product is the convolution with kernel =
+    stride = conv_patch as a strided-gather GEMM: row m is patch (b, py, px), its K elements are the patch's pixels in
+    (c, ky, kx) order, fetched from the image inside the kernel (no im2col buffer); `w` is the [N, C*patch*patch]
+    kernel matrix, zero-padded along K to a multiple of 8.
 
     `a_row_sumsq` (fp32 [M, SUMSQ_PARTS]) scales row m of the product by rsqrt(sum(parts)/K + norm_eps): an
     RMSNorm of `a` whose weight the caller has folded into the columns of `w`.  `c_row_sumsq` (same layout,
@@ -118,33 +124,59 @@ def gemm(
     Dispatches to `torch.ops.cornserve_amd.gemm_` (or the functional `gemm` when nothing is written in place)."""
     if out is None and c_row_sumsq is None and c_row_sum is None and out_lo is None and residual_lo is None:
         return torch.ops.cornserve_amd.gemm(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k,
-                                            a_row_sumsq, norm_eps, a_row_sum, w_col_sum)
+                                            a_row_sumsq, norm_eps, a_row_sum, w_col_sum, conv_patch)
     if out is None:  # (with c_rows: a permutation of the M rows; anything else needs the caller's `out`)
-        M = a.shape[0] if a_rows is None else a_rows.shape[0]
-        out = torch.empty((M, w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]), dtype=torch.bfloat16, device=a.device)
+        out = torch.empty((_gemm_rows(a, a_rows, conv_patch), w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]),
+                          dtype=torch.bfloat16, device=a.device)
     torch.ops.cornserve_amd.gemm_(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq,
-                                  c_row_sumsq, norm_eps, a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo)
+                                  c_row_sumsq, norm_eps, a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo, conv_patch)
     return out
 
 
-def _gemm_functional(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, norm_eps, a_row_sum,
-                     w_col_sum):
-    if a.dim() != 2 or w.dim() != 2:
+def _gemm_rows(a, a_rows, conv_patch) -> int:
+    """Output rows of a product: A's rows, the gathered rows, or the patches of NCHW pixels."""
+    if conv_patch:
+        if a.dim() != 4 or conv_patch < 1:
+            raise ValueError("with conv_patch, `a` must be NCHW pixels [B,C,H,W]")
+        return a.shape[0] * (a.shape[2] // conv_patch) * (a.shape[3] // conv_patch)
+    if a.dim() != 2:
         raise ValueError("gemm operands must be 2-D")
-    M = a.shape[0] if a_rows is None else a_rows.shape[0]
+    return a.shape[0] if a_rows is None else a_rows.shape[0]
+
+
+def _gemm_functional(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, norm_eps, a_row_sum,
+                     w_col_sum, conv_patch=0):
+    if w.dim() != 2:
+        raise ValueError("gemm operands must be 2-D")
+    M = _gemm_rows(a, a_rows, conv_patch)
     out = torch.empty((M, w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]), dtype=torch.bfloat16, device=a.device)
     _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, None, norm_eps,
-               a_row_sum, None, w_col_sum, None, None)
+               a_row_sum, None, w_col_sum, None, None, conv_patch)
     return out
 
 
 def _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, c_row_sumsq, norm_eps,
-               a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo) -> None:
+               a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo, conv_patch=0) -> None:
     """Implementation of cornserve_amd::gemm_: argument checks, then cs_gemm on the current stream."""
     lib = _l.load()
     _req(a, torch.bfloat16, "a")
-    if a.dim() != 2 or w.dim() != 2:
+    if w.dim() != 2:
         raise ValueError("gemm operands must be 2-D")
+    conv = None
+    if conv_patch:
+        if a.dim() != 4 or not a.is_contiguous() or conv_patch < 2 or conv_patch % 2 or a.shape[3] % 2:
+            raise ValueError("with conv_patch, `a` must be contiguous NCHW pixels with an even width and patch size")
+        if a_rows is not None or k is not None or epilogue != EPI_BIAS:
+            raise ValueError("the strided-gather product takes no a_rows / k and only the bias epilogue")
+        conv = (a.shape[1], a.shape[2], a.shape[3], conv_patch)
+        kreal = a.shape[1] * conv_patch * conv_patch
+        if w.shape[1] != (kreal + 7) // 8 * 8:
+            raise ValueError(f"w must have {(kreal + 7) // 8 * 8} columns (C*patch*patch = {kreal} rounded up to a multiple of 8)")
+        a2d_rows, a2d_cols = _gemm_rows(a, None, conv_patch), w.shape[1]
+    elif a.dim() != 2:
+        raise ValueError("gemm operands must be 2-D")
+    else:
+        a2d_rows, a2d_cols = a.shape
     fp8 = w.dtype in (torch.float8_e4m3fn, torch.uint8)
     if not fp8:
         _req(w, torch.bfloat16, "w")
@@ -155,11 +187,11 @@ def _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows
             _req(t, torch.int32, name)
             if t.dim() != 1 or not t.is_contiguous():
                 raise ValueError(f"{name} must be a contiguous int32 vector")
-    M = a.shape[0] if a_rows is None else a_rows.shape[0]
-    K = a.shape[1] if k is None else k
+    M = a2d_rows if a_rows is None else a_rows.shape[0]
+    K = a2d_cols if k is None else k
     N = w.shape[0]
-    if K > a.shape[1] or K < 1:
-        raise ValueError(f"k={K} exceeds the {a.shape[1]} columns of a")
+    if K > a2d_cols or K < 1:
+        raise ValueError(f"k={K} exceeds the {a2d_cols} columns of a")
     if w.shape[1] < K:
         raise ValueError(f"w has {w.shape[1]} columns, need at least K={K}")
     if c_rows is not None and c_rows.shape[0] < M:
@@ -202,7 +234,9 @@ def _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows
     if len(on) != 1:
         raise ValueError(f"gemm operands live on different devices: {sorted(map(str, on))}")
     args = _l.CsGemmArgs()
-    args.A, args.lda = a.data_ptr(), a.stride(0)
+    args.A, args.lda = a.data_ptr(), (0 if conv else a.stride(0))
+    if conv:
+        args.conv_c, args.conv_h, args.conv_w, args.conv_patch = conv
     args.W, args.ldw = w.data_ptr(), w.stride(0)
     args.w_scale = _ptr(w_scale)
     args.bias = _ptr(bias)
@@ -717,11 +751,11 @@ _LIBRARY = torch.library.Library("cornserve_amd", "DEF")
 _OPERATORS: dict[str, tuple[str, object]] = {
     "gemm": ("(Tensor a, Tensor w, Tensor? bias, int epilogue, Tensor? residual, Tensor? w_scale, Tensor? pos, "
              "Tensor? a_rows, Tensor? c_rows, int? k, Tensor? a_row_sumsq, float norm_eps, Tensor? a_row_sum, "
-             "Tensor? w_col_sum) -> Tensor", _gemm_functional),
+             "Tensor? w_col_sum, int conv_patch=0) -> Tensor", _gemm_functional),
     "gemm_": ("(Tensor(a!) out, Tensor a, Tensor w, Tensor? bias, int epilogue, Tensor? residual, Tensor? w_scale, "
               "Tensor? pos, Tensor? a_rows, Tensor? c_rows, int? k, Tensor? a_row_sumsq, Tensor(b!)? c_row_sumsq, "
               "float norm_eps, Tensor? a_row_sum, Tensor(c!)? c_row_sum, Tensor? w_col_sum, Tensor? residual_lo, "
-              "Tensor(d!)? out_lo) -> ()", _gemm_impl),
+              "Tensor(d!)? out_lo, int conv_patch=0) -> ()", _gemm_impl),
     "row_stats_": ("(Tensor(a!) sumsq_out, Tensor(b!)? sum_out, Tensor x) -> ()", _row_stats_impl),
     "rmsnorm_": ("(Tensor(a!) out, Tensor x, Tensor w, float eps, bool gemma) -> ()", _rmsnorm_impl),
     "layernorm_": ("(Tensor(a!) out, Tensor x, Tensor w, Tensor b, float eps) -> ()", _layernorm_impl),
@@ -744,8 +778,9 @@ _OPERATORS: dict[str, tuple[str, object]] = {
 }
 
 
-def _fake_gemm(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, norm_eps, a_row_sum, w_col_sum):
-    M = a.shape[0] if a_rows is None else a_rows.shape[0]
+def _fake_gemm(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, norm_eps, a_row_sum, w_col_sum,
+               conv_patch=0):
+    M = _gemm_rows(a, a_rows, conv_patch)
     return a.new_empty((M, w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]), dtype=torch.bfloat16)
 
 

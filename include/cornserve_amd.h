@@ -115,6 +115,14 @@ typedef struct CsGemmArgs {
    *              pair, so the stream can start from any bf16 tensor.  May alias residual_lo when C aliases residual. */
   const uint8_t* residual_lo;
   uint8_t* c_lo;
+  /* Convolution with stride = kernel as a strided-gather GEMM (Conv2d patch embedding, siglip.py:30-36,94-95).  With
+   * conv_patch > 0, A is not a matrix but NCHW pixels, bf16 [B, conv_c, conv_h, conv_w] (lda is ignored): output row m
+   * is patch (b, py, px) in row-major patch order, M = B * (conv_h / patch) * (conv_w / patch), and element k =
+   * (c, ky, kx) of its row is pixel [b, c, py*patch + ky, px*patch + kx]; k >= conv_c * patch^2 reads as zero, so K may
+   * be that product rounded up to the multiple of 8 the kernel needs (W then carries zero columns).  patch and conv_w
+   * must be even (pixel pairs are fetched as 4-byte words); pixels past the last whole patch are not read, as the
+   * convolution drops them.  CS_EPI_BIAS (with or without the position addend), bf16 W, no a_rows.                  */
+  int32_t conv_c, conv_h, conv_w, conv_patch;
 } CsGemmArgs;
 #define CS_SUMSQ_PARTS 8
 

@@ -892,6 +892,42 @@ def test_rows_bilinear_bit_exact(ops, dev):
                           torch.zeros((4, 2), dtype=torch.float32, device=dev))
 
 
+@pytest.mark.parametrize("B,C,H,W,patch,N", [(2, 3, 896, 896, 14, 1152), (3, 3, 384, 384, 14, 1152), (5, 3, 56, 84, 14, 64),
+                                               (2, 1, 48, 32, 16, 40), (1, 3, 30, 44, 6, 24)])
+def test_gemm_strided_gather_convolution(ops, dev, B, C, H, W, patch, N):
+    """Conv2d with kernel = stride = patch (siglip.py:30-36) as a GEMM whose activation operand is gathered from the
+    NCHW image inside the kernel: against torch's convolution, and bit for bit against the same GEMM on patches
+    materialised by cs_patchify_nchw (same K order, same kernel, so the same accumulation order).  384 / 14 and
+    30 / 6 leave pixels past the last whole patch, which neither form reads."""
+    g = torch.Generator().manual_seed(61)
+    px = (torch.rand((B, C, H, W), generator=g) * 2 - 1).bfloat16()
+    wt = (torch.randn((N, C, patch, patch), generator=g) * 0.05).bfloat16()
+    bias = (torch.randn((N,), generator=g) * 0.02).bfloat16()
+    kraw = C * patch * patch
+    kp = (kraw + 7) // 8 * 8
+    w2 = torch.zeros((N, kp), dtype=torch.bfloat16)
+    w2[:, :kraw] = wt.reshape(N, kraw)
+    hp, wp = H // patch, W // patch
+    pos = (torch.randn((hp * wp, N), generator=g) * 0.1).bfloat16()
+    dpx, dw, db, dpos = px.to(dev), w2.to(dev), bias.to(dev), pos.to(dev)
+    got = ops.gemm(dpx, dw, db, conv_patch=patch)
+    assert got.shape == (B * hp * wp, N)
+    ref = F.conv2d(px.float(), wt.float(), bias.float(), stride=patch).flatten(2).transpose(1, 2).reshape(-1, N)
+    close(got, ref, 2**-7, "strided-gather GEMM vs conv2d")
+    mat = ops.gemm(ops.patchify_nchw(dpx, patch, kp), dw, db)
+    assert torch.equal(got, mat)
+    with_pos = ops.gemm(dpx, dw, db, pos=dpos, conv_patch=patch)
+    assert torch.equal(with_pos, ops.gemm(ops.patchify_nchw(dpx, patch, kp), dw, db, pos=dpos))
+    out = torch.empty_like(got)
+    assert torch.equal(ops.gemm(dpx, dw, db, conv_patch=patch, out=out), got)
+    for bad in (dict(conv_patch=patch + 1), dict(conv_patch=patch, epilogue=ops.EPI_GELU_TANH),
+                dict(conv_patch=patch, a_rows=torch.zeros(4, dtype=torch.int32, device=dev))):
+        with pytest.raises(ValueError):
+            ops.gemm(dpx, dw, db, **bad)
+    with pytest.raises(ValueError):
+        ops.gemm(dpx, dw[:, : kp - 8].contiguous(), db, conv_patch=patch)
+
+
 def test_patchify_nchw_drops_the_partial_patches(ops, dev):
     """384 = 27 * 14 + 6: a convolution with stride = kernel and no padding ignores the last 6 rows and columns."""
     px = rnd((3, 3, 384, 384), 1.0, 72)
