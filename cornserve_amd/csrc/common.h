@@ -13,6 +13,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
 typedef __attribute__((__vector_size__(4 * sizeof(int)))) int i32x4_t;
 typedef __attribute__((__vector_size__(2 * sizeof(int)))) int i32x2_t;
 typedef __attribute__((__vector_size__(2 * sizeof(uint32_t)))) uint32_t u32x2_t;

@@ -59,6 +59,9 @@ namespace {
 using namespace csgemm;
 
 constexpr int CS_EPI_BIAS_POS = 100;  // internal: CS_EPI_BIAS plus the (row % pos_period) position addend
+// internal: the QKV projection of one head per column tile with rotary and window attention as its epilogue (see
+// cs_qkv_window_attn): the tile's 256 columns are the head's q (5 fragments), k (5), v (5) and one all-zero fragment
+constexpr int CS_EPI_QKV_WATTN = 101;
 constexpr int NW = 4;                 // waves per workgroup, one per SIMD
 constexpr int LDS_BYTES = 160 * 1024;
 
@@ -209,9 +212,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   uint32_t a_src[A_LD];
   uint32_t w_src[W_LD];
   auto setup_sources = [&](int m0, int n0) {
-    // (an opaque copy of the lane number: the swizzled chunk offsets are recomputed at every call instead of being
-    // kept in registers across the main loop)
-    int lane_s = lane;
+    // (the lane number afresh from the hardware, behind an opaque copy: the swizzled chunk offsets are recomputed at
+    // every call instead of being kept in registers across the main loop)
+    int lane_s = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
     asm volatile("" : "+v"(lane_s));
     const int l_row = lane_s >> 3, l_slot = lane_s & 7;
 #pragma unroll
@@ -270,19 +273,23 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   // ---- fragment addressing.  Lane (a = lane%16, kq = lane/16) reads chunk ks*4 + kq of its fragment row.
   //      Both keys depend only on the lane, so the per-lane part of the address is loop-invariant.
   const int fa = lane & 15, kq = lane >> 4;
-  const int fq = fa >> 2, fr = fa & 3;
-  const int x_key = (fa >> 1) & 7;
-  const int w_key = (fq << 1) | ((fr >> 1) & 1);
   // byte offset inside an operand tile of fragment (i or j), k-step ks: row*128 + (((ks*4 + kq) ^ key) << 4)
   int x_off[2], w_off[2];
+  auto setup_frag_offsets = [&](int ln) {
+    const int fa = ln & 15, kq = ln >> 4;
+    const int fq = fa >> 2, fr = fa & 3;
+    const int x_key = (fa >> 1) & 7;
+    const int w_key = (fq << 1) | ((fr >> 1) & 1);
 #pragma unroll
-  for (int ks = 0; ks < 2; ++ks) {
-    x_off[ks] = (wm * WTM + fa) * 128 + (((ks * 4 + kq) ^ x_key) << 4);
-    if constexpr (W_FP8)  // 8 bytes: half (kq%2) of chunk 2ks + kq/2, which sits in slot chunk ^ q
-      w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 2 + (kq >> 1)) ^ fq) << 4) + (kq & 1) * 8;
-    else
-      w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 4 + kq) ^ w_key) << 4);
-  }
+    for (int ks = 0; ks < 2; ++ks) {
+      x_off[ks] = (wm * WTM + fa) * 128 + (((ks * 4 + kq) ^ x_key) << 4);
+      if constexpr (W_FP8)  // 8 bytes: half (kq%2) of chunk 2ks + kq/2, which sits in slot chunk ^ q
+        w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 2 + (kq >> 1)) ^ fq) << 4) + (kq & 1) * 8;
+      else
+        w_off[ks] = (wn * WTN + fq * (4 * G) + fr) * W_ROW + (((ks * 4 + kq) ^ w_key) << 4);
+    }
+  };
+  setup_frag_offsets(lane);
   // Operand fragments: two sets.  fp8 weights are read as 8 raw bytes per fragment and converted into one of
   // two bf16 registers sets right before use.
   bf16x8_t wf[2][W_FP8 ? 1 : NT], xf[2][MT];
@@ -330,7 +337,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       // compiler pads that for its own MFMAs but cannot see into these.  Only the first MFMA after a
       // conversion can be that close.
       if constexpr (W_FP8 && I == 0) asm volatile("s_nop 3");
-      if constexpr (ZERO)
+      if constexpr (EPI == CS_EPI_QKV_WATTN && J >= 10) {
+        // The V fragments are computed TRANSPOSED (activation rows as the first operand): a lane then owns one
+        // head dim and four consecutive keys, the operand layout of the P.V product.  Fragment 15 is padding.
+        if constexpr (J < 15) {
+          if constexpr (ZERO)
+            asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %1, %0, 0" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
+          else
+            asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %1, %0, a[%2:%3]" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
+        }
+      } else if constexpr (ZERO)
         asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
       else
         asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(w), "v"(xf[B][I]), "n"(R), "n"(R + 3));
@@ -462,6 +478,225 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     // epilogue reads the accumulation registers
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 
+    // ---- QKV projection + rotary + window attention for one head and four windows (one window of 64 rows per
+    //      wave), entirely in registers.  Accumulator fragment (I, J) of a wave: rows 16I .. 16I+15 of its window;
+    //      J = 0..4 q, 5..9 k, 10..14 v (transposed), 15 padding.  For q and k a lane (row lr = lane%16, kq = lane/16)
+    //      holds four values per fragment, 20 per tensor: "slot" s = 4(J mod 5) + r stands for head dim 10kq + s
+    //      (s < 10) or 40 + 10kq + (s - 10): the caller packs the weight rows in that order, so that both halves of
+    //      every rotary pair sit in one lane, and so that eight slots of a lane are exactly one MFMA operand: S^T =
+    //      K.Q^T is two 16x16x32 steps and one 16x16x16 step per 16x16 block, straight from the rotated registers.
+    //      S^T's accumulators hold four consecutive keys per lane, the layout of the second product's operand, and
+    //      the transposed V fragments hold four consecutive keys per head dim: O^T = V^T.P^T needs no transposition.
+    auto wattn_epilogue = [&](auto) {   // (generic: only instantiated for the kernel that calls it)
+      static_assert(EPI != CS_EPI_QKV_WATTN || (BM == 256 && BN == 256 && WAVES_M == 4 && WAVES_N == 1 && !W_FP8),
+                    "one 64-row window per wave, one head per column tile");
+      constexpr int HD = 80, HALF = 40;
+      constexpr bool NORM_A = FUSE == FUSE_NORM_A;
+      auto s_reg = [](int b) constexpr { return b < 10 ? 4 * b : 64 + 4 * (b - 10); };   // first register of S^T block b
+      int lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));   // the lane number, afresh
+      asm volatile("" : "+v"(lane_e));
+      const int lr = lane_e & 15, kq = lane_e >> 4;
+      // lane exchanges through bpermute with addresses derived from the opaque lane number: the library shuffles
+      // derive them from a lane id that the compiler computes once per kernel and would keep in a register -- an
+      // accumulation register -- across the main loop
+      const int x16 = (lane_e ^ 16) << 2, x32 = (lane_e ^ 32) << 2;
+      auto lane_xchg = [](float v, int byte_addr) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(byte_addr, __builtin_bit_cast(int, v)));
+      };
+      const int row0 = m0 + wm * 64;                 // first row of this wave's window
+      if (row0 >= p.M) return;                       // (no barrier below: waves may leave independently)
+      const int head = n0 / BN;
+      const bf16_t* const pBias = (const bf16_t*)p.bias + n0;
+      const float sl2 = p.attn_scale_log2e;
+      // per-row scale of the folded RMSNorm: rows row0 + 16I + lr
+      float rstd[4];
+#pragma unroll
+      for (int I = 0; I < 4; ++I) {
+        rstd[I] = 1.0f;
+        if constexpr (NORM_A) {
+          const float* parts = p.a_row_sumsq + (int64_t)(row0 + 16 * I + lr) * CS_SUMSQ_PARTS;
+          const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
+          const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
+          rstd[I] = rsqrtf(ss / (float)p.K + p.norm_eps);
+        }
+      }
+      // bias of the lane's q / k slots (packed like the weight rows: fragment J, lane kq -> 4 consecutive entries)
+      bf16x4_t bias_qk[10];
+#pragma unroll
+      for (int J = 0; J < 10; ++J) bias_qk[J] = *(const bf16x4_t*)(pBias + (J / 2) * 32 + kq * 8 + (J % 2) * 4);
+      bf16x8_t qf8[4][2], kf8[4][2];
+      bf16x4_t qf4[4], kf4[4];
+      // q and k: scale, bias, rotary (fp32, one rounding), packed as operands
+      static_for<4>([&](auto i_c) {
+        constexpr int I = decltype(i_c)::value;
+        const float* cs = p.attn_cos_sin + (int64_t)(row0 + 16 * I + lr) * HD + 10 * kq;
+        float co[10], si[10];
+#pragma unroll
+        for (int t = 0; t < 10; t += 2) {   // 8-byte aligned: 40 kq bytes into a 320-byte row
+          const f32x2_t c2 = *(const f32x2_t*)(cs + t), s2 = *(const f32x2_t*)(cs + HALF + t);
+          co[t] = c2[0];
+          co[t + 1] = c2[1];
+          si[t] = s2[0];
+          si[t + 1] = s2[1];
+        }
+        static_for<2>([&](auto which_c) {
+          constexpr int WHICH = decltype(which_c)::value;   // 0: q (fragments 0..4), 1: k (fragments 5..9)
+          float x[20];
+          static_for<20>([&](auto s_c) {
+            constexpr int S = decltype(s_c)::value, J = WHICH * 5 + S / 4, R = (I * NT + J) * 4 + S % 4;
+            float t;
+            asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R));
+            x[S] = t * rstd[I] + bf2f(bias_qk[J][S % 4]);
+          });
+          float o[20];
+#pragma unroll
+          for (int t = 0; t < 10; ++t) {
+            o[t] = rot_first(x[t], x[t + 10], co[t], si[t]);
+            o[t + 10] = rot_second(x[t], x[t + 10], co[t], si[t]);
+          }
+          bf16x8_t f0, f1;
+          bf16x4_t f2;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            f0[e] = f2bf(o[e]);
+            f1[e] = f2bf(o[8 + e]);
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) f2[e] = f2bf(o[16 + e]);
+          bf16x8_t(&dst8)[4][2] = WHICH == 0 ? qf8 : kf8;
+          bf16x4_t(&dst4)[4] = WHICH == 0 ? qf4 : kf4;
+          dst8[I][0] = f0;
+          dst8[I][1] = f1;
+          dst4[I] = f2;
+        });
+      });
+      // ---- S^T[key][query] = K.Q^T, block b = 4kb + qb in registers that the q and k accumulators have left free
+      //      (the transposed V accumulators are still where the main loop put them: fragments 10..14 of every row
+      //      block): a[4b ..] for b < 10, a[64 + 4(b - 10) ..] above.  Steps outermost, so that consecutive MFMAs
+      //      never depend on each other.
+      asm volatile("s_nop 7" ::: "memory");   // the operands above were written by vector instructions
+      static_for<16>([&](auto b_c) {
+        constexpr int KB = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = s_reg(KB * 4 + QB);
+        const bf16x8_t ka = kf8[KB][0], qb = qf8[QB][0];   // (named copies: asm operands alone do not capture)
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
+      });
+      static_for<16>([&](auto b_c) {
+        constexpr int KB = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = s_reg(KB * 4 + QB);
+        const bf16x8_t ka = kf8[KB][1], qb = qf8[QB][1];
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
+      });
+      static_for<16>([&](auto b_c) {
+        constexpr int KB = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = s_reg(KB * 4 + QB);
+        const bf16x4_t ka = kf4[KB], qb = qf4[QB];
+        asm volatile("v_mfma_f32_16x16x16_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
+      });
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      // ---- softmax over the 64 keys of a query row (16 per lane, 4 lanes per row); P packed as the operand of the
+      //      second product: key step t = blocks 2t, 2t+1
+      bf16x8_t pf8[4][2];
+      float inv_l[4];
+      static_for<4>([&](auto q_c) {
+        constexpr int QB = decltype(q_c)::value;
+        float sv[16];
+        static_for<16>([&](auto e_c) {
+          constexpr int E = decltype(e_c)::value, KB = E / 4, R = s_reg(KB * 4 + QB) + E % 4;
+          float t;
+          asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R));
+          sv[E] = t;
+        });
+        float mx = sv[0];
+#pragma unroll
+        for (int e = 1; e < 16; ++e) mx = fmaxf(mx, sv[e]);
+        mx = fmaxf(mx, lane_xchg(mx, x16));
+        mx = fmaxf(mx, lane_xchg(mx, x32));
+        const float mb = mx * sl2;
+        float sum = 0.f;
+        bf16x8_t f[2];
+#pragma unroll
+        for (int e = 0; e < 16; ++e) {
+          const float pv = __builtin_amdgcn_exp2f(sv[e] * sl2 - mb);
+          const bf16_t pb = f2bf(pv);
+          sum += bf2f(pb);   // the denominator of exactly the weights the second product uses
+          f[e >> 3][e & 7] = pb;
+        }
+        sum += lane_xchg(sum, x16);
+        sum += lane_xchg(sum, x32);
+        inv_l[QB] = 1.0f / sum;
+        pf8[QB][0] = f[0];
+        pf8[QB][1] = f[1];
+      });
+      // v (transposed fragments): lane (head dim 16d + lr, kq) holds keys 16I + 4kq + r; operand of key step t = keys
+      // of row blocks 2t and 2t+1
+      bf16x8_t vf8[5][2];
+      {
+        // (addresses re-derived behind an opaque copy of the lane number, so that these loads are not hoisted to the
+        // top of the epilogue, where the registers are needed for the q and k operands)
+        int lane_v = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+        asm volatile("" : "+v"(lane_v));
+        const int lrv = lane_v & 15;
+        float bias_v[5];   // fragment row lr of the transposed V fragments
+#pragma unroll
+        for (int d = 0; d < 5; ++d) bias_v[d] = bf2f(pBias[((10 + d) / 2) * 32 + (lrv >> 2) * 8 + ((10 + d) % 2) * 4 + (lrv & 3)]);
+        // the folded norm's scale of rows 16I + 4kq + r: recomputed for rows 16I + lr (not kept in registers since the
+        // q / k phase) and fetched from the lanes that hold them
+        float rv[4][4];
+#pragma unroll
+        for (int I = 0; I < 4; ++I) {
+          float rs = 1.0f;
+          if constexpr (NORM_A) {
+            const float* parts = p.a_row_sumsq + (int64_t)(row0 + 16 * I + lrv) * CS_SUMSQ_PARTS;
+            const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
+            const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
+            rs = rsqrtf(ss / (float)p.K + p.norm_eps);
+          }
+#pragma unroll
+          for (int r = 0; r < 4; ++r) rv[I][r] = NORM_A ? lane_xchg(rs, ((lane_v >> 4) * 4 + r) << 2) : 1.0f;
+        }
+        static_for<5>([&](auto d_c) {
+          constexpr int Dd = decltype(d_c)::value, J = 10 + Dd;
+          static_for<2>([&](auto t_c) {
+            constexpr int T = decltype(t_c)::value;
+            bf16x8_t f;
+            static_for<8>([&](auto e_c) {
+              constexpr int E = decltype(e_c)::value, I = 2 * T + E / 4, R = (I * NT + J) * 4 + E % 4;
+              float t;
+              asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R));
+              f[E] = f2bf(t * rv[I][E % 4] + bias_v[Dd]);
+            });
+            vf8[Dd][T] = f;
+          });
+        });
+      }
+      // ---- O^T[dim][query] = V^T.P^T: block (d, qb) in a[4(4d + qb) ..] (every accumulator has been read by now)
+      asm volatile("s_nop 7" ::: "memory");
+      static_for<20>([&](auto b_c) {
+        constexpr int Dd = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = (Dd * 4 + QB) * 4;
+        const bf16x8_t va = vf8[Dd][0], pb = pf8[QB][0];
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(va), "v"(pb), "n"(R), "n"(R + 3));
+      });
+      static_for<20>([&](auto b_c) {
+        constexpr int Dd = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = (Dd * 4 + QB) * 4;
+        const bf16x8_t va = vf8[Dd][1], pb = pf8[QB][1];
+        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(va), "v"(pb), "n"(R), "n"(R + 3));
+      });
+      asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+      // ---- out[row0 + 16qb + lr][head*80 + 16d + 4kq ..+3] = O^T / l
+      bf16_t* const out0 = (bf16_t*)p.C + (int64_t)(row0 + lr) * p.ldc + head * HD + 4 * kq;
+      static_for<4>([&](auto q_c) {
+        constexpr int QB = decltype(q_c)::value;
+        static_for<5>([&](auto d_c) {
+          constexpr int Dd = decltype(d_c)::value, R = (Dd * 4 + QB) * 4;
+          bf16x4_t o;
+          static_for<4>([&](auto r_c) {
+            constexpr int Rr = decltype(r_c)::value;
+            float t;
+            asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R + Rr));
+            o[Rr] = f2bf(t * inv_l[QB]);
+          });
+          *(bf16x4_t*)(out0 + (int64_t)(16 * QB) * p.ldc + 16 * Dd) = o;
+        });
+      });
+    };
     // ---- epilogue.  Accumulator (i, j), element r = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
     //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
     //      With one wave per SIMD nothing overlaps the epilogue and it is bound by instruction issue (a vector
@@ -788,7 +1023,17 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       });
     };
     // (p.fast_epilogue: the host has checked that every matrix the epilogue touches lies within 32-bit byte offsets)
-    if (p.fast_epilogue && m0 + BM <= p.M && n0 + BN <= p.N) epilogue(std::true_type{});
+    if constexpr (EPI == CS_EPI_QKV_WATTN) {
+      wattn_epilogue(0);
+      // the next tile's source offsets and the fragment offsets are recomputed rather than kept in registers across
+      // this epilogue (the lane number comes from the hardware again, not from a register held since the start)
+      if (!has_next) break;
+      setup_sources(m0_next, n0_next);
+      int lane_again = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+      asm volatile("" : "+v"(lane_again));   // else the compiler proves the offsets loop-invariant and keeps them
+      setup_frag_offsets(lane_again);
+    }
+    else if (p.fast_epilogue && m0 + BM <= p.M && n0 + BN <= p.N) epilogue(std::true_type{});
     else epilogue(std::false_type{});
     if (!has_next) break;
     vb = vb_next;

@@ -61,6 +61,8 @@ class CsGemmArgs(ctypes.Structure):
         ("conv_h", c_int32),
         ("conv_w", c_int32),
         ("conv_patch", c_int32),
+        ("attn_cos_sin", c_void_p),
+        ("attn_scale_log2e", ctypes.c_float),
     ]
 
 
@@ -69,6 +71,7 @@ _SIGNATURES: dict[str, list] = {
     "cs_abi_version": [],
     "cs_gemm": [POINTER(CsGemmArgs), c_void_p],
     "cs_gemm_rmsnorm_noalloc": [POINTER(CsGemmArgs), c_void_p],
+    "cs_qkv_window_attn": [POINTER(CsGemmArgs), c_void_p, c_float, c_int32, c_int32, c_void_p],
     "cs_row_sumsq": [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p],
     "cs_row_stats": [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
     "cs_rmsnorm": [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_float, c_int32, c_void_p],

@@ -742,6 +742,99 @@ def _patchify_nchw_impl(out, pixels, patch) -> None:
              "cs_patchify_nchw")
 
 
+# ------------------------------------------------- QKV projection + rotary + window attention in one launch
+QKV_WATTN_HEAD_DIM = 80      # the head dim the fused kernel is written for (Qwen2.5-VL: 1280 / 16)
+QKV_WATTN_TILE_ROWS = 256    # packed weight rows per head
+QKV_WATTN_WINDOW = 64        # rows of every attention segment
+
+
+def qkv_window_attn_row_order(heads: int) -> torch.Tensor:
+    """Row r of the packed [heads*256, K] weight of `qkv_window_attn` is row order[r] of the reference's qkv weight
+    [3*heads*80, K] (q | k | v blocks, qwen2_5_vl.py:65-84), or -1 for a zero row.  Per head: tile row
+    rho = 32 (J/2) + 8 kq + 4 (J%2) + r for fragment J, lane group kq, element r; q and k fragments (J < 5, J < 10) put
+    both halves of every rotary pair into one lane group, the v fragments (J < 15) hold 16 consecutive head dims."""
+    d, half = QKV_WATTN_HEAD_DIM, QKV_WATTN_HEAD_DIM // 2
+    order = torch.full((heads, QKV_WATTN_TILE_ROWS), -1, dtype=torch.int64)
+    for J in range(15):
+        for kq in range(4):
+            for r in range(4):
+                rho = 32 * (J // 2) + 8 * kq + 4 * (J % 2) + r
+                if J < 10:
+                    s = 4 * (J % 5) + r
+                    dim = 10 * kq + s if s < 10 else half + 10 * kq + (s - 10)
+                    block = 0 if J < 5 else 1
+                else:
+                    dim = 16 * (J - 10) + 4 * kq + r
+                    block = 2
+                for h in range(heads):
+                    order[h, rho] = block * heads * d + h * d + dim
+    return order.reshape(-1)
+
+
+def pack_qkv_window_attn(w: torch.Tensor, b: torch.Tensor, heads: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """The qkv weight [3*heads*80, K] and bias [3*heads*80] in the row order `qkv_window_attn` takes (done once, at load)."""
+    if w.dim() != 2 or w.shape[0] != 3 * heads * QKV_WATTN_HEAD_DIM or b.shape != (w.shape[0],):
+        raise ValueError(f"qkv weight must be [3*{heads}*{QKV_WATTN_HEAD_DIM}, K] with a matching bias")
+    order = qkv_window_attn_row_order(heads).to(w.device)
+    keep = (order >= 0).unsqueeze(1)
+    rows = order.clamp_min(0)
+    wp = torch.where(keep, w[rows], torch.zeros((), dtype=w.dtype, device=w.device)).contiguous()
+    bp = torch.where(keep[:, 0], b[rows], torch.zeros((), dtype=b.dtype, device=b.device)).contiguous()
+    return wp, bp
+
+
+def qkv_window_attn(x: torch.Tensor, w_packed: torch.Tensor, b_packed: torch.Tensor, cos_sin: torch.Tensor, heads: int,
+                    scale: float, *, a_row_sumsq: torch.Tensor | None = None, norm_eps: float = 0.0,
+                    out: torch.Tensor | None = None) -> torch.Tensor:
+    """attention(rotary(x . Wq^T + bq), rotary(x . Wk^T + bk), x . Wv^T + bv) over windows of 64 rows, one launch.
+
+    Replaces qkv Linear -> split -> rotary -> flash_attn_varlen_func (qwen2_5_vl.py:93-120) for a sequence whose
+    attention segments are ALL 64 rows starting at multiples of 64.  `w_packed`, `b_packed` come from
+    `pack_qkv_window_attn`; with `a_row_sumsq` the rows of `x` are RMS-normalised on the way (the norm weight folded
+    into the packed weight's columns, as for `gemm`).  Raises ValueError for shapes the kernel does not take."""
+    if out is None:
+        out = torch.empty((x.shape[0], heads * QKV_WATTN_HEAD_DIM), dtype=torch.bfloat16, device=x.device)
+    torch.ops.cornserve_amd.qkv_window_attn_(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps)
+    return out
+
+
+def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps) -> None:
+    lib = _l.load()
+    _rows_2d(x, torch.bfloat16, "x")
+    _rows_2d(w_packed, torch.bfloat16, "w_packed")
+    _rows_2d(out, torch.bfloat16, "out")
+    _req(b_packed, torch.bfloat16, "b_packed")
+    _req(cos_sin, torch.float32, "cos_sin")
+    M, K = x.shape
+    d = QKV_WATTN_HEAD_DIM
+    if heads < 1 or tuple(w_packed.shape) != (heads * QKV_WATTN_TILE_ROWS, K):
+        raise ValueError(f"w_packed must be [{heads}*{QKV_WATTN_TILE_ROWS}, {K}], got {tuple(w_packed.shape)}")
+    if tuple(b_packed.shape) != (heads * QKV_WATTN_TILE_ROWS,) or not b_packed.is_contiguous():
+        raise ValueError(f"b_packed must be a contiguous [{heads * QKV_WATTN_TILE_ROWS}] tensor")
+    if M % QKV_WATTN_WINDOW:
+        raise ValueError(f"the rows of x ({M}) must be a whole number of {QKV_WATTN_WINDOW}-row windows")
+    if tuple(cos_sin.shape) != (M, d) or not cos_sin.is_contiguous():
+        raise ValueError(f"cos_sin must be a contiguous fp32 [{M}, {d}] table")
+    if out.shape[0] < M or out.shape[1] < heads * d:
+        raise ValueError(f"out must be bf16 [>={M}, >={heads * d}], got {tuple(out.shape)}")
+    if a_row_sumsq is not None:
+        _req(a_row_sumsq, torch.float32, "a_row_sumsq")
+        if a_row_sumsq.dim() != 2 or a_row_sumsq.shape[1] != SUMSQ_PARTS or not a_row_sumsq.is_contiguous() or a_row_sumsq.shape[0] < M:
+            raise ValueError(f"a_row_sumsq must be a contiguous fp32 [>=M, {SUMSQ_PARTS}] tensor")
+    on = {t.device for t in (out, x, w_packed, b_packed, cos_sin, a_row_sumsq) if t is not None}
+    if len(on) != 1:
+        raise ValueError(f"qkv_window_attn operands live on different devices: {sorted(map(str, on))}")
+    args = _l.CsGemmArgs()
+    args.A, args.lda = x.data_ptr(), x.stride(0)
+    args.W, args.ldw = w_packed.data_ptr(), w_packed.stride(0)
+    args.bias = b_packed.data_ptr()
+    args.C, args.ldc = out.data_ptr(), out.stride(0)
+    args.M, args.N, args.K = M, heads * QKV_WATTN_TILE_ROWS, K
+    args.a_row_sumsq = _ptr(a_row_sumsq)
+    args.norm_eps = norm_eps
+    _l.check(lib.cs_qkv_window_attn(ctypes.byref(args), cos_sin.data_ptr(), scale, heads, d, _stream()), "cs_qkv_window_attn")
+
+
 # ------------------------------------------------------------------------------- operator registration
 # One operator per kernel entry point, in the `cornserve_amd` namespace.  Operators ending in `_` write into their
 # leading tensor argument(s) and return nothing; every argument that reaches a kernel as a pointer is a Tensor of the
@@ -775,6 +868,8 @@ _OPERATORS: dict[str, tuple[str, object]] = {
     "qwen_patchify_u8_": ("(Tensor(a!) out, Tensor frames, Tensor table, int patch, int merge, int temporal) -> ()",
                           _qwen_patchify_u8_impl),
     "patchify_nchw_": ("(Tensor(a!) out, Tensor pixels, int patch) -> ()", _patchify_nchw_impl),
+    "qkv_window_attn_": ("(Tensor(a!) out, Tensor x, Tensor w_packed, Tensor b_packed, Tensor cos_sin, int heads, "
+                         "float scale, Tensor? a_row_sumsq, float norm_eps) -> ()", _qkv_window_attn_impl),
 }
 
 

@@ -123,6 +123,9 @@ typedef struct CsGemmArgs {
    * must be even (pixel pairs are fetched as 4-byte words); pixels past the last whole patch are not read, as the
    * convolution drops them.  CS_EPI_BIAS (with or without the position addend), bf16 W, no a_rows.                  */
   int32_t conv_c, conv_h, conv_w, conv_patch;
+  /* filled in by cs_qkv_window_attn (the rotary table and softmax scale of its fused epilogue)                      */
+  const float* attn_cos_sin;
+  float attn_scale_log2e;
 } CsGemmArgs;
 #define CS_SUMSQ_PARTS 8
 
@@ -247,6 +250,27 @@ int cs_attn_varlen(const void* q, const void* k, const void* v, int64_t ld, void
 int cs_attn_varlen_keys_rotated(const void* q, const void* k, const void* v, int64_t ld, void* out, int64_t ldo,
                                 const int32_t* work, int32_t n_work, int32_t heads, int32_t head_dim, float scale,
                                 const float* cos_sin, int32_t max_seqlen, void* stream);
+/* QKV projection + rotary + window attention in ONE launch, for a sequence whose windows are all full: every segment of
+ * cu_window_seqlens (qwen2_5_vl.py:357-386,431-436) is 64 rows starting at a multiple of 64 -- any batch of images whose
+ * sides are multiples of 8 patches.  Replaces, for the window-attention blocks, the chain F.linear (qkv, linear.py:183)
+ * -> split_qkv (:65-84) -> apply_rotary_pos_emb_vision (:26-33) -> flash_attn_varlen_func (:110-120): each workgroup
+ * computes the q, k and v of ONE head for four windows (the GEMM of cs_gemm's direct-to-LDS kernel, one window per
+ * wavefront), rotates q and k in fp32, and runs softmax(q k^T scale) v on the matrix cores without leaving registers;
+ * the [L, 3*heads*head_dim] qkv tensor never exists.
+ *   gemm->A, lda, K, M: the activations [M, K] (M a multiple of 64); a_row_sumsq / norm_eps as for cs_gemm (folded RMSNorm)
+ *   gemm->W, ldw, bias: the qkv weight and bias PACKED per head, [heads * 256, K] and [heads * 256]: tile row
+ *     rho = 32 (J/2) + 8 kq + 4 (J%2) + r of head h, for fragment J = 0..15, kq = 0..3, r = 0..3, holds
+ *       J < 5:   q row h*80 + dim(kq, 4J + r)          with dim(kq, s) = 10 kq + s (s < 10), 40 + 10 kq + s - 10 (s >= 10)
+ *       J < 10:  k row h*80 + dim(kq, 4(J-5) + r)
+ *       J < 15:  v row h*80 + 16 (J-10) + 4 kq + r
+ *       J = 15:  zeros
+ *     (both halves of a rotary pair in one lane; eight consecutive slots of a lane = one MFMA operand)
+ *   gemm->C, ldc: out [M, heads * 80] bf16;  gemm->N = heads * 256;  other fields zero
+ *   cos_sin: the [M, 80] fp32 table of cs_vit_index;  scale = head_dim^-0.5;  head_dim must be 80.
+ * CS_ERR_UNSUPPORTED for any other shape (the caller then takes cs_gemm + cs_attn_varlen).                          */
+int cs_qkv_window_attn(const CsGemmArgs* gemm, const float* cos_sin, float scale, int32_t heads, int32_t head_dim,
+                       void* stream);
+
 /* Host routine: expand cu_seqlens_host[n_seg+1] into query-block work items of at most block_q rows
  * (block_q = cs_attn_block_q(max_seqlen)).  Writes n_work items of 4 int32 into work_host.      */
 int cs_attn_block_q(int32_t max_seqlen);

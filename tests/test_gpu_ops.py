@@ -1039,3 +1039,58 @@ def test_attention_random_segments(ops, dev):
         plan = ops.attn_plan(np.array(cu, np.int32), dev)
         got = ops.attn_varlen(qkv[:, :H], qkv[:, H:2 * H], qkv[:, 2 * H:], plan, nh, d, d**-0.5, cs)
         close(got, attn_ref(qkv, cu, nh, d, ang), 2**-6, f"attention d={d} heads={nh} lens={lens[:8]} rotary={rotary}")
+
+
+# ------------------------------------------------ QKV projection + rotary + window attention in one launch
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,K,heads,fold", [(256, 192, 1, False), (512, 1280, 16, False), (8192, 1280, 16, True),
+                                            (320, 256, 3, True), (64, 1280, 2, False)])
+def test_qkv_window_attn_against_fp32_and_the_unfused_chain(ops, dev, M, K, heads, fold):
+    d = 80
+    x = rnd((M, K), 1.0, 11, dev)
+    w = rnd((3 * heads * d, K), K**-0.5, 12, dev)
+    b = rnd((3 * heads * d,), 0.5, 13, dev)
+    g = torch.Generator().manual_seed(14)
+    ang = torch.rand((M, d // 2), generator=g) * 6.0
+    cs = torch.cat([ang.cos(), ang.sin()], dim=1).float().contiguous().to(dev)
+    eps = 1e-6
+    sums = ops.row_sumsq(x) if fold else None
+    wp, bp = ops.pack_qkv_window_attn(w, b, heads)
+    got = ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, a_row_sumsq=sums, norm_eps=eps)
+    # fp32 restatement: (normalised) rows . W^T + b, rotary, softmax attention inside windows of 64 rows
+    xf = x.float().cpu()
+    if fold:
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    qkv = xf @ w.float().cpu().T + b.float().cpu()
+    cu = list(range(0, M + 1, 64))
+    ref = attn_ref(qkv, cu, heads, d, ang)
+    close(got, ref, 2**-6, f"fused qkv + window attention M={M} K={K} heads={heads} fold={fold}")
+    # the chain it replaces (bf16 qkv tensor in between) sits within the same distance of the fp32 result
+    qkv_dev = ops.gemm(x, w, b, a_row_sumsq=sums, norm_eps=eps)
+    H = heads * d
+    plan = ops.attn_plan(np.array(cu, np.int32), dev)
+    chain = ops.attn_varlen(qkv_dev[:, :H], qkv_dev[:, H:2 * H], qkv_dev[:, 2 * H:], plan, heads, d, d**-0.5, cs)
+    close(chain, ref, 2**-6, "unfused chain")
+    err_fused = (got.float().cpu() - ref).abs().max().item()
+    err_chain = (chain.float().cpu() - ref).abs().max().item()
+    assert err_fused <= 1.5 * err_chain + 1e-3, (err_fused, err_chain)
+
+
+@pytest.mark.gpu
+def test_qkv_window_attn_rejects_what_the_kernel_does_not_take(ops, dev):
+    d, heads, K = 80, 2, 192
+    x = rnd((128, K), 1.0, 1, dev)
+    w = rnd((3 * heads * d, K), 0.1, 2, dev)
+    b = rnd((3 * heads * d,), 0.1, 3, dev)
+    wp, bp = ops.pack_qkv_window_attn(w, b, heads)
+    cs = torch.zeros((128, d), device=dev)
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x[:100], wp, bp, cs[:100], heads, d**-0.5)            # not whole windows
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x, wp[:256], bp, cs, heads, d**-0.5)                  # weight not packed per head
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x, wp, bp, cs[:, :40].contiguous(), heads, d**-0.5)   # table of another head dim
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x, wp, bp, cs.double(), heads, d**-0.5)
+    with pytest.raises(ValueError):
+        ops.pack_qkv_window_attn(w[:100], b[:100], heads)

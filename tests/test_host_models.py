@@ -439,3 +439,20 @@ def test_scheduler_batches_like_the_reference_and_bounds_patches():
     assert b.to_worker_batch()._uploaded is marker
     tiles = sc.ProcessedEmbeddingData("t", Modality.IMAGE, "m", {"pixel_values": torch.zeros(3, 3, 28, 42)})
     assert sc.patch_count(tiles) == 3 * 2 * 3 and sc.patch_count(item(0, grid=(2, 4, 6))) == 48
+
+
+def test_qkv_window_attn_row_order_is_a_permutation_with_padding():
+    from cornserve_amd import ops as o
+    heads = 3
+    order = o.qkv_window_attn_row_order(heads)
+    assert order.shape == (heads * 256,)
+    used = order[order >= 0]
+    assert sorted(used.tolist()) == list(range(3 * heads * 80))      # every qkv row exactly once
+    pad = [32 * 7 + 8 * kq + 4 + r for kq in range(4) for r in range(4)]
+    assert (order.reshape(heads, 256)[:, pad] == -1).all()           # fragment 15 of every head is padding
+    # both halves of a rotary pair sit in the same lane group of the same head: dims d and d + 40
+    per_head = order.reshape(heads, 256)[1]
+    pos = {int(r): i for i, r in enumerate(per_head.tolist()) if r >= 0}
+    for d in range(40):
+        a, b = pos[80 + d], pos[80 + d + 40]      # q rows of head 1
+        assert (a % 32) // 8 == (b % 32) // 8
