@@ -248,8 +248,14 @@ class QwenVisionBase(EricModel):
 
 class Qwen2_5_VisionTransformer(QwenVisionBase):
     def __init__(self, config: Any, weight_format: str = "bf16", fold_norm: bool = True,
-                 split_residual: bool = True) -> None:
-        """`split_residual`: carry the residual stream (:175,177) with 16 significant bits -- the bf16 tensor every
+                 split_residual: bool = True, fuse_window_attn: bool = True) -> None:
+        """`fuse_window_attn`: run qkv projection + rotary + window attention of a block (:93-120) as ONE launch
+        (`ops.qkv_window_attn`: q, k and v stay in registers, the [L, 3*hidden] tensor is never written) whenever every
+        window of the batch is a full 64-row window -- all images with sides that are multiples of 8 patches.  Other
+        batches, fp8 weights and head dims other than 80 take the separate kernels.  q and k are then rounded to bf16
+        once (after the rotation) instead of twice; results stay inside the parity tolerance.
+
+        `split_residual`: carry the residual stream (:175,177) with 16 significant bits -- the bf16 tensor every
         kernel reads plus a byte plane with the next 8 mantissa bits, joined and re-split inside the two residual GEMMs
         of a block -- so that the 2 x depth additions do not each round the stream to 8 bits.  A bf16 stream (False:
         the reference's arithmetic when loaded in bf16) drifts from the exact result by about 2e-2 of the output range
@@ -288,6 +294,12 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         self.fold_norm = (bool(fold_norm) and weight_format == "bf16" and H % 64 == 0 and 192 <= H <= 160 * ops.SUMSQ_PARTS
                           and _round_up(self.intermediate_size, 64) >= 192)
 
+        # (one launch for qkv + rotary + window attention: bf16 weights, heads of 80, K a multiple of 64 from 192 up,
+        # windows of 64 rows)
+        win_rows = (self.window_size // self.spatial_merge_size // self.patch_size) ** 2 * self.spatial_merge_unit
+        self.fuse_window_attn = (bool(fuse_window_attn) and weight_format == "bf16" and H % 64 == 0 and H >= 192
+                                 and self.head_dim == ops.QKV_WATTN_HEAD_DIM and win_rows == ops.QKV_WATTN_WINDOW)
+
         self.patch_embed = _PatchEmbed(self.in_channels, self.hidden_size, self.temporal_patch_size, self.patch_size)
         self.blocks = nn.ModuleList([_Block(self.hidden_size, self.intermediate_size) for _ in range(vc.depth)])
         self.merger = _Merger(self.out_hidden_size, self.hidden_size, self.spatial_merge_size)
@@ -305,7 +317,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         pk: dict = {"Ip": Ip}
         pk["pe_w"] = self.patch_embed.proj.weight.reshape(H, -1).contiguous()
         blocks = []
-        for blk in self.blocks:
+        for i, blk in enumerate(self.blocks):
             gu_w = torch.zeros((2 * Ip, H), dtype=self.dtype, device=dev)
             gu_b = torch.zeros(2 * Ip, dtype=self.dtype, device=dev)
             gu_w[0 : 2 * I : 2] = blk.mlp.gate_proj.weight
@@ -328,6 +340,8 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                     "down": self._lin(down_w, blk.mlp.down_proj.bias),
                 }
             )
+            if self.fuse_window_attn and i not in self.fullatt_block_indexes:
+                blocks[-1]["qkv_wattn"] = ops.pack_qkv_window_attn(qkv_w, blk.attn.qkv.bias.to(self.dtype), self.num_heads)
         pk["blocks"] = blocks
         pk["ln_q"] = self.merger.ln_q.weight
         pk["fc1"] = self._lin(self.merger.mlp[0].weight, self.merger.mlp[0].bias)
@@ -359,8 +373,10 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         # one host-to-device copy for the three small arrays
         meta, dwin, dfull = ops.host_to_device_packed([sl.item_meta, work_win, work_full], dev)
         ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, merge, win, self._ensure_packed()["inv_freq"])
+        # every window a whole one (64 rows from a multiple of 64 on): the fused window-attention launch applies
+        windows_whole = bool(np.all(np.diff(sl.cu_window) == ops.QKV_WATTN_WINDOW))
         return (ix, ops.AttnPlan(dwin, work_win.shape[0], max_win), ops.AttnPlan(dfull, work_full.shape[0], max_full),
-                sl.total_patches)
+                sl.total_patches, windows_whole)
 
     def forward_device(self, pixel_values: torch.Tensor, grid_thw: np.ndarray, mark=None) -> list[torch.Tensor]:
         """pixel_values: bf16 [L, C*T*P*P] already on the device; grid_thw: host int64 [n,3].
@@ -382,7 +398,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
             if len(groups) > 1:
                 return self._forward_in_groups(pixel_values, grid_thw, groups, mark)
         mark("index")
-        ix, plan_win, plan_full, L = self._index(grid_thw)
+        ix, plan_win, plan_full, L, windows_whole = self._index(grid_thw)
         if pixel_values.shape[0] != L:
             raise ValueError(f"pixel_values has {pixel_values.shape[0]} rows but grid_thw describes {L} patches")
 
@@ -405,16 +421,27 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         for i, b in enumerate(pk["blocks"]):
             full = i in self.fullatt_block_indexes
             plan = plan_full if full else plan_win
-            if fold:
-                mark("gemm_qkv")
-                self._g(x, b["qkv"], out=qkv, a_row_sumsq=ss, norm_eps=eps)
+            if windows_whole and "qkv_wattn" in b:
+                wp, bp = b["qkv_wattn"]
+                if fold:
+                    mark("gemm_qkv_attn_window")
+                    ops.qkv_window_attn(x, wp, bp, ix.cos_sin, nh, scale, a_row_sumsq=ss, norm_eps=eps, out=att)
+                else:
+                    mark("norm")
+                    ops.rmsnorm(x, b["n1"], eps, out=n)
+                    mark("gemm_qkv_attn_window")
+                    ops.qkv_window_attn(n, wp, bp, ix.cos_sin, nh, scale, out=att)
             else:
-                mark("norm")
-                ops.rmsnorm(x, b["n1"], eps, out=n)
-                mark("gemm_qkv")
-                self._g(n, b["qkv"], out=qkv)
-            mark("attn_full" if full else "attn_window")
-            ops.attn_varlen_rotary_(qkv, plan, nh, d, scale, ix.cos_sin, out=att)
+                if fold:
+                    mark("gemm_qkv")
+                    self._g(x, b["qkv"], out=qkv, a_row_sumsq=ss, norm_eps=eps)
+                else:
+                    mark("norm")
+                    ops.rmsnorm(x, b["n1"], eps, out=n)
+                    mark("gemm_qkv")
+                    self._g(n, b["qkv"], out=qkv)
+                mark("attn_full" if full else "attn_window")
+                ops.attn_varlen_rotary_(qkv, plan, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")
             if fold:
                 self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss, **res)

@@ -40,12 +40,12 @@ def check(got: torch.Tensor, ref: torch.Tensor, rel: float, what: str):
     assert err <= rel, f"{what}: max rel err {err:.4g} > {rel}"
 
 
-def build_qwen(dev, depth, fullatt, seed, weight_format="bf16", fold_norm=True):
+def build_qwen(dev, depth, fullatt, seed, weight_format="bf16", fold_norm=True, **kw):
     from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
 
     cfg = synth.qwen_vision_config(depth=depth, fullatt_block_indexes=fullatt)
     sd = synth.qwen_state_dict(cfg, seed=seed)
-    model = Qwen2_5_VisionTransformer(cfg, weight_format=weight_format, fold_norm=fold_norm)
+    model = Qwen2_5_VisionTransformer(cfg, weight_format=weight_format, fold_norm=fold_norm, **kw)
     inc = model.load_state_dict(sd, strict=False)
     assert not inc.missing_keys and not inc.unexpected_keys
     model = model.to(device=dev, dtype=torch.bfloat16).eval()
@@ -82,6 +82,37 @@ def test_qwen_without_folded_norms(dev, golden_dir):
     assert folded.fold_norm
     out_f = folded(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})[0]
     check(out_f, out, REL_BF16, "folded vs unfolded")
+
+
+@pytest.mark.parametrize("fold_norm", [True, False])
+def test_qwen_one_launch_window_attention_against_separate_kernels(dev, fold_norm):
+    """Batches whose windows are all whole (sides multiples of 8 patches) run qkv + rotary + window attention of a
+    block as one launch; the same weights through the separate kernels, and both against the oracle.  A ragged batch
+    takes the separate kernels in either model."""
+    fused, sd, ocfg = build_qwen(dev, 4, (3,), seed=5, fold_norm=fold_norm)
+    plain, _, _ = build_qwen(dev, 4, (3,), seed=5, fold_norm=fold_norm, fuse_window_attn=False)
+    assert fused.fuse_window_attn and not plain.fuse_window_attn
+    px, grid = synth.qwen_inputs([(1, 32, 32), (2, 8, 16), (1, 24, 40)], seed=5)
+    g = torch.cat(grid).numpy().astype(np.int64)
+    pv = torch.cat(px).to(dev, torch.bfloat16)
+    stages: list[str] = []
+    a = torch.cat(fused.forward_device(pv, g, mark=stages.append))
+    assert stages.count("gemm_qkv_attn_window") == 3 and stages.count("attn_window") == 0 and stages.count("attn_full") == 1
+    stages.clear()
+    b = torch.cat(plain.forward_device(pv, g, mark=stages.append))
+    assert stages.count("gemm_qkv_attn_window") == 0 and stages.count("attn_window") == 3
+    check(a, b, REL_BF16, "one launch vs separate kernels")
+    ref = torch.cat(oq.forward(sd, ocfg, px, grid, dtype=torch.float32))
+    check(a, ref, REL_BF16, "one launch vs fp32 oracle")
+    check(a, torch.cat(oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)), REL_BF16, "one launch vs bf16 oracle")
+    # ragged sides: windows at the edges are partial, so the fused model runs the separate kernels too -- same bits
+    px, grid = synth.qwen_inputs([(1, 20, 36), (1, 32, 32)], seed=6)
+    g = torch.cat(grid).numpy().astype(np.int64)
+    pv = torch.cat(px).to(dev, torch.bfloat16)
+    stages.clear()
+    a = torch.cat(fused.forward_device(pv, g, mark=stages.append))
+    assert stages.count("gemm_qkv_attn_window") == 0
+    assert torch.equal(a, torch.cat(plain.forward_device(pv, g)))
 
 
 def test_qwen_shapes_the_folded_gemms_cannot_take(dev):
