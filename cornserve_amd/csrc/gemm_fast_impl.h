@@ -491,6 +491,11 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       static_assert(EPI != CS_EPI_QKV_WATTN || (BM == 256 && BN == 256 && WAVES_M == 4 && WAVES_N == 1 && !W_FP8),
                     "one 64-row window per wave, one head per column tile");
       constexpr int HD = 80, HALF = 40;
+      // A register written by a vector instruction must not be read by an MFMA in the next few cycles.  The compiler
+      // pads that for its own MFMAs but cannot see into these, and it is free to place the instruction that produces
+      // an operand right in front of the statement that uses it: every MFMA of this epilogue carries its own wait
+      // (the previous MFMA still occupies the pipeline meanwhile, so the wait costs nothing).
+#define CS_OPERAND_SETTLE "s_nop 3\n\t"
       constexpr bool NORM_A = FUSE == FUSE_NORM_A;
       auto s_reg = [](int b) constexpr { return b < 10 ? 4 * b : 64 + 4 * (b - 10); };   // first register of S^T block b
       int lane_e = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));   // the lane number, afresh
@@ -551,8 +556,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           float o[20];
 #pragma unroll
           for (int t = 0; t < 10; ++t) {
-            o[t] = rot_first(x[t], x[t + 10], co[t], si[t]);
-            o[t + 10] = rot_second(x[t], x[t + 10], co[t], si[t]);
+            // (fused multiply-adds: one rounding less than the stand-alone rotary kernel, one instruction less too)
+            o[t] = __builtin_fmaf(x[t], co[t], -(x[t + 10] * si[t]));
+            o[t + 10] = __builtin_fmaf(x[t + 10], co[t], x[t] * si[t]);
           }
           bf16x8_t f0, f1;
           bf16x4_t f2;
@@ -574,27 +580,25 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       //      (the transposed V accumulators are still where the main loop put them: fragments 10..14 of every row
       //      block): a[4b ..] for b < 10, a[64 + 4(b - 10) ..] above.  Steps outermost, so that consecutive MFMAs
       //      never depend on each other.
-      asm volatile("s_nop 7" ::: "memory");   // the operands above were written by vector instructions
       static_for<16>([&](auto b_c) {
         constexpr int KB = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = s_reg(KB * 4 + QB);
         const bf16x8_t ka = kf8[KB][0], qb = qf8[QB][0];   // (named copies: asm operands alone do not capture)
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
+        asm volatile(CS_OPERAND_SETTLE "v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
       });
       static_for<16>([&](auto b_c) {
         constexpr int KB = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = s_reg(KB * 4 + QB);
         const bf16x8_t ka = kf8[KB][1], qb = qf8[QB][1];
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
+        asm volatile(CS_OPERAND_SETTLE "v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
       });
       static_for<16>([&](auto b_c) {
         constexpr int KB = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = s_reg(KB * 4 + QB);
         const bf16x4_t ka = kf4[KB], qb = qf4[QB];
-        asm volatile("v_mfma_f32_16x16x16_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
+        asm volatile(CS_OPERAND_SETTLE "v_mfma_f32_16x16x16_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(ka), "v"(qb), "n"(R), "n"(R + 3));
       });
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
       // ---- softmax over the 64 keys of a query row (16 per lane, 4 lanes per row); P packed as the operand of the
       //      second product: key step t = blocks 2t, 2t+1
       bf16x8_t pf8[4][2];
-      float inv_l[4];
       static_for<4>([&](auto q_c) {
         constexpr int QB = decltype(q_c)::value;
         float sv[16];
@@ -610,18 +614,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         mx = fmaxf(mx, lane_xchg(mx, x16));
         mx = fmaxf(mx, lane_xchg(mx, x32));
         const float mb = mx * sl2;
-        float sum = 0.f;
         bf16x8_t f[2];
 #pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const float pv = __builtin_amdgcn_exp2f(sv[e] * sl2 - mb);
-          const bf16_t pb = f2bf(pv);
-          sum += bf2f(pb);   // the denominator of exactly the weights the second product uses
-          f[e >> 3][e & 7] = pb;
-        }
-        sum += lane_xchg(sum, x16);
-        sum += lane_xchg(sum, x32);
-        inv_l[QB] = 1.0f / sum;
+        for (int e = 0; e < 16; ++e) f[e >> 3][e & 7] = f2bf(__builtin_amdgcn_exp2f(sv[e] * sl2 - mb));
         pf8[QB][0] = f[0];
         pf8[QB][1] = f[1];
       });
@@ -668,22 +663,41 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         });
       }
       // ---- O^T[dim][query] = V^T.P^T: block (d, qb) in a[4(4d + qb) ..] (every accumulator has been read by now)
-      asm volatile("s_nop 7" ::: "memory");
       static_for<20>([&](auto b_c) {
         constexpr int Dd = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = (Dd * 4 + QB) * 4;
         const bf16x8_t va = vf8[Dd][0], pb = pf8[QB][0];
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(va), "v"(pb), "n"(R), "n"(R + 3));
+        asm volatile(CS_OPERAND_SETTLE "v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(va), "v"(pb), "n"(R), "n"(R + 3));
       });
       static_for<20>([&](auto b_c) {
         constexpr int Dd = decltype(b_c)::value / 4, QB = decltype(b_c)::value % 4, R = (Dd * 4 + QB) * 4;
         const bf16x8_t va = vf8[Dd][1], pb = pf8[QB][1];
-        asm volatile("v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(va), "v"(pb), "n"(R), "n"(R + 3));
+        asm volatile(CS_OPERAND_SETTLE "v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(va), "v"(pb), "n"(R), "n"(R + 3));
       });
+      // the softmax denominators come from the matrix cores as well: a row block of ones in place of V^T sums exactly
+      // the rounded weights that the product above used, and leaves the sum of query lr in every register of the lane
+      {
+        bf16x8_t ones;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) ones[e] = f2bf(1.0f);
+        static_for<4>([&](auto q_c) {
+          constexpr int QB = decltype(q_c)::value, R = 80 + 4 * QB;
+          const bf16x8_t pb = pf8[QB][0], one = ones;
+          asm volatile(CS_OPERAND_SETTLE "v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, 0" ::"v"(one), "v"(pb), "n"(R), "n"(R + 3));
+        });
+        static_for<4>([&](auto q_c) {
+          constexpr int QB = decltype(q_c)::value, R = 80 + 4 * QB;
+          const bf16x8_t pb = pf8[QB][1], one = ones;
+          asm volatile(CS_OPERAND_SETTLE "v_mfma_f32_16x16x32_bf16 a[%2:%3], %0, %1, a[%2:%3]" ::"v"(one), "v"(pb), "n"(R), "n"(R + 3));
+        });
+      }
       asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
       // ---- out[row0 + 16qb + lr][head*80 + 16d + 4kq ..+3] = O^T / l
       bf16_t* const out0 = (bf16_t*)p.C + (int64_t)(row0 + lr) * p.ldc + head * HD + 4 * kq;
       static_for<4>([&](auto q_c) {
         constexpr int QB = decltype(q_c)::value;
+        float l_sum;
+        asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(l_sum) : "n"(80 + 4 * QB));
+        const float inv = 1.0f / l_sum;
         static_for<5>([&](auto d_c) {
           constexpr int Dd = decltype(d_c)::value, R = (Dd * 4 + QB) * 4;
           bf16x4_t o;
@@ -691,12 +705,13 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
             constexpr int Rr = decltype(r_c)::value;
             float t;
             asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R + Rr));
-            o[Rr] = f2bf(t * inv_l[QB]);
+            o[Rr] = f2bf(t * inv);
           });
           *(bf16x4_t*)(out0 + (int64_t)(16 * QB) * p.ldc + 16 * Dd) = o;
         });
       });
     };
+#undef CS_OPERAND_SETTLE
     // ---- epilogue.  Accumulator (i, j), element r = C[m][n], m = m0 + wm*WTM + 16i + lane%16,
     //      n = n0 + wn*WTN + (j/G)*16G + (lane/16)*4G + (j%G)*4 + r : 4G consecutive columns per lane, row and group.
     //      With one wave per SIMD nothing overlaps the epilogue and it is bound by instruction issue (a vector
