@@ -39,34 +39,38 @@ ConfigT = TypeVar("ConfigT")
 
 
 class BaseAdapterModule(nn.Module, Generic[ConfigT], ABC):
-    """Container of named adapters (reference: base.py:57-90).
+    """Named adapters behind one module (the interface of reference base.py:57-90: `make_adapter`, call by name,
+    `named_modules` of the default adapter, which is the first one made).
 
-    Adapters live in a plain dict, not in `_modules`: the reference does the same, so an adapter's
-    parameters are loaded and moved through the adapter object itself.
-    """
+    The adapters are kept in an insertion-ordered dict outside `_modules`, so `state_dict()` / `.to()` of the
+    enclosing model do not see them: weights are loaded into, and moved with, each adapter object on its own, as the
+    reference's loader expects."""
 
     def __init__(self, adapter_cls: Callable[[ConfigT], nn.Module]) -> None:
         super().__init__()
-        self.default_adapter_name: str | None = None
         self.adapter_cls = adapter_cls
         self.adapters: dict[str, nn.Module] = {}
 
+    @property
+    def default_adapter_name(self) -> str | None:
+        return next(iter(self.adapters), None)
+
+    def _adapter(self, name: str | None) -> nn.Module:
+        try:
+            return self.adapters[name]   # type: ignore[index]
+        except KeyError:
+            known = ", ".join(self.adapters) or "none made yet"
+            raise ValueError(f"no adapter named {name!r} (adapters: {known})") from None
+
     def make_adapter(self, name: str, config: ConfigT) -> nn.Module:
-        if self.default_adapter_name is None:
-            self.default_adapter_name = name
-        adapter = self.adapter_cls(config).eval()
-        self.adapters[name] = adapter
-        return adapter
+        self.adapters[name] = self.adapter_cls(config).eval()
+        return self.adapters[name]
 
     def forward(self, name: str, *args: Any, **kwargs: Any):
-        if name not in self.adapters:
-            raise ValueError(f"Adapter '{name}' not found.")
-        return self.adapters[name](*args, **kwargs)
+        return self._adapter(name)(*args, **kwargs)
 
     def named_modules(self, memo: set[nn.Module] | None = None, prefix: str = "", remove_duplicate: bool = True):
-        if self.default_adapter_name is None:
-            raise ValueError("No default adapter name set.")
-        return self.adapters[self.default_adapter_name].named_modules(memo, prefix, remove_duplicate)
+        return self._adapter(self.default_adapter_name).named_modules(memo, prefix, remove_duplicate)
 
 
 class BaseModalityProcessor:
