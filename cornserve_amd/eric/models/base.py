@@ -60,7 +60,7 @@ class BaseAdapterModule(nn.Module, Generic[ConfigT], ABC):
             return self.adapters[name]   # type: ignore[index]
         except KeyError:
             known = ", ".join(self.adapters) or "none made yet"
-            raise ValueError(f"no adapter named {name!r} (adapters: {known})") from None
+            raise ValueError(f"adapter {name!r} not found (adapters: {known})") from None
 
     def make_adapter(self, name: str, config: ConfigT) -> nn.Module:
         self.adapters[name] = self.adapter_cls(config).eval()
