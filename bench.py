@@ -48,7 +48,7 @@ N_IMAGES = 8
 # HBM-side bytes per gate|up call (its two launches together), measured with rocprofv3 --pmc (not live):
 # FETCH_SIZE 93,167 + 18,180 KiB scaled by 2.00 (what the same counter reads for a plain 1 GiB copy) +
 # WRITE_SIZE 49,152 + 6,144 KiB scaled by 1.00.
-GATE_UP_HBM_BYTES_PER_LAUNCH = int(((93167 + 18180) * 2.00 + (49152 + 6144) * 1.00) * 1024)
+GATE_UP_HBM_BYTES_PER_LAUNCH = int(((93147 + 18179) * 2.00 + (49152 + 6144) * 1.00) * 1024)
 GRID = (1, 32, 32)          # 448 x 448, patch 14
 
 
