@@ -267,11 +267,11 @@ def test_full_size_configs_through_properties(dev):
     alone = run([px[5]], [grid[5]])[0]
     assert not torch.equal(out[0], out[1])
     dist = lambda a, b: ((a.float() - b.float()).abs().max() / b.float().abs().max()).item()
-    assert dist(alone, out[5]) <= REL_BF16 / 2, dist(alone, out[5])
+    assert dist(alone, out[5]) <= REL_BF16, dist(alone, out[5])
     model.fuse_window_attn = False
     out_sep = run(px, grid)
     assert torch.equal(alone, out_sep[5]), "an item alone equals the item in the batch"
-    assert dist(torch.cat(out_sep), torch.cat(out)) <= REL_BF16 / 2
+    assert dist(torch.cat(out_sep), torch.cat(out)) <= REL_BF16
     model.fuse_window_attn = True
     # the whole batch against the fp32 oracle on the same bf16-rounded weights and inputs, at the flat bar: the
     # residual stream carries 16 significant bits, so 64 residual additions do not use up the tolerance (the
