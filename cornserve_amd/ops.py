@@ -13,6 +13,7 @@ return nothing; `gemm` also exists in a functional form.  There is no eager-PyTo
 from __future__ import annotations
 
 import ctypes
+import functools
 from dataclasses import dataclass
 
 import numpy as np
@@ -748,7 +749,8 @@ QKV_WATTN_TILE_ROWS = 256    # packed weight rows per head
 QKV_WATTN_WINDOW = 64        # rows of every attention segment
 
 
-def qkv_window_attn_row_order(heads: int) -> torch.Tensor:
+@functools.lru_cache(maxsize=8)
+def _qkv_window_attn_row_order(heads: int) -> torch.Tensor:
     """Row r of the packed [heads*256, K] weight of `qkv_window_attn` is row order[r] of the reference's qkv weight
     [3*heads*80, K] (q | k | v blocks, qwen2_5_vl.py:65-84), or -1 for a zero row.  Per head: tile row
     rho = 32 (J/2) + 8 kq + 4 (J%2) + r for fragment J, lane group kq, element r; q and k fragments (J < 5, J < 10) put
@@ -769,6 +771,12 @@ def qkv_window_attn_row_order(heads: int) -> torch.Tensor:
                 for h in range(heads):
                     order[h, rho] = block * heads * d + h * d + dim
     return order.reshape(-1)
+
+
+def qkv_window_attn_row_order(heads: int) -> torch.Tensor:
+    """Row order of the packed weight of `qkv_window_attn` (see `_qkv_window_attn_row_order`; computed once per head
+    count)."""
+    return _qkv_window_attn_row_order(int(heads)).clone()
 
 
 def pack_qkv_window_attn(w: torch.Tensor, b: torch.Tensor, heads: int) -> tuple[torch.Tensor, torch.Tensor]:
