@@ -335,7 +335,7 @@ class Gemma3VisionEncoder(SiglipEncoderBase):
             assert pixels.ndim == 4
             assert pixels.shape[1] == 3
             assert pixels.shape[2] == pixels.shape[3] == size
-        pixel_values = torch.cat(batch["pixel_values"]).to(device=self.device, dtype=self.dtype)
+        pixel_values = ops.cat_to_device(batch["pixel_values"], self.device, self.dtype)
         num_patches = torch.cat([c.reshape(-1) for c in batch["num_crops"]]).cpu() + 1
         feats = self.vision_tower_forward(pixel_values)
         embeds = self.multi_modal_projector(adapter_name, feats)

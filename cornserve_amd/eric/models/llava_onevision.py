@@ -203,7 +203,7 @@ class LlavaOneVisionEncoder(SiglipEncoderBase):
         strategy = self.config.vision_feature_select_strategy
         if strategy not in ("default", "full"):
             raise ValueError(f"Unexpected select feature strategy: {strategy}")
-        stacked = torch.cat(pixel_values, dim=0).to(device=self.device, dtype=self.dtype)
+        stacked = ops.cat_to_device(pixel_values, self.device, self.dtype)
         feats = self.vision_tower_forward(stacked)            # [tiles, tokens, H]
         if strategy == "default":
             feats = feats[:, 1:].contiguous()

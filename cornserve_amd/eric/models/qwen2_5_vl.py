@@ -241,7 +241,7 @@ class QwenVisionBase(EricModel):
             raise ValueError(f"Unsupported modality: {modality}")
         if frame_key in batch:
             return self.forward_device(*self.patchify_frames(batch[frame_key]))
-        pixel_values = torch.cat(batch[px_key], dim=0).to(device=self.device, dtype=self.dtype)
+        pixel_values = ops.cat_to_device(batch[px_key], self.device, self.dtype)
         grid = torch.cat([g.reshape(-1, 3) for g in batch[grid_key]], dim=0).cpu().numpy().astype(np.int64)
         return self.forward_device(pixel_values, grid)
 

@@ -67,6 +67,25 @@ def host_to_device_packed(arrays: list[np.ndarray], device: torch.device) -> lis
     return out
 
 
+def cat_to_device(tensors: list[torch.Tensor], device: torch.device, dtype: torch.dtype) -> torch.Tensor:
+    """`torch.cat(tensors).to(device, dtype)` (the reference's hand-over, qwen2_5_vl.py:415-419) without its two host
+    passes when the tensors are floating-point HOST tensors: every item is converted to `dtype` straight into its rows
+    of ONE pinned staging buffer (no concatenated fp32 copy; half the bytes cross PCIe when the source is fp32 and the
+    target bf16; the conversion is the same round-to-nearest-even the device cast performs, so the result is
+    bit-identical), followed by one asynchronous copy.  Anything else takes the plain route."""
+    host = all(isinstance(t, torch.Tensor) and t.device.type == "cpu" and t.is_floating_point() and t.dim() >= 1
+               for t in tensors)
+    if not host or device.type != "cuda" or len({t.shape[1:] for t in tensors}) != 1 or sum(t.shape[0] for t in tensors) == 0:
+        return torch.cat(tensors, dim=0).to(device=device, dtype=dtype)
+    rows = sum(t.shape[0] for t in tensors)
+    staged = torch.empty((rows, *tensors[0].shape[1:]), dtype=dtype, pin_memory=True)
+    r = 0
+    for t in tensors:
+        staged[r : r + t.shape[0]].copy_(t)
+        r += t.shape[0]
+    return staged.to(device, non_blocking=True)
+
+
 def _ptr(t: torch.Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 

@@ -838,3 +838,22 @@ def test_llava_onevision_real_tile_size_images_and_video(dev):
     fout = folded(Modality.IMAGE, "", {"pixel_values": px[:2], "image_sizes": szs[:2]})
     for i in range(2):
         check(fout[i], ref[i], REL_BF16, f"llava-onevision 384 image {i}, folded norms")
+
+
+def test_host_tensors_reach_the_device_with_the_device_cast_s_bits(dev):
+    """The hand-over of fp32 host tensors converts on the host straight into pinned staging (one pass, half the PCIe
+    bytes): same bits as concatenating, copying and casting on the device, for contiguous and strided items alike;
+    device tensors and other dtypes take the plain route."""
+    from cornserve_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    items = [torch.randn((n, 1176), generator=g) * s for n, s in ((1024, 1.0), (4, 300.0), (64, 1e-3))]
+    items.append(torch.randn((8, 2352), generator=g)[:, ::2])                       # a strided view
+    items[1][0, :4] = torch.tensor([float("inf"), -0.0, 1e-45, 3.3895e38])           # specials and the rounding edge
+    want = torch.cat(items, dim=0).to(device=dev, dtype=torch.bfloat16)
+    got = ops.cat_to_device(items, dev, torch.bfloat16)
+    assert got.is_cuda and got.dtype == torch.bfloat16 and torch.equal(got.view(torch.int16), want.view(torch.int16))
+    on_dev = [t.to(dev) for t in items]
+    assert torch.equal(ops.cat_to_device(on_dev, dev, torch.bfloat16).view(torch.int16), want.view(torch.int16))
+    halves = [t.half() for t in items[:3]]
+    assert torch.equal(ops.cat_to_device(halves, dev, torch.bfloat16), torch.cat(halves).to(dev, torch.bfloat16))
