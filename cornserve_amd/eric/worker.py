@@ -163,7 +163,10 @@ class Worker:
                 for t in tensors:
                     if (isinstance(t, torch.Tensor) and t.device.type == "cpu" and t.numel() > 0
                             and (t.is_floating_point() or t.dtype == torch.uint8)):
-                        pinned = torch.empty(t.shape, dtype=t.dtype, pin_memory=True)
+                        # floating-point tensors are converted to the model's dtype on the way into the staging buffer
+                        # (the rounding the device cast would apply, on half the bytes); uint8 frames stay bytes
+                        staged_dtype = self.model.dtype if t.is_floating_point() else t.dtype
+                        pinned = torch.empty(t.shape, dtype=staged_dtype, pin_memory=True)
                         pinned.copy_(t)
                         out.append(pinned.to(device, non_blocking=True))
                     else:
