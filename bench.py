@@ -51,6 +51,8 @@ N_IMAGES = 8
 # FETCH_SIZE 93,147 + 18,179 KiB scaled by 2.00 (what the same counter reads for a plain 1 GiB copy) +
 # WRITE_SIZE 49,152 + 6,144 KiB scaled by 1.00.
 GATE_UP_HBM_BYTES_PER_LAUNCH = int(((93147 + 18179) * 2.00 + (49152 + 6144) * 1.00) * 1024)
+GATE_UP_TRAFFIC_SOURCE = ("profiles/qwen2_5_vl_cfg2_bench_kernels_and_traffic.md (rocprofv3 --pmc runs of this script; a "
+                          "constant read from that file, not a live measurement)")
 GRID = (1, 32, 32)          # 448 x 448, patch 14
 
 
@@ -126,6 +128,38 @@ def power_limit_probe(torch, ops, model, L: int, launches: int = 200) -> dict:
     return res
 
 
+def power_limit_probe_step(dev, sd, pixel_values, grid_np, steps: int = 10, warmup: int = 3) -> float:
+    """ms per step of the whole forward with every weight MATRIX (patch embedding, the linear layers of every block
+    and of the merger) zeroed; biases and norm scales stay, so activations are not all zero.  Launches, addresses and
+    memory traffic equal the timed step's; only the switching activity in the multipliers differs."""
+    import torch
+
+    zero_sd = {k: (torch.zeros_like(v) if k.endswith(".weight") and v.dim() >= 2 else v) for k, v in sd.items()}
+    model = _qwen_model(dev, zero_sd)
+    with torch.inference_mode():
+        for _ in range(warmup):
+            model.forward_device(pixel_values, grid_np)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            model.forward_device(pixel_values, grid_np)
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) / steps * 1e3
+    del model
+    torch.cuda.empty_cache()
+    return ms
+
+
+def cpu_model_name() -> str:
+    try:
+        for line in Path("/proc/cpuinfo").read_text().splitlines():
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: list | None = None) -> dict:
     """Time the CPU oracle (bf16, all host threads) on `n_sample_images` of the batch's 8 images, repeating
     the pass until about `min_seconds` of CPU work have been measured.  `gpu_out`: the embeddings of the timed
@@ -135,7 +169,11 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: l
     from cornserve_amd import synth
     from oracle import qwen2_5_vl as oq
 
-    threads = int(os.environ.get("OMP_NUM_THREADS", 0)) or min(os.cpu_count() or 1, 16)
+    # every core this process may run on (a GPU box gives a job a share of the host: the affinity mask or
+    # OMP_NUM_THREADS says how many, os.cpu_count() what the machine has)
+    host_cores = os.cpu_count() or 1
+    usable = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else host_cores
+    threads = min(int(os.environ.get("OMP_NUM_THREADS", 0)) or usable, usable)
     torch.set_num_threads(threads)
     ocfg = oq.QwenVisionConfig()
     px, grid = synth.qwen_inputs([GRID] * n_sample_images, seed=0)
@@ -151,7 +189,8 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: l
         iters += 1
         assert len(out) == n_sample_images
     res = {
-        "value": patches * iters / dt, "unit": "patches/s", "cores": threads, "kind": "port",
+        "value": patches * iters / dt, "unit": "patches/s", "cores": threads, "host_cores": host_cores,
+        "cpu_model": cpu_model_name(), "kind": "port",
         "sample": f"{n_sample_images} of the 8 images ({patches} patches) through the full 32-block encoder, "
                   f"bf16 step-wise CPU oracle, {iters} iteration(s), {dt:.1f} s in total",
     }
@@ -159,9 +198,7 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: l
         # Full-size check (untimed): the GPU embeddings and this bf16 oracle pass, each against the oracle in fp32 on
         # the same bf16-rounded weights and inputs.  At 32 blocks of random-init weights the bf16 oracle itself sits
         # at the edge of the max-error bar, so its distance is printed beside the GPU's.
-        def dist(a, b):
-            return {"cosine": torch.nn.functional.cosine_similarity(a.flatten(), b.flatten(), dim=0).item(),
-                    "max_rel_err": ((a - b).abs().max() / b.abs().max()).item()}
+        from oracle.metrics import distances as dist
 
         sd32 = {k: v.float() for k, v in sd16.items()}
         px32 = [p.to(torch.bfloat16).float() for p in px]
@@ -252,7 +289,118 @@ def hbm_kernels(dev, rows_list=(8192, 131072), reps: int = 20) -> dict:
             "kernels": out}
 
 
-OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl", "llava_ov", "hbm_kernels")
+
+def _qwen_model(dev, sd, weight_format="bf16", **kw):
+    import torch
+
+    from cornserve_amd import synth
+    from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
+
+    model = Qwen2_5_VisionTransformer(synth.qwen_vision_config(), weight_format=weight_format, **kw)
+    model.load_state_dict(sd, strict=False)
+    return model.to(device=dev, dtype=torch.bfloat16).eval()
+
+
+def parity_cfg2(dev, seed: int = 0, n_images: int = N_IMAGES) -> dict:
+    """configs[1] at its full depth against the CPU oracle, three ways: the default kernels, the kernels restricted to
+    the reference's own rounding points (norms as kernels, bf16 residual stream, separate QKV / rotary / attention
+    launches), and the bf16 step-wise oracle evaluated in a second summation order -- each against the fp32 oracle
+    and against the bf16 step-wise oracle on the same bf16-rounded weights and inputs."""
+    import numpy as np
+    import torch
+
+    from cornserve_amd import synth
+    from oracle import qwen2_5_vl as oq
+    from oracle.metrics import distances
+
+    sd = synth.qwen_state_dict(synth.qwen_vision_config(), seed=seed)
+    px, grid = synth.qwen_inputs([GRID] * n_images, seed=seed)
+    sd16 = {k: v.bfloat16() for k, v in sd.items()}
+    sd32 = {k: v.float() for k, v in sd16.items()}
+    px16 = [p.bfloat16() for p in px]
+    g = torch.cat(grid).numpy().astype(np.int64)
+    pv = torch.cat(px16).to(dev)
+    ocfg = oq.QwenVisionConfig()
+    with torch.inference_mode():
+        model = _qwen_model(dev, sd)
+        got = torch.cat(model.forward_device(pv, g)).float().cpu()
+        del model
+        model = _qwen_model(dev, sd, fold_norm=False, split_residual=False, fuse_window_attn=False)
+        got_ref_rounding = torch.cat(model.forward_device(pv, g)).float().cpu()
+        del model
+    torch.cuda.empty_cache()
+    ref32 = torch.cat(oq.forward(sd32, ocfg, [p.float() for p in px16], grid, dtype=torch.float32))
+    ref16 = torch.cat(oq.forward(sd16, ocfg, px16, grid, dtype=torch.bfloat16)).float()
+    ref16b = torch.cat(oq.forward(sd16, ocfg, px16, grid, dtype=torch.bfloat16, linear_mode="fp32_accumulate")).float()
+    return {
+        "what": f"configs[1], {n_images} images of 448x448, 32 blocks, seed {seed}",
+        "gpu_default_vs_fp32_oracle": distances(got, ref32),
+        "gpu_default_vs_bf16_oracle": distances(got, ref16),
+        "gpu_reference_rounding_vs_fp32_oracle": distances(got_ref_rounding, ref32),
+        "gpu_reference_rounding_vs_bf16_oracle": distances(got_ref_rounding, ref16),
+        "bf16_oracle_vs_fp32_oracle": distances(ref16, ref32),
+        "bf16_oracle_second_summation_order_vs_fp32_oracle": distances(ref16b, ref32),
+        "bf16_oracle_vs_bf16_oracle_second_summation_order": distances(ref16, ref16b),
+    }
+
+
+def parity_cfg4(dev, seed: int = 22, items=(12, 0)) -> dict:
+    """configs[3] (16 ragged images, every one with partial windows at its edges) at full depth: the embeddings of
+    `items` (by default the smallest image and a mid-size one), taken from the forward of the WHOLE batch, against the
+    fp32 oracle run on those items alone (items are independent)."""
+    import numpy as np
+    import torch
+
+    from cornserve_amd import synth
+    from oracle import qwen2_5_vl as oq
+    from oracle.metrics import distances
+
+    sd = synth.qwen_state_dict(synth.qwen_vision_config(), seed=seed)
+    grids = synth.ragged_grids(16, seed=4)
+    px, grid = synth.qwen_inputs(grids, seed=seed)
+    px16 = [p.bfloat16() for p in px]
+    with torch.inference_mode():
+        model = _qwen_model(dev, sd)
+        out = model.forward_device(torch.cat(px16).to(dev), torch.cat(grid).numpy().astype(np.int64))
+        got = {i: out[i].float().cpu() for i in items}
+        del model, out
+    torch.cuda.empty_cache()
+    sd32 = {k: v.bfloat16().float() for k, v in sd.items()}
+    res = {"what": f"configs[3], 16 ragged images = {sum(h * w for _, h, w in grids)} patches, 32 blocks, seed {seed}"}
+    for i in items:
+        ref = oq.forward(sd32, oq.QwenVisionConfig(), [px16[i].float()], [grid[i]], dtype=torch.float32)[0]
+        res[f"item_{i}_grid_{grids[i][1]}x{grids[i][2]}_vs_fp32_oracle"] = distances(got[i], ref)
+    return res
+
+
+def parity_cfg5(dev, seed: int = 23) -> dict:
+    """configs[4] (fp8-e4m3 weights, two clips of 8 x 24 x 42 patches) at full depth: the first clip's embeddings,
+    taken from the forward of both clips, against the fp32 oracle on the de-quantised weights."""
+    import numpy as np
+    import torch
+
+    from cornserve_amd import synth
+    from oracle import qwen2_5_vl as oq
+    from oracle.metrics import distances
+
+    cfg = synth.qwen_vision_config()
+    sd = synth.qwen_state_dict(cfg, seed=seed)
+    px, grid = synth.qwen_inputs([(8, 24, 42)] * 2, seed=seed)
+    px16 = [p.bfloat16() for p in px]
+    with torch.inference_mode():
+        model = _qwen_model(dev, sd, weight_format="fp8_e4m3")
+        out = model.forward_device(torch.cat(px16).to(dev), torch.cat(grid).numpy().astype(np.int64))
+        got = out[0].float().cpu()
+        del model, out
+    torch.cuda.empty_cache()
+    # the model quantises the bf16 weights it was loaded with
+    sd_dq = oq.dequantized_state_dict({k: v.bfloat16().float() for k, v in sd.items()}, synth.qwen_linear_weight_keys(cfg))
+    ref = oq.forward(sd_dq, oq.QwenVisionConfig(), [px16[0].float()], [grid[0]], dtype=torch.float32)[0]
+    return {"what": f"configs[4], fp8-e4m3 weights, clip 0 of 2 (8064 patches), 32 blocks, seed {seed}",
+            "gpu_fp8_vs_dequantised_fp32_oracle": distances(got, ref)}
+
+
+OTHER_WORKLOADS = ("cfg3", "cfg4", "cfg5", "qwen2_vl", "qwen3_vl", "llava_ov", "hbm_kernels", "parity")
 
 
 def other_workload(name: str, steps: int, warmup: int, dev) -> dict:
@@ -368,6 +516,11 @@ def main() -> None:
     dev = torch.device("cuda:0")
     if args.workload == "hbm_kernels":
         print(json.dumps(hbm_kernels(dev)))
+        return
+    if args.workload == "parity":
+        print(json.dumps({"metric": "full-depth parity of the Qwen2.5-VL encoder against the CPU oracle", "n_gpus": 1,
+                          "bar": "cosine >= 0.999 and max |err| / max |ref| <= 2e-2 (5e-2 with fp8 weights)",
+                          "cfg2": parity_cfg2(dev), "cfg4": parity_cfg4(dev), "cfg5": parity_cfg5(dev)}))
         return
     if args.workload != "cfg2":
         print(json.dumps(other_workload(args.workload, args.steps, args.warmup, dev)))
@@ -491,6 +644,18 @@ def main() -> None:
         torch.cuda.synchronize()
         one_ms = (time.perf_counter() - t0) / 10 * 1e3
         probe = power_limit_probe(torch, ops, model, L) if model.fold_norm and not args.no_power_probe else None
+        # the timed step again, right next to the same step on zeroed weight matrices
+        step_zero_ms = step_again_ms = None
+        if not args.no_power_probe:
+            step_zero_ms = power_limit_probe_step(dev, sd, pixel_values, grid_np)
+            for _ in range(3):
+                model.forward_device(pixel_values, grid_np)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(10):
+                model.forward_device(pixel_values, grid_np)
+            torch.cuda.synchronize()
+            step_again_ms = (time.perf_counter() - t0) / 10 * 1e3
     stage_ms = {k: sum(v) / 3 for k, v in full.durations_ms().items()}
     mfma_keys = [k for k in stage_ms if k.startswith("gemm_") or k.startswith("attn_") or k == "patch_embed"]
     # The instrumented pass records an event between stages, which costs a little device time per mark: its
@@ -523,7 +688,8 @@ def main() -> None:
                                        "back to back by one cs_gemm call (8192x6912x1280 launched, 8192x6840x1280 algorithmic)",
             "achieved": achieved, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
             "avg_launch_ms": gu_ms, "launches_timed": len(gu), "traffic": GATE_UP_HBM_BYTES_PER_LAUNCH,
-            "traffic_unit": "bytes per call, both launches (rocprofv3 FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00, see profiles/)",
+            "traffic_unit": "bytes per call, both launches (rocprofv3 FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00)",
+            "traffic_source": GATE_UP_TRAFFIC_SOURCE,
         },
         "breakdown": {
             "stage_ms_per_step": {k: round(v, 4) for k, v in sorted(stage_ms.items())},
@@ -534,6 +700,17 @@ def main() -> None:
             "mfma_frac_over_whole_step": flops["total"] / (ms_per_step * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         },
     }
+    if step_zero_ms is not None:
+        target_ms = flops["total"] / (0.5 * PEAK_BF16_TFLOPS * 1e12) * 1e3
+        result["breakdown"]["power_limit_probe_step"] = {
+            "zero_weight_matrices_ms_per_step": step_zero_ms, "random_weights_ms_per_step": step_again_ms,
+            "ms_per_step_at_half_of_peak": target_ms,
+            "mfma_frac_whole_step_zero_weight_matrices": flops["total"] / (step_zero_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+            "note": "the whole forward, 10 steps each, back to back outside the timed region: with the model's weights and "
+                    "with every weight matrix zeroed (same launches, addresses and traffic; biases and norm scales "
+                    "kept).  The zero-weight figure is what this schedule reaches when the multipliers draw no "
+                    "switching power",
+        }
     if probe is not None:
         result["roofline"]["power_limit_probe"] = {
             "random_weights_ms": probe["random"], "zero_weights_ms": probe["zero_weights"],

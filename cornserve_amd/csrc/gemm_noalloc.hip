@@ -44,9 +44,24 @@ extern "C" int cs_gemm_rmsnorm_noalloc(const CsGemmArgs* args, void* stream) {
   // The library supplies the row sums: the caller must not, and A must be a plain matrix whose K columns are the
   // normalised width (no row gather: the sums are taken over A's own rows 0..M-1).
   if (args->a_row_sumsq || args->a_row_sum || args->a_rows || args->w_fp8) return CS_ERR_INVALID_ARG;
-  if (args->M < 0 || args->K <= 0) return CS_ERR_INVALID_ARG;
+  if (args->M < 0 || args->K <= 0 || args->N <= 0) return CS_ERR_INVALID_ARG;
   if (args->M > CS_NOALLOC_MAX_ROWS) return CS_ERR_TOO_LARGE;
   if (args->K > 160 * CS_SUMSQ_PARTS) return CS_ERR_TOO_LARGE;
+  // Everything cs_gemm would refuse for a folded-norm launch is refused HERE, before the row-sums launch is
+  // enqueued: the folded form exists in the direct-to-LDS kernel only (K a multiple of 64 and at least 192, N a
+  // multiple of 8, 16-byte aligned rows of C), with the plain-bias and the SiLU-gate epilogues, and without the
+  // position addend or output row sums.
+  if (!args->A || !args->W || !args->C) return CS_ERR_INVALID_ARG;
+  if (args->K % 64 || args->K < 192) return CS_ERR_UNSUPPORTED;
+  if (args->epilogue != CS_EPI_BIAS && args->epilogue != CS_EPI_SWIGLU) return CS_ERR_UNSUPPORTED;
+  if (args->pos || args->c_row_sumsq || args->c_row_sum || args->w_col_sum || args->w_scale || args->conv_patch ||
+      args->c_lo || args->residual_lo)
+    return CS_ERR_UNSUPPORTED;
+  if (args->N < 8 || args->N % 8 || args->ldc % 8 || args->lda % 8 || args->ldw % 8) return CS_ERR_UNSUPPORTED;
+  if ((((uintptr_t)args->A | (uintptr_t)args->W | (uintptr_t)args->C) & 15) || ((uintptr_t)args->bias & 7))
+    return CS_ERR_INVALID_ARG;
+  if ((int64_t)args->M * args->lda * 2 >= (int64_t)UINT32_MAX || (int64_t)args->N * args->ldw * 2 >= (int64_t)UINT32_MAX)
+    return CS_ERR_UNSUPPORTED;
   int st = CS_OK;
   float* sums = scratch_on_current_device(&st);
   if (!sums) return st;

@@ -139,7 +139,9 @@ class Scheduler:
             self._slot_of[(request.request_id, item.id)] = slot
 
     def has_waiting_requests(self) -> bool:
-        """Requests that are not finished yet (waiting or in flight), as the reference's method counts them."""
+        """Requests that are not finished yet (waiting or in flight), as the reference's method counts them.  A loop that
+        calls `schedule()` again before `process_batch_result()` (upload-ahead) must gate on `has_schedulable_items()`
+        instead: with every item in flight this stays True and `schedule()` has nothing to return (it raises)."""
         return bool(self._open)
 
     def has_schedulable_items(self) -> bool:
@@ -176,11 +178,16 @@ class Scheduler:
         """Report items as done.  Returns the requests whose last item this was, in the order given."""
         if len(request_ids) != len(data_ids):
             raise ValueError("request_ids and data_ids must have one entry per item")
-        finished: list[str] = []
-        for key in zip(request_ids, data_ids):
-            slot = self._slot_of.pop(key, None)
-            if slot is None:
+        # every pair is checked before any state changes: a bad pair leaves the bookkeeping as it was
+        keys = list(zip(request_ids, data_ids))
+        if len(set(keys)) != len(keys):
+            raise KeyError("an item is reported twice in one call")
+        for key in keys:
+            if key not in self._slot_of:
                 raise KeyError(f"item {key[1]} of request {key[0]} is not queued (reported twice?)")
+        finished: list[str] = []
+        for key in keys:
+            slot = self._slot_of.pop(key)
             slot.state = None                          # finished: dropped from the line below
             self._open[key[0]] -= 1
             if self._open[key[0]] == 0:

@@ -85,35 +85,53 @@ class Download:
 
     def __init__(self, host: list[torch.Tensor], done: "torch.cuda.Event") -> None:
         self._host, self._done = host, done
+        self._consumed = False
 
     def ready(self) -> bool:
         return self._done.query()
 
     def wait(self) -> list[torch.Tensor]:
-        """Block until the copies have landed; the host tensors (views of one pinned buffer) stay valid until the
-        second `Worker.download` call after the one that returned this object."""
+        """Block until the copies have landed and return the host tensors.  They are views of one pinned buffer of the
+        worker's ring and stay valid until that buffer's turn comes again, i.e. for `download_slots` - 1 further
+        `Worker.download` calls (one, with the default two buffers); a consumer that keeps them longer must copy
+        them, or the worker must be built with a deeper ring.  Waiting marks the buffer as handed over: a download that
+        is neither waited on nor released blocks the reuse of its buffer (`Worker.download` raises)."""
         self._done.synchronize()
+        self._consumed = True
         return self._host
+
+    def release(self) -> None:
+        """Give the buffer back without reading it (the copy, if still running, is waited for first)."""
+        self._done.synchronize()
+        self._consumed = True
+        self._host = []
 
 
 class Worker:
     """Runs batches through one encoder and forwards the embeddings (reference: Worker.execute_model)."""
 
-    def __init__(self, model, sender_sidecar_client=None) -> None:
+    def __init__(self, model, sender_sidecar_client=None, download_slots: int = 2) -> None:
+        """`download_slots`: depth of the ring of pinned host buffers `download` cycles through (at least 2: one being
+        filled while the previous one is read)."""
+        if download_slots < 2:
+            raise ValueError("download_slots must be at least 2")
         self.model = model
         if sender_sidecar_client is None and mock_sidecar_enabled():
             sender_sidecar_client = MockSidecar()
         self.sender_sidecar_client = sender_sidecar_client
         self._copy_stream: torch.cuda.Stream | None = None
         self._d2h_stream: torch.cuda.Stream | None = None
-        self._d2h_slots: list[torch.Tensor | None] = [None, None]   # two pinned buffers, used alternately
+        self._d2h_slots: list[torch.Tensor | None] = [None] * download_slots   # pinned buffers, used in turn
+        self._d2h_owner: list[Download | None] = [None] * download_slots       # the download each one was last lent to
         self._d2h_turn = 0
 
     def download(self, embeddings: list[torch.Tensor]) -> Download:
         """Start copying a batch's embeddings to pinned host memory on a side stream (default priority) and return at
         once: the copy waits for the kernels that produce the embeddings (an event on the compute stream) and runs
-        while the next batch computes.  Two pinned buffers are used alternately and grown on demand, so the steady
-        state allocates nothing."""
+        while the next batch computes.  The pinned buffers of the ring are used in turn and grown on demand, so the
+        steady state allocates nothing.  A buffer is only lent again once the download it was last lent to has been
+        waited on or released; otherwise the consumer would read the next batch's bytes in the previous batch's views
+        without any error, so this raises RuntimeError instead (wait on downloads in order, or deepen the ring)."""
         device = self.model.device
         if device.type != "cuda":
             raise RuntimeError("download needs the model on a GPU")
@@ -125,7 +143,11 @@ class Worker:
         sizes = [(e.numel() * e.element_size() + 255) // 256 * 256 for e in embeddings]
         total = max(sum(sizes), 256)
         turn = self._d2h_turn
-        self._d2h_turn ^= 1
+        owner = self._d2h_owner[turn]
+        if owner is not None and not owner._consumed:
+            raise RuntimeError(f"download ring overrun: the download started {len(self._d2h_slots)} calls ago has been "
+                               "neither waited on nor released, and its pinned buffer is due for reuse")
+        self._d2h_turn = (turn + 1) % len(self._d2h_slots)
         slot = self._d2h_slots[turn]
         if slot is None or slot.numel() < total:
             slot = self._d2h_slots[turn] = torch.empty((total,), dtype=torch.uint8, pin_memory=True)
@@ -143,7 +165,8 @@ class Worker:
                 offset += size
             done = torch.cuda.Event()
             done.record(self._d2h_stream)
-        return Download(host, done)
+        started = self._d2h_owner[turn] = Download(host, done)
+        return started
 
     def upload(self, batch: WorkerBatch) -> WorkerBatch:
         """Start copying the batch's host tensors to the model's device and return at once.  Every host tensor is

@@ -138,9 +138,16 @@ int cs_gemm(const CsGemmArgs* args, void* stream);
  * allocate device memory -- code under HIP graph capture, serving loops and harnesses that forbid hipMalloc.  It
  * allocates and frees nothing.  args as for cs_gemm, with a_row_sumsq, a_row_sum and a_rows NULL and bf16 W; K is the
  * normalised width (<= 160 * CS_SUMSQ_PARTS); norm_eps as for cs_gemm.  M above CS_NOALLOC_MAX_ROWS (or K above that
- * width) returns CS_ERR_TOO_LARGE.  Every GPU the library is used on holds the array (CS_NOALLOC_MAX_ROWS *
- * CS_SUMSQ_PARTS floats = 2 MiB) until the process ends; all calls on one GPU share it, so calls that overlap on one
- * GPU (different streams, or threads) race -- serialise them on one stream.                                          */
+ * width) returns CS_ERR_TOO_LARGE.  The folded form exists for K a multiple of 64 and at least 192, N a multiple of
+ * 8, ldc a multiple of 8 with C 16-byte aligned, the epilogues CS_EPI_BIAS and CS_EPI_SWIGLU, and none of pos,
+ * c_row_sumsq, c_row_sum, w_col_sum, w_scale, conv_patch, c_lo, residual_lo; anything else returns
+ * CS_ERR_UNSUPPORTED (or CS_ERR_INVALID_ARG) BEFORE any kernel is enqueued.  Every GPU the library is used on holds
+ * the array (CS_NOALLOC_MAX_ROWS * CS_SUMSQ_PARTS floats = 2 MiB) until the process ends; all calls on one GPU share
+ * it, so calls that overlap on one GPU (different streams, or threads) race -- serialise them on one stream.
+ * Under HIP graph capture: the first call on a device looks the array's address up (hipGetSymbolAddress) and the
+ * first launch of every kernel form (tile shape x epilogue) sets that kernel's dynamic-LDS attribute
+ * (hipFuncSetAttribute); neither is a stream operation, so make one call per shape and epilogue on each device
+ * BEFORE capture begins -- later calls issue kernel launches only.                                                   */
 #define CS_NOALLOC_MAX_ROWS 65536
 int cs_gemm_rmsnorm_noalloc(const CsGemmArgs* args, void* stream);
 

@@ -94,10 +94,22 @@ def rot_pos_emb(cfg: QwenVisionConfig, grid_thw) -> torch.Tensor:
 
 
 def forward(sd: dict, cfg: QwenVisionConfig, pixel_values: list, grid_thw: list, dtype=torch.float32,
-            collect: dict | None = None) -> list:
+            collect: dict | None = None, linear_mode: str = "native") -> list:
     """sd: state dict with the checkpoint's names (after `visual.` is stripped), any float dtype.
-    pixel_values: list of [L_i, 1176]; grid_thw: list of [1,3] (or [3]) integer arrays."""
+    pixel_values: list of [L_i, 1176]; grid_thw: list of [1,3] (or [3]) integer arrays.
+
+    `linear_mode`: "native" runs every linear layer as F.linear in `dtype`; "fp32_accumulate" (meaningful for
+    bf16) computes it on fp32 copies of the same bf16 operands and rounds the result to `dtype` once -- the same
+    definition (fp32 accumulation, one rounding, as the reference's GEMM library does), evaluated in a different
+    summation order.  The distance between the two is what the order of accumulation alone is worth."""
     W = {k: v.to(dtype) for k, v in sd.items()}
+    if linear_mode == "native":
+        linear = F.linear
+    elif linear_mode == "fp32_accumulate":
+        def linear(a, w, b=None):
+            return F.linear(a.float(), w.float(), None if b is None else b.float()).to(a.dtype)
+    else:
+        raise ValueError(f"unknown linear_mode {linear_mode}")
     H, nh = cfg.hidden_size, cfg.num_heads
     d = H // nh
     unit = cfg.spatial_merge_size**2
@@ -124,23 +136,23 @@ def forward(sd: dict, cfg: QwenVisionConfig, pixel_values: list, grid_thw: list,
         cu = cu_full if i in cfg.fullatt_block_indexes else cu_window
         p = f"blocks.{i}."
         n1 = rms_norm(x, W[p + "norm1.weight"], cfg.rms_norm_eps)
-        qkv = F.linear(n1, W[p + "attn.qkv.weight"], W[p + "attn.qkv.bias"])
+        qkv = linear(n1, W[p + "attn.qkv.weight"], W[p + "attn.qkv.bias"])
         q, k, v = (t.reshape(L, nh, d) for t in qkv.chunk(3, dim=-1))
         q = apply_rotary(q, rotary)
         k = apply_rotary(k, rotary)
         o = varlen_attention(q, k, v, cu, d**-0.5).reshape(L, H)
-        x = x + F.linear(o, W[p + "attn.proj.weight"], W[p + "attn.proj.bias"])
+        x = x + linear(o, W[p + "attn.proj.weight"], W[p + "attn.proj.bias"])
         n2 = rms_norm(x, W[p + "norm2.weight"], cfg.rms_norm_eps)
-        g = F.silu(F.linear(n2, W[p + "mlp.gate_proj.weight"], W[p + "mlp.gate_proj.bias"]))
-        u = F.linear(n2, W[p + "mlp.up_proj.weight"], W[p + "mlp.up_proj.bias"])
-        x = x + F.linear(g * u, W[p + "mlp.down_proj.weight"], W[p + "mlp.down_proj.bias"])
+        g = F.silu(linear(n2, W[p + "mlp.gate_proj.weight"], W[p + "mlp.gate_proj.bias"]))
+        u = linear(n2, W[p + "mlp.up_proj.weight"], W[p + "mlp.up_proj.bias"])
+        x = x + linear(g * u, W[p + "mlp.down_proj.weight"], W[p + "mlp.down_proj.bias"])
         if collect is not None:
             collect[f"block{i}"] = x.clone()
 
     x = rms_norm(x, W["merger.ln_q.weight"], cfg.rms_norm_eps).view(-1, H * unit)
-    x = F.linear(x, W["merger.mlp.0.weight"], W["merger.mlp.0.bias"])
+    x = linear(x, W["merger.mlp.0.weight"], W["merger.mlp.0.bias"])
     x = F.gelu(x)
-    x = F.linear(x, W["merger.mlp.2.weight"], W["merger.mlp.2.bias"])
+    x = linear(x, W["merger.mlp.2.weight"], W["merger.mlp.2.bias"])
     x = x[torch.argsort(wi)]
     seqlens = (grid[:, 0] * grid[:, 1] * grid[:, 2]) // unit
     return list(x.split([int(s) for s in seqlens], dim=0))

@@ -65,6 +65,18 @@ def test_invalid_arguments_are_rejected_without_a_gpu():
     assert l.cs_rmsnorm(None, 0, None, None, 0, 1, 8, 1e-6, 0, None) == lib.CS_ERR_INVALID_ARG
     assert l.cs_attn_varlen(None, None, None, 0, None, 0, None, 0, 16, 80, 0.1, None, 64, None) == lib.CS_ERR_INVALID_ARG
     assert l.cs_rope_qk(None, 0, None, 0, 16, 80, None) == lib.CS_ERR_INVALID_ARG
+    # the entry point that allocates nothing refuses what its folded-norm GEMM cannot take before it touches the GPU
+    # (fake, suitably aligned addresses: nothing is dereferenced on the way to the refusal)
+    na = lib.CsGemmArgs()
+    na.A, na.W, na.C = 0x1000, 0x2000, 0x3000
+    na.lda = na.ldw = 1280
+    na.ldc = na.N = 3840
+    na.M, na.K, na.epilogue = 256, 1240, lib.EPI_BIAS
+    assert l.cs_gemm_rmsnorm_noalloc(ctypes.byref(na), None) == lib.CS_ERR_UNSUPPORTED      # K not a multiple of 64
+    na.K, na.epilogue = 1280, lib.EPI_RESIDUAL
+    assert l.cs_gemm_rmsnorm_noalloc(ctypes.byref(na), None) == lib.CS_ERR_UNSUPPORTED      # no folded form of it
+    na.epilogue, na.M = lib.EPI_BIAS, 65537
+    assert l.cs_gemm_rmsnorm_noalloc(ctypes.byref(na), None) == lib.CS_ERR_TOO_LARGE
     g = np.array([[1, 3, 4]], np.int64)  # odd height cannot be merged 2x2
     with pytest.raises(ValueError):
         ops.vit_seqlens_host(g, 2, 4)

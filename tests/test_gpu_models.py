@@ -310,6 +310,54 @@ def test_full_size_configs_through_properties(dev):
     assert torch.equal(twice[0], twice[1]) and torch.equal(twice[0], out[1]), "equal clips give equal embeddings"
 
 
+def _holds_bar(d: dict, rel: float, what: str):
+    assert d["cosine"] >= COS_MIN and d["max_rel_err"] <= rel, (what, d)
+    assert d["min_row_cosine"] >= COS_MIN - 1e-3, (what, d)
+
+
+def test_full_depth_config2_default_and_reference_rounding_against_both_oracles(dev):
+    """Config 2 at 32 blocks, all 8 images.  The bar (cosine >= 0.999, max |err| / max |ref| <= 2e-2) is held against the
+    fp32 oracle.  Against the bf16 step-wise oracle -- the reference's arithmetic -- two bf16 evaluations of the same
+    network cannot be expected inside 2e-2 of each other at this depth: the bf16 oracle itself sits about 2.3e-2 from
+    fp32, and so do this build's kernels when restricted to the reference's rounding points (norms as kernels, bf16
+    residual stream, separate QKV / rotary / attention launches).  What is asserted against it: the cosine bar, and that
+    the GPU is no further from the bf16 oracle than that oracle is from fp32 (plus a margin of 0.5e-2)."""
+    import bench
+
+    d = bench.parity_cfg2(dev, seed=21)
+    print(d)
+    _holds_bar(d["gpu_default_vs_fp32_oracle"], REL_BF16, "default kernels vs fp32 oracle")
+    noise = d["bf16_oracle_vs_fp32_oracle"]["max_rel_err"]
+    for key in ("gpu_default_vs_bf16_oracle", "gpu_reference_rounding_vs_bf16_oracle", "gpu_reference_rounding_vs_fp32_oracle"):
+        assert d[key]["cosine"] >= COS_MIN and d[key]["min_row_cosine"] >= COS_MIN - 1e-3, (key, d[key])
+        assert d[key]["max_rel_err"] <= noise + 0.5e-2, (key, d[key], noise)
+    # the summation order of the linear layers alone moves the bf16 oracle by about as much as it is from fp32
+    assert d["bf16_oracle_vs_bf16_oracle_second_summation_order"]["cosine"] >= COS_MIN
+
+
+def test_full_depth_config4_ragged_images_against_fp32_oracle(dev):
+    """Config 4 (16 ragged images; every one has partial windows at its edges) at 32 blocks: the smallest image and a
+    mid-size one, taken from the forward of the whole batch, against the fp32 oracle at the bf16 bar."""
+    import bench
+
+    d = bench.parity_cfg4(dev)
+    print(d)
+    items = [k for k in d if k.startswith("item_")]
+    assert len(items) == 2
+    for k in items:
+        _holds_bar(d[k], REL_BF16, k)
+
+
+def test_full_depth_config5_fp8_weights_against_dequantised_fp32_oracle(dev):
+    """Config 5 (fp8-e4m3 weights, 2 clips of 8 x 24 x 42 patches) at 32 blocks: one whole clip (8064 patches) against
+    the fp32 oracle on the de-quantised weights at the fp8 bar (5e-2)."""
+    import bench
+
+    d = bench.parity_cfg5(dev)
+    print(d)
+    _holds_bar(d["gpu_fp8_vs_dequantised_fp32_oracle"], REL_FP8, "fp8 weights, full depth")
+
+
 def test_scheduler_upload_ahead_pipeline(dev):
     """The pipelined loop: batch k+1 is taken from the scheduler and its host tensors sent ahead on the side stream
     while batch k is still queued on the device; the upload event survives `to_worker_batch`, and every embedding
@@ -406,6 +454,17 @@ def test_worker_download_overlaps_and_matches(dev):
     assert results == [True] * len(sets)
     with pytest.raises(ValueError):
         worker.download([torch.zeros(3)])
+    # a buffer of the ring is not lent again while the download it was lent to is unread: two downloads nobody waited
+    # on, and the third call refuses instead of overwriting the first one's host views; a deeper ring takes three
+    a, b = worker.download(out), worker.download(out)
+    with pytest.raises(RuntimeError, match="overrun"):
+        worker.download(out)
+    a.release()
+    c = worker.download(out)
+    assert all(torch.equal(h, o.cpu()) for h, o in zip(c.wait(), out)) and all(torch.equal(h, o.cpu()) for h, o in zip(b.wait(), out))
+    deep = Worker(model, download_slots=3)
+    three = [deep.download(out) for _ in range(3)]
+    assert all(torch.equal(h, o.cpu()) for d in three for h, o in zip(d.wait(), out))
 
 
 def test_worker_hand_off_of_real_embeddings(dev, tmp_path):

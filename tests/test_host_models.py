@@ -427,6 +427,11 @@ def test_scheduler_batches_like_the_reference_and_bounds_patches():
     assert s.process_batch_result(b0.request_ids, b0.data_ids) == ["r0"]
     with pytest.raises(KeyError):
         s.process_batch_result(["r0"], ["d0"])                             # reported twice
+    with pytest.raises(KeyError):
+        s.process_batch_result(["r1", "r1"], ["d4", "nope"])               # a bad pair behind a good one ...
+    with pytest.raises(KeyError):
+        s.process_batch_result(["r1", "r1"], ["d4", "d4"])
+    assert s.has_waiting_requests()                                        # ... leaves d4 queued: nothing was changed
     assert s.process_batch_result(["r1", "r1"], ["d4", "d3"]) == ["r1"] and not s.has_waiting_requests()
     with pytest.raises(ValueError):
         s.enqueue(sc.EngineEnqueueRequest("r5", []))

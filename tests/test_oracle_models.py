@@ -327,3 +327,41 @@ def test_llava_onevision_merge_special_cases():
     assert torch.equal(out[25:].view(kept, 21, 8)[:, 20], nl.expand(kept, 8))
     with pytest.raises(ValueError, match="not consistent"):
         ol.merge_image(ocfg, torch.randn(2, 24, 8), (70, 70), nl)
+
+
+def test_distance_measures_known_answers():
+    """oracle.metrics.distances on cases with closed-form answers (a wrong normaliser, a missed row or an fp32
+    reduction would fail one of them)."""
+    from oracle.metrics import distances
+
+    ref = torch.tensor([[3.0, 4.0], [0.0, 2.0], [1.0, 0.0]])
+    d = distances(ref.clone(), ref)
+    assert d == {"cosine": 1.0, "max_rel_err": 0.0, "min_row_cosine": 1.0, "max_row_rel_l2": 0.0}
+    got = ref.clone()
+    got[1] = torch.tensor([2.0, 0.0])                    # one row rotated by 90 degrees, same norm
+    d = distances(got, ref)
+    assert abs(d["min_row_cosine"]) < 1e-15 and abs(d["max_row_rel_l2"] - 2**0.5) < 1e-12
+    assert abs(d["max_rel_err"] - 2.0 / 4.0) < 1e-15     # |err| max 2 against the largest reference magnitude 4
+    assert abs(d["cosine"] - 26.0 / 30.0) < 1e-12        # (25 + 0 + 1) / (sqrt(30) sqrt(30))
+    big = torch.full((4000, 2000), 1.0 + 2.0**-12)       # an fp32 dot product of 8M equal terms drifts above 1
+    c = distances(big, big)["cosine"]
+    assert c <= 1.0 and 1.0 - c < 1e-12
+    with pytest.raises(ValueError):
+        distances(ref, ref[:2])
+
+
+def test_oracle_linear_in_a_second_summation_order():
+    """`linear_mode="fp32_accumulate"` is the same network: identical in fp32, and in bf16 within the rounding noise of
+    one shallow pass (the two modes differ in the order of the fp32 accumulation only)."""
+    cfg = synth.qwen_vision_config(depth=2, fullatt_block_indexes=(1,))
+    sd = synth.qwen_state_dict(cfg, seed=3)
+    ocfg = oq.QwenVisionConfig(depth=2, fullatt_block_indexes=[1])
+    px, grid = synth.qwen_inputs([(1, 8, 12)], seed=3)
+    a = oq.forward(sd, ocfg, px, grid, dtype=torch.float32)[0]
+    b = oq.forward(sd, ocfg, px, grid, dtype=torch.float32, linear_mode="fp32_accumulate")[0]
+    assert torch.equal(a, b)
+    a16 = oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)[0].float()
+    b16 = oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16, linear_mode="fp32_accumulate")[0].float()
+    assert (a16 - b16).abs().max() <= 1e-2 * a.abs().max() and (b16 - a).abs().max() <= 1e-2 * a.abs().max()
+    with pytest.raises(ValueError):
+        oq.forward(sd, ocfg, px, grid, linear_mode="other")

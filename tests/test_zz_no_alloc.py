@@ -71,4 +71,13 @@ def test_no_alloc_entry_point_equals_the_workspace_form():
     assert dll.cs_gemm_rmsnorm_noalloc(ctypes.byref(wide), stream) == lib.CS_ERR_TOO_LARGE
     own = _args(lib, a, w, b, got, lib.EPI_BIAS, 1e-6, sums)
     assert dll.cs_gemm_rmsnorm_noalloc(ctypes.byref(own), stream) == lib.CS_ERR_INVALID_ARG
+    # shapes and epilogues the folded form does not exist for are refused before anything is enqueued
+    odd_k = _args(lib, a, w, b, got, lib.EPI_BIAS, 1e-6)
+    odd_k.K = 296
+    assert dll.cs_gemm_rmsnorm_noalloc(ctypes.byref(odd_k), stream) == lib.CS_ERR_UNSUPPORTED
+    short_k = _args(lib, a, w, b, got, lib.EPI_BIAS, 1e-6)
+    short_k.K = 128
+    assert dll.cs_gemm_rmsnorm_noalloc(ctypes.byref(short_k), stream) == lib.CS_ERR_UNSUPPORTED
+    gelu = _args(lib, a, w, b, got, lib.EPI_GELU_ERF, 1e-6)
+    assert dll.cs_gemm_rmsnorm_noalloc(ctypes.byref(gelu), stream) == lib.CS_ERR_UNSUPPORTED
     torch.cuda.synchronize()
