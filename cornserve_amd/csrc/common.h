@@ -45,20 +45,24 @@ CS_DEVICE void split24(float v, uint32_t& hi_bits, uint32_t& lo_byte) {
 }
 
 // Four values at once: the addend's planes as raw words (two bf16 per word, four bytes in one word) joined with four
-// fp32 increments, and the sums split again.
+// fp32 increments, and the sums split again.  Same results as join24 / split24 element by element, in byte-select form
+// (seven vector instructions per value instead of eleven): with the correction byte's top bit flipped (lo' = lo ^ 0x80,
+// all four bytes of a word at once) the pair is an unsigned 24-bit word offset by half a bf16 unit,
+//   bits(value) = ((hi << 16) | (lo' << 8)) - 0x8000        and        (hi << 16) | (lo' << 8) = (bits(sum) + 0x8080) & ~0xFF
+// (adding 0x80 rounds to 24 bits, adding 0x8000 more rounds those half-up to hi and flips the top bit of the byte below).
 CS_DEVICE void add_split24(const float (&delta)[4], u32x2_t hi_in, uint32_t lo_in, u32x2_t& hi_out, uint32_t& lo_out) {
-  uint32_t h[2] = {0u, 0u}, l = 0u;
-#pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const uint32_t hi_r = (hi_in[r >> 1] >> (16 * (r & 1))) & 0xFFFFu;
-    const uint32_t lo_r = (lo_in >> (8 * r)) & 0xFFu;
-    uint32_t ho, lo;
-    split24(delta[r] + join24(hi_r, lo_r), ho, lo);
-    h[r >> 1] |= (ho & 0xFFFFu) << (16 * (r & 1));
-    l |= lo << (8 * r);
-  }
-  hi_out = u32x2_t{h[0], h[1]};
-  lo_out = l;
+  const uint32_t lo_f = lo_in ^ 0x80808080u;
+  // v_perm_b32: selector byte 0..3 picks that byte of the second source, 4..7 of the first, 0x0c a zero byte
+  const uint32_t w0 = __builtin_amdgcn_perm(hi_in[0], lo_f, 0x0504000cu);   // [hi0.b1 hi0.b0 lo'.b0 0]
+  const uint32_t w1 = __builtin_amdgcn_perm(hi_in[0], lo_f, 0x0706010cu);
+  const uint32_t w2 = __builtin_amdgcn_perm(hi_in[1], lo_f, 0x0504020cu);
+  const uint32_t w3 = __builtin_amdgcn_perm(hi_in[1], lo_f, 0x0706030cu);
+  const uint32_t c0 = __builtin_bit_cast(uint32_t, delta[0] + __builtin_bit_cast(float, w0 - 0x8000u)) + 0x8080u;
+  const uint32_t c1 = __builtin_bit_cast(uint32_t, delta[1] + __builtin_bit_cast(float, w1 - 0x8000u)) + 0x8080u;
+  const uint32_t c2 = __builtin_bit_cast(uint32_t, delta[2] + __builtin_bit_cast(float, w2 - 0x8000u)) + 0x8080u;
+  const uint32_t c3 = __builtin_bit_cast(uint32_t, delta[3] + __builtin_bit_cast(float, w3 - 0x8000u)) + 0x8080u;
+  hi_out = u32x2_t{__builtin_amdgcn_perm(c1, c0, 0x07060302u), __builtin_amdgcn_perm(c3, c2, 0x07060302u)};
+  lo_out = (__builtin_amdgcn_perm(c1, c0, 0x0c0c0501u) | __builtin_amdgcn_perm(c3, c2, 0x05010c0cu)) ^ 0x80808080u;
 }
 
 // One rotary pair in fp32 with every product and sum rounded on its own (no fused multiply-add), as the

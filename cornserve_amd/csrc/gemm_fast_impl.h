@@ -82,6 +82,13 @@ CS_DEVICE void buf_st_u32x4(__amdgpu_buffer_rsrc_t r, uint32_t off, u32x4_t v) {
 CS_DEVICE void buf_st_u32x2(__amdgpu_buffer_rsrc_t r, uint32_t off, u32x2_t v) { __builtin_amdgcn_raw_buffer_store_b64(v, r, off, 0, 0); }
 CS_DEVICE void buf_st_u32(__amdgpu_buffer_rsrc_t r, uint32_t off, uint32_t v) { __builtin_amdgcn_raw_buffer_store_b32(v, r, off, 0, 0); }
 
+// acc + a.lo * b.lo + a.hi * b.hi on words of two bf16 each (v_dot2c_f32_bf16): the row sums of the folded norms are
+// taken over the packed output words with it, by every form of the epilogue in the same order.
+CS_DEVICE float dot2_bf16(uint32_t a, uint32_t b, float acc) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), acc, false);
+}
+constexpr uint32_t BF16_ONE_PAIR = 0x3F803F80u;   // {1.0, 1.0}
+
 // Workgroup barrier without the full memory fence of __syncthreads(): the callers order LDS traffic with
 // explicit waits, and the asm statements keep the compiler from moving memory operations across it.
 CS_DEVICE void wg_barrier() {
@@ -142,6 +149,14 @@ struct RingShape {
 // rstd * (acc - mean * w_col_sum[n]) + bias[n] with mean and rstd from the two sets of parts (the norm's weight is
 // folded into W, its bias into the GEMM bias, and w_col_sum[n] = sum_k W'[n,k] carries the mean term).
 constexpr int FUSE_NORM_A = 1, FUSE_SUMSQ_C = 2, FUSE_LN_A = 3, FUSE_STATS_C = 4;
+// The forms whose epilogue takes its residual piece through the LDS ring (see the kernel): residual epilogue on the split
+// stream, one wave spanning the tile's columns, bf16 weights.  They use 4 KB of LDS behind the ring.
+template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE, bool SPLIT_RES>
+constexpr bool residual_piece_through_ring() {
+  constexpr int MT = BM / WAVES_M / 16, NT = BN / WAVES_N / 16;
+  return SPLIT_RES && EPI == CS_EPI_RESIDUAL && NT % 2 == 0 && !W_FP8 && !RingShape<BM, BN, W_FP8>::FIVE_UNITS && WAVES_N == 1 &&
+         (MT == 2 || MT == 4) && FUSE != FUSE_NORM_A && FUSE != FUSE_LN_A;
+}
 template <int BM, int BN, int WAVES_M, int WAVES_N, int EPI, bool W_FP8, int FUSE, bool SPLIT_RES>
 __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -397,6 +412,73 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     const int vb_next = vb + gridDim.x;
     const bool has_next = vb_next < ntiles;
     int m0_next = 0, n0_next = 0;
+    // ---- Residual GEMMs on the split 16-bit stream (the 160-column forms: one wave spans the tile's columns).  Their
+    //      epilogue reads a [rows x 160] piece of the residual stream, three bytes per value, that nothing has touched
+    //      since the previous encoder block, and with one wave per SIMD nothing hides that latency.  The last output
+    //      tile of a workgroup requests no further K tiles, so the slots of the ring fall free one by one in its last
+    //      iterations, and the piece is requested straight into them with the same direct-to-LDS loads as the operands
+    //      (no registers), per row block of 16 rows: NP loads of the bf16 plane (every lane fetches the 16 bytes of each
+    //      pair of pieces it will need, so it reads back its own bytes) and LO_LD loads of the byte plane (the row
+    //      block's [16][BN] bytes as one run of 16-byte chunks; 4-byte loads would cost the memory pipeline as much per
+    //      load as 16-byte ones).  A wave reads back only what it requested itself, so no barrier is involved.  The
+    //      memory pipeline takes about two clocks per cache line a load touches, whoever waits for it, so the loads
+    //      are spread: row block 0 (and the bias, into the 4 KB behind the ring) over the second half of the
+    //      third-last K iteration and the first half of the second-last, row block 1 over the two half-iterations
+    //      after that; row blocks 2 and 3 are requested during the epilogue itself, while row blocks 0 and 1 are
+    //      worked on.
+    constexpr bool PRE = residual_piece_through_ring<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE, SPLIT_RES>();
+    constexpr int NP = NT / 2;                          // pairs of pieces: 16 bytes of the bf16 plane per lane
+    constexpr int LO_CHUNKS = 16 * BN / 16;             // 16-byte chunks of a row block's byte plane
+    constexpr int LO_LD = (LO_CHUNKS + 63) / 64;        // ... and the loads that move them
+    constexpr int ROW_LD = NP + LO_LD;                  // direct loads per wave and row block
+    constexpr int ROW_HI_BYTES = NW * NP * 1024, ROW_LO_BYTES = NW * LO_LD * 1024, ROW_BYTES = ROW_HI_BYTES + ROW_LO_BYTES;
+    static_assert(!PRE || ((MT <= 2 ? ROW_BYTES : ROW_BYTES + ROW_HI_BYTES) <= STAGE && Ring::BYTES + NW * 1024 <= LDS_BYTES && BN * 2 <= 1024 &&
+                           2 * (ROW_LD + 1) <= NMFMA && MT <= 4),
+                  "two row blocks' bf16 planes and one byte plane fit a ring slot, the bias the room behind the ring");
+    const bool fast_tile = p.fast_epilogue && m0 + BM <= p.M && n0 + BN <= p.N;
+    const bool pre_on = PRE && fast_tile && !has_next;
+    // lane-only byte offsets of the direct loads (the tile and the row block go into the scalar offset)
+    uint32_t pre_hi_v = 0, pre_lo_v[PRE ? LO_LD : 1] = {}, pre_bias_v = 0;
+    int pre_sbase = 0;   // element offset of the wave's first row and the tile's first column in the residual matrix
+    if constexpr (PRE) {
+      if (pre_on) {
+        int lane_p = lane;
+        asm volatile("" : "+v"(lane_p));
+        pre_hi_v = ((uint32_t)(lane_p & 15) * (uint32_t)p.ldr + (uint32_t)(lane_p >> 4) * (4 * G)) * 2;
+#pragma unroll
+        for (int k = 0; k < LO_LD; ++k) {
+          const uint32_t g = (uint32_t)min(k * 64 + lane_p, LO_CHUNKS - 1), r = g / (BN / 16), c = g - r * (BN / 16);
+          pre_lo_v[k] = r * (uint32_t)p.ldr + c * 16;
+        }
+        pre_bias_v = (uint32_t)min(lane_p, BN * 2 / 16 - 1) * 16;
+        pre_sbase = (m0 + wm * WTM) * (int)p.ldr + n0;
+      }
+    }
+    // Direct load IDX (bf16 plane of pair IDX, then the byte plane's chunks, then -- IDX == ROW_LD -- the bias) of row
+    // block I; hi_base / lo_base are the LDS byte offsets of the row block's two regions.  A missing byte plane or
+    // bias is replaced by loads of the same size from the bf16 plane (never read back): the waits count loads, so every
+    // wave always issues the same number.  (Row block and piece go into the scalar offset: an immediate offset of a
+    // direct load would move the LDS side as well.)
+    // (a plain lambda around the device-only builtin: see load_a)
+    auto dma16 = [&](const __amdgpu_buffer_rsrc_t rs, char* lds_dst, uint32_t voff, int soff) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (lds_void_t*)lds_dst, 16, voff, soff, 0, 0);
+    };
+    auto residual_to_lds = [&](auto i_c, auto idx_c, int hi_base, int lo_base) {
+      constexpr int I = decltype(i_c)::value, IDX = decltype(idx_c)::value;
+      if constexpr (IDX < NP) {
+        constexpr int COL = (2 * IDX / G) * 16 * G + (2 * IDX % G) * 4;
+        dma16(rsrc_res, smem + hi_base + (wave * NP + IDX) * 1024, pre_hi_v, (pre_sbase + I * 16 * (int)p.ldr + COL) * 2);
+      } else if constexpr (IDX < ROW_LD) {
+        constexpr int Kk = IDX - NP;
+        dma16(p.residual_lo ? rsrc_reslo : rsrc_res, smem + lo_base + (wave * LO_LD + Kk) * 1024, pre_lo_v[PRE ? Kk : 0],
+              pre_sbase + I * 16 * (int)p.ldr);
+      } else {
+        dma16(p.bias ? rsrc_bias : rsrc_res, smem + Ring::BYTES + wave * 1024, pre_bias_v, p.bias ? n0 * 2 : 0);
+      }
+    };
+    // loads of row block 0 (+ bias) issued in the second half of the third-last iteration; the rest follows in the
+    // first half of the second-last.  Row block 1 likewise, one half-iteration later.
+    constexpr int PRE_N0 = ROW_LD + 1, PRE_N0A = (PRE_N0 + 1) / 2, PRE_N1 = ROW_LD, PRE_N1A = (PRE_N1 + 1) / 2;
     // K tile 0 has landed once at most the loads issued after it are outstanding.  (Loads complete in
     // order; stores of the previous epilogue that are still in flight only make this wait longer.)
     __builtin_amdgcn_s_waitcnt(waitcnt_vm(PENDING_AT_TILE_START));
@@ -434,13 +516,23 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           if constexpr (CUR_A) ld();
           else if (has_next) ld();
         }
+        // the rest of row block 0 (second-last iteration) / row block 1 (last): their slot was the current one an
+        // iteration ago
+        if constexpr (PRE && (TAIL == 2 || TAIL == 1)) {
+          constexpr int FIRST_LD = TAIL == 2 ? PRE_N0A : PRE_N1A, COUNT = (TAIL == 2 ? PRE_N0 : PRE_N1) - FIRST_LD, EVERY = NMFMA / COUNT;
+          if constexpr (N % EVERY == 0 && N / EVERY < COUNT) {
+            if (pre_on) residual_to_lds(ic<2 - TAIL>{}, ic<FIRST_LD + N / EVERY>{}, a_base_of(2, ring), a_base_of(2, ring) + ROW_HI_BYTES);
+          }
+        }
       });
       // K tile kt+1 has landed in this wave's part of LDS once at most the loads issued after it are
       // outstanding, and this wave has received its last fragments of K tile kt.
       if constexpr (TAIL == 1) {
         __builtin_amdgcn_s_waitcnt(WAITCNT_LGKM0);  // nothing more is read from LDS for this output tile
       } else if (!CUR_A && !has_next) {
-        __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));  // nothing was requested after K tile kt+1
+        // nothing was requested after K tile kt+1 -- except row block 0 of the residual piece, which may stay in flight
+        if (PRE && pre_on) __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(PRE ? PRE_N0 : 0));
+        else __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(0));
       } else {
         __builtin_amdgcn_s_waitcnt(waitcnt_vm_lgkm0(PENDING_AT_BARRIER));
       }
@@ -456,6 +548,14 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           auto ld = [&]() { direct_load(k_b, a_base_of(AHEAD_B, ring), w_base_of(AHEAD_B, ring), ic<PB_FIRST + N / EB>{}); };
           if constexpr (CUR_B) ld();
           else if (has_next) ld();
+        }
+        // the residual piece of the workgroup's last tile: first loads of row block 0 (third-last iteration) / row
+        // block 1 (second-last) into the slot that the barrier has just freed (the tile requests no K tile any more)
+        if constexpr (PRE && (TAIL == 3 || TAIL == 2)) {
+          constexpr int COUNT = TAIL == 3 ? PRE_N0A : PRE_N1A, EVERY = NMFMA / COUNT;
+          if constexpr (N % EVERY == 0 && N / EVERY < COUNT) {
+            if (pre_on) residual_to_lds(ic<3 - TAIL>{}, ic<N / EVERY>{}, a_base_of(0, ring), a_base_of(0, ring) + ROW_HI_BYTES);
+          }
         }
       });
       ring = slot_add(ring, RING5 ? 2 : 1);
@@ -722,6 +822,97 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     //      (row map, bias, residual / position rows) are issued ahead of the stores that follow them: a load inside the
     //      store loop would make the compiler wait for ALL outstanding memory operations (vmcnt counts stores too),
     //      i.e. for every store issued so far and for the next tile's prefetch, once per row block.
+    // ---- epilogue of a residual tile whose residual piece travels through the ring (pre_on).  Per value: accumulator
+    //      read, + bias (converted to fp32 once per tile), join / add / split by byte selects (add_split24), the row sums
+    //      over the packed output words.  `ring` has moved on three slots since row block 0 was requested, so row block 0
+    //      sits in slot ring, row block 1 in slot ring + 1; row block 2 goes to slot ring + 2 and row block 3 behind it
+    //      (bf16 plane) and behind row block 0 (byte plane), requested while row blocks 0 and 1 are worked on.
+    auto epilogue_from_lds = [&](auto) {
+      int lane_e = lane;
+      asm volatile("" : "+v"(lane_e));
+      const int kq = lane_e >> 4, fa = lane_e & 15;
+      const uint32_t row0 = (uint32_t)(m0 + wm * WTM + fa);
+      const uint32_t n_lane = (uint32_t)(n0 + wn * WTN + kq * (4 * G));
+      const int slot0 = a_base_of(0, ring), slot1 = a_base_of(1, ring), slot2 = a_base_of(2, ring);
+      auto hi_base_of = [&](int i) { return i == 0 ? slot0 : i == 1 ? slot1 : i == 2 ? slot2 : slot2 + ROW_BYTES; };
+      auto lo_base_of = [&](int i) { return i == 0 ? slot0 + ROW_HI_BYTES : i == 1 ? slot1 + ROW_HI_BYTES : i == 2 ? slot2 + ROW_HI_BYTES : slot0 + ROW_BYTES; };
+      // Row block 0 and the bias have landed once at most row block 1, requested after them, is outstanding: loads and
+      // stores complete in the order issued.  Row block i > 0 was requested before row block i - 1 was worked on, so it
+      // has landed once at most what that work issued is outstanding: 2 NP stores and the loads of row block i + 1.
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(ROW_LD) : "memory");
+      const uint32_t lo_mask = p.residual_lo ? 0xFFFFFFFFu : 0u, bias_mask = p.bias ? 0xFFFFFFFFu : 0u;
+      float bias_f[NT][4];
+      {
+        const char* const bsrc = smem + Ring::BYTES + wave * 1024 + kq * (4 * G) * 2;
+#pragma unroll
+        for (int jp = 0; jp < NP; ++jp) {
+          const u32x4_t bw = *(const u32x4_t*)(bsrc + piece_col(2 * jp) * 2);
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            bias_f[2 * jp + w / 2][2 * (w % 2)] = __builtin_bit_cast(float, (bw[w] & bias_mask) << 16);
+            bias_f[2 * jp + w / 2][2 * (w % 2) + 1] = __builtin_bit_cast(float, bw[w] & bias_mask & 0xFFFF0000u);
+          }
+        }
+      }
+      static_for<MT>([&](auto i_c) {
+        constexpr int i = decltype(i_c)::value;
+        if constexpr (i > 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * NP + (i + 1 < MT ? ROW_LD : 0)) : "memory");
+        // (a wave's chunk of a direct load is 64 lanes x 16 bytes; the bf16 plane: every lane reads back what it
+        // requested; the byte plane: rows of BN bytes, one after the other)
+        const char* const hi_src = smem + hi_base_of(i) + (wave * NP) * 1024 + lane_e * 16;
+        const char* const lo_src = smem + lo_base_of(i) + (wave * LO_LD) * 1024 + fa * BN + kq * (4 * G);
+        const uint32_t off = (row0 + 16 * i) * (uint32_t)p.ldc + n_lane;   // in elements
+        float ss = 0.f, sm = 0.f;
+        static_for<NP>([&](auto jp_c) {
+          constexpr int JP = decltype(jp_c)::value;
+          // row block i + 2 is requested while this one is worked on: its loads are spread over the pairs
+          if constexpr (i + 2 < MT) {
+            constexpr int PER = (ROW_LD + NP - 1) / NP;
+            static_for<PER>([&](auto q_c) {
+              constexpr int Q = JP * PER + decltype(q_c)::value;
+              if constexpr (Q < ROW_LD) residual_to_lds(ic<i + 2>{}, ic<Q>{}, hi_base_of(i + 2), lo_base_of(i + 2));
+            });
+          }
+          const u32x4_t hi_in = *(const u32x4_t*)(hi_src + JP * 1024);
+          // (without a byte plane the ring holds stand-in bytes: masked to zero, no branch)
+          const u32x2_t lo_raw = *(const u32x2_t*)(lo_src + piece_col(2 * JP));
+          const u32x2_t lo_in = {lo_raw[0] & lo_mask, lo_raw[1] & lo_mask};
+          u32x2_t hi_o[2];
+          uint32_t lo_o[2];
+          static_for<2>([&](auto h_c) {
+            constexpr int Hh = decltype(h_c)::value, J = 2 * JP + Hh;
+            float v[4];
+            static_for<4>([&](auto r_c) {
+              constexpr int Rr = decltype(r_c)::value;
+              float t;
+              asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"((i * NT + J) * 4 + Rr));
+              v[Rr] = t + bias_f[J][Rr];
+            });
+            add_split24(v, u32x2_t{hi_in[2 * Hh], hi_in[2 * Hh + 1]}, lo_in[Hh], hi_o[Hh], lo_o[Hh]);
+            if constexpr (FUSE == FUSE_SUMSQ_C || FUSE == FUSE_STATS_C) {
+              ss = dot2_bf16(hi_o[Hh][0], hi_o[Hh][0], ss);
+              ss = dot2_bf16(hi_o[Hh][1], hi_o[Hh][1], ss);
+            }
+            if constexpr (FUSE == FUSE_STATS_C) {
+              sm = dot2_bf16(hi_o[Hh][0], BF16_ONE_PAIR, sm);
+              sm = dot2_bf16(hi_o[Hh][1], BF16_ONE_PAIR, sm);
+            }
+          });
+          buf_st_u32x4(rsrc_c, (off + piece_col(2 * JP)) * 2, u32x4_t{hi_o[0][0], hi_o[0][1], hi_o[1][0], hi_o[1][1]});
+          buf_st_u32x2(rsrc_clo, off + piece_col(2 * JP), u32x2_t{lo_o[0], lo_o[1]});
+        });
+        if constexpr (FUSE == FUSE_SUMSQ_C || FUSE == FUSE_STATS_C) {
+          ss += __shfl_xor(ss, 16);
+          ss += __shfl_xor(ss, 32);
+          if (kq == 0) p.c_row_sumsq[(int64_t)(row0 + 16 * i) * CS_SUMSQ_PARTS + n0 / BN] = ss;
+        }
+        if constexpr (FUSE == FUSE_STATS_C) {
+          sm += __shfl_xor(sm, 16);
+          sm += __shfl_xor(sm, 32);
+          if (kq == 0) p.c_row_sum[(int64_t)(row0 + 16 * i) * CS_SUMSQ_PARTS + n0 / BN] = sm;
+        }
+      });
+    };
     auto epilogue = [&](auto fast_c) {
       constexpr bool FAST = decltype(fast_c)::value;
       const bf16_t* const pBias = (const bf16_t*)p.bias;
@@ -785,14 +976,15 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         for (int j = 0; j < NT; ++j) csum_v[j] = *(const f32x4_t*)(p.w_col_sum + clamp_n(n_lane + piece_col(j)));
       }
       bf16x4_t bias_v[NT];  // kept packed: half the registers of fp32 copies
+      if (pBias) {   // (one branch around all the loads, not one per load)
 #pragma unroll
-      for (int j = 0; j < NT; ++j) {
-        bias_v[j] = bf16x4_t{0, 0, 0, 0};
-        if constexpr (FAST) {
-          if (pBias) bias_v[j] = __builtin_bit_cast(bf16x4_t, buf_ld_u32x2(rsrc_bias, (uint32_t)(n_lane + piece_col(j)) * 2));
-        } else {
-          if (pBias) bias_v[j] = *(const bf16x4_t*)(pBias + clamp_n(n_lane + piece_col(j)));
+        for (int j = 0; j < NT; ++j) {
+          if constexpr (FAST) bias_v[j] = __builtin_bit_cast(bf16x4_t, buf_ld_u32x2(rsrc_bias, (uint32_t)(n_lane + piece_col(j)) * 2));
+          else bias_v[j] = *(const bf16x4_t*)(pBias + clamp_n(n_lane + piece_col(j)));
         }
+      } else {
+#pragma unroll
+        for (int j = 0; j < NT; ++j) bias_v[j] = bf16x4_t{0, 0, 0, 0};
       }
       f32x4_t scale_v[W_FP8 ? NT : 1];
       if constexpr (W_FP8) {
@@ -925,11 +1117,12 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
 #pragma unroll
           for (int j = 0; j < NT; ++j) {
             const bool nok = FAST || n_lane + piece_col(j) < p.N;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const float o = nok ? bf2f(out[j][r]) : 0.f;
-              ss += o * o;
-              if constexpr (FUSE == FUSE_STATS_C) sm += o;
+            const u32x2_t ow = nok ? __builtin_bit_cast(u32x2_t, out[j]) : u32x2_t{0u, 0u};
+            ss = dot2_bf16(ow[0], ow[0], ss);
+            ss = dot2_bf16(ow[1], ow[1], ss);
+            if constexpr (FUSE == FUSE_STATS_C) {
+              sm = dot2_bf16(ow[0], BF16_ONE_PAIR, sm);
+              sm = dot2_bf16(ow[1], BF16_ONE_PAIR, sm);
             }
           }
           ss += __shfl_xor(ss, 16);
@@ -1048,7 +1241,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       asm volatile("" : "+v"(lane_again));   // else the compiler proves the offsets loop-invariant and keeps them
       setup_frag_offsets(lane_again);
     }
-    else if (p.fast_epilogue && m0 + BM <= p.M && n0 + BN <= p.N) epilogue(std::true_type{});
+    else if (PRE && pre_on) {
+      if constexpr (PRE) epilogue_from_lds(0);
+    } else if (fast_tile) epilogue(std::true_type{});
     else epilogue(std::false_type{});
     if (!has_next) break;
     vb = vb_next;
@@ -1066,7 +1261,8 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   // matrix bases, and takes output row m for accumulator row m.
   const int64_t lim = (int64_t)UINT32_MAX - 64;
   p.fast_epilogue = !p.c_rows && (int64_t)p.M * p.ldc * 2 < lim && (!p.residual || (int64_t)p.M * p.ldr * 2 < lim);
-  constexpr int lds = RingShape<BM, BN, W_FP8>::BYTES;
+  constexpr int lds = RingShape<BM, BN, W_FP8>::BYTES +
+                      (residual_piece_through_ring<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE, SPLIT_RES>() ? NW * 1024 : 0);
   static bool attr_set = false;
   auto kern = gemm_fast_kernel<BM, BN, WAVES_M, WAVES_N, EPI, W_FP8, FUSE, SPLIT_RES>;
   if (!attr_set) {
