@@ -19,7 +19,7 @@
 namespace {
 
 struct ItemMeta {  // matches the int32[8] record documented in cornserve_amd.h
-  int t, gh, gw, unit_base, nwr, nwc, patch_base, reserved;
+  int t, gh, gw, unit_base, nwr, nwc, patch_base, src_unit_base;
 };
 
 __global__ __launch_bounds__(256) void vit_index_kernel(const ItemMeta* __restrict__ meta, int merge, int win,
@@ -53,7 +53,8 @@ __global__ __launch_bounds__(256) void vit_index_kernel(const ItemMeta* __restri
   const int w = c * merge + s % merge;
   const int64_t row_orig = (int64_t)u * mm + s;
   const int64_t row_win = (int64_t)up * mm + s;
-  if (src_rows) src_rows[row_win] = (int32_t)row_orig;
+  // (the caller's patch matrix may hold the items in another order than they are processed in)
+  if (src_rows) src_rows[row_win] = (int32_t)((int64_t)(it.src_unit_base + ul) * mm + s);
   if (pos_ids) {
     pos_ids[row_orig * 2 + 0] = h;
     pos_ids[row_orig * 2 + 1] = w;
@@ -275,7 +276,7 @@ extern "C" int cs_vit_seqlens_host(const int64_t* grid_thw_host, int32_t n_items
     m[4] = (int32_t)((gh + win - 1) / win);
     m[5] = (int32_t)((gw + win - 1) / win);
     m[6] = (int32_t)(unit_base * mm);
-    m[7] = 0;
+    m[7] = (int32_t)unit_base;
     unit_base += t * gh * gw;
   }
   *n_cu_window = nw;

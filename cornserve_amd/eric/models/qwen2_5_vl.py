@@ -248,14 +248,17 @@ class QwenVisionBase(EricModel):
 
 class Qwen2_5_VisionTransformer(QwenVisionBase):
     def __init__(self, config: Any, weight_format: str = "bf16", fold_norm: bool = True,
-                 split_residual: bool = True, fuse_window_attn: bool = True) -> None:
+                 split_residual: bool = True, fuse_window_attn: bool = True, fuse_min_rows: int = 0) -> None:
         """`fuse_window_attn`: run qkv projection + rotary + window attention of a block (:93-120) as ONE launch
-        (`ops.qkv_window_attn`: q, k and v stay in registers, the [L, 3*hidden] tensor is never written) whenever every
-        window of the batch is a full 64-row window -- all images with sides that are multiples of 8 patches.  Other
-        batches, batches of fewer than 3072 patches, fp8 weights and head dims other than 80 take the separate kernels.
-        q and k are then rounded to bf16 once (after the rotation) instead of twice: results stay inside the parity
-        tolerance, but an item's embedding is bit-identical across batches only among batches that take the same route
-        (setting the attribute to False afterwards selects the separate kernels for every batch).
+        (`ops.qkv_window_attn`: q, k and v stay in registers, the [L, 3*hidden] tensor is never written) for every ITEM
+        whose windows are all full 64-row windows -- images and videos with sides that are multiples of 8 patches.  Other
+        items of the same batch, fp8 weights and head dims other than 80 take the separate kernels.  The one launch
+        rounds q and k to bf16 once (after the rotation) instead of twice, so the two routes agree within the parity
+        tolerance, not bit for bit; since the route depends on the item alone, an item's embedding is the same bits
+        whatever it is batched with (setting the attribute to False afterwards selects the separate kernels for every
+        item).  `fuse_min_rows` > 0 is a deployment knob that gives this up for latency: a batch with fewer one-launch
+        rows than that takes the separate kernels throughout, whose GEMM has narrower tiles for few rows (one
+        1024-patch image alone: 3.99 against 4.28 ms; 3072 is where the one launch starts to pay).
 
         `split_residual`: carry the residual stream (:175,177) with 16 significant bits -- the bf16 tensor every
         kernel reads plus a byte plane with the next 8 mantissa bits, joined and re-split inside the two residual GEMMs
@@ -275,6 +278,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
             raise ValueError(f"Unknown weight_format: {weight_format}")
         self.weight_format = weight_format
         self.split_residual = bool(split_residual)
+        self.fuse_min_rows = int(fuse_min_rows)
         self.hidden_size = vc.hidden_size
         self.out_hidden_size = vc.out_hidden_size
         self.num_heads = vc.num_heads
@@ -366,19 +370,43 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
 
     def _index(self, grid_thw: np.ndarray):
         """Everything that depends on the grids only: window permutation, rotary table, attention work lists
-        (reference: rot_pos_emb :325-355, get_window_index :357-386, cu_seqlens :445-448)."""
+        (reference: rot_pos_emb :325-355, get_window_index :357-386, cu_seqlens :445-448), and the route of every item
+        through the window blocks.
+
+        An item whose windows are all whole (both sides multiples of the window, i.e. of 8 patches) takes the one-launch
+        form of qkv + rotary + window attention, every other item the separate kernels.  The choice depends on the item
+        alone, so an item's embedding does not depend on what it is batched with.  The items are PROCESSED with the
+        one-launch items first (a stable reordering: their rows are then one leading block of the batch); the index
+        kernel takes each item's place in the caller's patch matrix separately from its place in the processing
+        order, and `order` maps processing position to the caller's item number."""
         merge = self.spatial_merge_size
         win = self.window_size // merge // self.patch_size
         dev = self.device
-        sl = ops.vit_seqlens_host(grid_thw, merge, win)
-        (work_win, max_win), (work_full, max_full) = ops.attn_work_host(sl.cu_window), ops.attn_work_host(sl.cu_full)
+        g = np.asarray(grid_thw, dtype=np.int64).reshape(-1, 3)
+        n = g.shape[0]
+        units = g[:, 0] * (g[:, 1] // merge) * (g[:, 2] // merge)
+        if self.fuse_window_attn and n:
+            whole = ((g[:, 1] // merge) % win == 0) & ((g[:, 2] // merge) % win == 0)
+        else:
+            whole = np.zeros(n, dtype=bool)
+        fused_rows = int(units[whole].sum()) * merge * merge
+        if fused_rows < self.fuse_min_rows:
+            whole[:] = False
+            fused_rows = 0
+        order = np.concatenate([np.flatnonzero(whole), np.flatnonzero(~whole)]) if n else np.zeros(0, np.int64)
+        sl = ops.vit_seqlens_host(g[order], merge, win)
+        if n:
+            caller_unit_base = np.concatenate([[0], np.cumsum(units)[:-1]])
+            sl.item_meta[:, 7] = caller_unit_base[order]
+        # the separate kernels' work list covers the windows behind the one-launch rows (absolute row numbers)
+        first_sep = int(np.searchsorted(sl.cu_window, fused_rows))
+        work_win, max_win = ops.attn_work_host(sl.cu_window[first_sep:])
+        work_full, max_full = ops.attn_work_host(sl.cu_full)
         # one host-to-device copy for the three small arrays
         meta, dwin, dfull = ops.host_to_device_packed([sl.item_meta, work_win, work_full], dev)
         ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, merge, win, self._ensure_packed()["inv_freq"])
-        # every window a whole one (64 rows from a multiple of 64 on): the fused window-attention launch applies
-        windows_whole = bool(np.all(np.diff(sl.cu_window) == ops.QKV_WATTN_WINDOW))
         return (ix, ops.AttnPlan(dwin, work_win.shape[0], max_win), ops.AttnPlan(dfull, work_full.shape[0], max_full),
-                sl.total_patches, windows_whole)
+                sl.total_patches, fused_rows, order)
 
     def forward_device(self, pixel_values: torch.Tensor, grid_thw: np.ndarray, mark=None) -> list[torch.Tensor]:
         """pixel_values: bf16 [L, C*T*P*P] already on the device; grid_thw: host int64 [n,3].
@@ -400,7 +428,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
             if len(groups) > 1:
                 return self._forward_in_groups(pixel_values, grid_thw, groups, mark)
         mark("index")
-        ix, plan_win, plan_full, L, windows_whole = self._index(grid_thw)
+        ix, plan_win, plan_full, L, fused_rows, order = self._index(grid_thw)
         if pixel_values.shape[0] != L:
             raise ValueError(f"pixel_values has {pixel_values.shape[0]} rows but grid_thw describes {L} patches")
 
@@ -420,33 +448,33 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         att = torch.empty((L, H), dtype=torch.bfloat16, device=dev)
         hmid = torch.empty((L, pk["Ip"]), dtype=torch.bfloat16, device=dev)
         scale = d**-0.5
-        # one head and four windows per workgroup: below some 192 workgroups (3072 rows at 16 heads) the separate kernels,
-        # whose GEMM takes narrower tiles for few rows, fill the chip better (one 1024-patch image: 3.99 against 4.28 ms)
-        fused_windows = self.fuse_window_attn and windows_whole and (L // 256) * nh >= 192
+        # rows [0, fused_rows) belong to the items whose window blocks run as one launch, the rest to the others
+        xf = x[:fused_rows]
         for i, b in enumerate(pk["blocks"]):
             full = i in self.fullatt_block_indexes
-            plan = plan_full if full else plan_win
-            if fused_windows and "qkv_wattn" in b:
+            if not full and fused_rows:
                 wp, bp = b["qkv_wattn"]
                 if fold:
                     mark("gemm_qkv_attn_window")
-                    ops.qkv_window_attn(x, wp, bp, ix.cos_sin, nh, scale, a_row_sumsq=ss, norm_eps=eps, out=att)
+                    ops.qkv_window_attn(xf, wp, bp, ix.cos_sin[:fused_rows], nh, scale, a_row_sumsq=ss[:fused_rows], norm_eps=eps,
+                                        out=att[:fused_rows])
                 else:
                     mark("norm")
-                    ops.rmsnorm(x, b["n1"], eps, out=n)
+                    ops.rmsnorm(xf, b["n1"], eps, out=n[:fused_rows])
                     mark("gemm_qkv_attn_window")
-                    ops.qkv_window_attn(n, wp, bp, ix.cos_sin, nh, scale, out=att)
-            else:
+                    ops.qkv_window_attn(n[:fused_rows], wp, bp, ix.cos_sin[:fused_rows], nh, scale, out=att[:fused_rows])
+            if full or fused_rows < L:
+                lo = 0 if full else fused_rows           # first row the separate kernels work on in this block
                 if fold:
                     mark("gemm_qkv")
-                    self._g(x, b["qkv"], out=qkv, a_row_sumsq=ss, norm_eps=eps)
+                    self._g(x[lo:], b["qkv"], out=qkv[lo:], a_row_sumsq=ss[lo:], norm_eps=eps)
                 else:
                     mark("norm")
-                    ops.rmsnorm(x, b["n1"], eps, out=n)
+                    ops.rmsnorm(x[lo:], b["n1"], eps, out=n[lo:])
                     mark("gemm_qkv")
-                    self._g(n, b["qkv"], out=qkv)
+                    self._g(n[lo:], b["qkv"], out=qkv[lo:])
                 mark("attn_full" if full else "attn_window")
-                ops.attn_varlen_rotary_(qkv, plan, nh, d, scale, ix.cos_sin, out=att)
+                ops.attn_varlen_rotary_(qkv, plan_full if full else plan_win, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")
             if fold:
                 self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss, **res)
@@ -471,9 +499,13 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         # merged row m sits at window-order position m; it belongs at row window_index[m]
         self._g(y, pk["fc2"], c_rows=ix.window_index32, out=out)
         mark("end")
-        g = grid_thw.reshape(-1, 3)
+        g = np.asarray(grid_thw, dtype=np.int64).reshape(-1, 3)[order]
         seqlens = (g[:, 0] * g[:, 1] * g[:, 2]) // unit
-        return list(out.split([int(s) for s in seqlens], dim=0))
+        parts = out.split([int(s) for s in seqlens], dim=0)     # in processing order
+        result: list = [None] * len(parts)
+        for pos, item in enumerate(order.tolist()):
+            result[item] = parts[pos]
+        return result
 
 class ModalityProcessor(BaseModalityProcessor):
     """Qwen2.5-VL modality processor (reference: :488-512). Wraps the HF image processor, which has to be

@@ -179,7 +179,9 @@ int cs_layernorm(const void* x, int64_t ldx, const void* w, const void* b, void*
  *   cu_full_host    int32, n_cu_full entries written   (capacity cap_full)
  *   item_meta_host  int32 [n_items][8]: t, gh = h/merge, gw = w/merge, first merged unit of the item,
  *                   ceil(gh/win), ceil(gw/win) (non-empty windows along h and w), first patch row of the
- *                   item, reserved (0)
+ *                   item, first merged unit of the item in the CALLER'S patch matrix (written equal to the
+ *                   fourth entry; a caller that processes the items in another order than its patch matrix
+ *                   holds them overwrites it, and src_rows of cs_vit_index then points into that matrix)
  * merge = spatial merge size (2), win = window side in merged units (window_size/merge/patch = 4).
  * Returns CS_ERR_TOO_LARGE if a capacity is too small.                                            */
 int cs_vit_seqlens_host(const int64_t* grid_thw_host, int32_t n_items, int32_t merge, int32_t win,
@@ -192,7 +194,8 @@ int cs_vit_seqlens_host(const int64_t* grid_thw_host, int32_t n_items, int32_t m
  *   window_index  int32 [U]   qwen2_5_vl.py:357-386 (value = original unit at window-order position;
  *                             the reference holds the same values as int64)
  *   reverse_index int32 [U]   argsort(window_index), :478
- *   src_rows      int32 [L]   original patch row feeding window-order row m (units of merge^2 rows), :438-440
+ *   src_rows      int32 [L]   original patch row feeding window-order row m (units of merge^2 rows), :438-440,
+ *                             counted from the item's eighth meta entry (its first unit in the caller's matrix)
  *   pos_ids       int32 [L,2] (h,w) of each patch in ORIGINAL order, rot_pos_emb :325-350
  *   cos_sin       fp32  [L, 2*rot_dim] window-order rotary table: cos(angles) | sin(angles) with
  *                 angles = [h*inv_freq | w*inv_freq], :251-259,352-354,441-443 and :26-29
