@@ -174,7 +174,7 @@ def cpu_baseline(sd, n_sample_images: int, min_seconds: float = 10.0, gpu_out: l
     GPU step for the same (leading) images; the oracle's output then also serves as the checker at full size."""
     import torch
 
-    from cornserve_amd import synth
+    from tests import synth
     from oracle import qwen2_5_vl as oq
 
     # every core this process may run on (a GPU box gives a job a share of the host: the affinity mask or
@@ -301,7 +301,7 @@ def hbm_kernels(dev, rows_list=(8192, 131072), reps: int = 20) -> dict:
 def _qwen_model(dev, sd, weight_format="bf16", **kw):
     import torch
 
-    from cornserve_amd import synth
+    from tests import synth
     from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
 
     model = Qwen2_5_VisionTransformer(synth.qwen_vision_config(), weight_format=weight_format, **kw)
@@ -317,7 +317,7 @@ def parity_cfg2(dev, seed: int = 0, n_images: int = N_IMAGES) -> dict:
     import numpy as np
     import torch
 
-    from cornserve_amd import synth
+    from tests import synth
     from oracle import qwen2_5_vl as oq
     from oracle.metrics import distances
 
@@ -359,7 +359,7 @@ def parity_cfg4(dev, seed: int = 22, items=(12, 0)) -> dict:
     import numpy as np
     import torch
 
-    from cornserve_amd import synth
+    from tests import synth
     from oracle import qwen2_5_vl as oq
     from oracle.metrics import distances
 
@@ -387,7 +387,7 @@ def parity_cfg5(dev, seed: int = 23) -> dict:
     import numpy as np
     import torch
 
-    from cornserve_amd import synth
+    from tests import synth
     from oracle import qwen2_5_vl as oq
     from oracle.metrics import distances
 
@@ -419,7 +419,7 @@ def other_workload(name: str, steps: int, warmup: int, dev) -> dict:
     import numpy as np
     import torch
 
-    from cornserve_amd import synth
+    from tests import synth
 
     def qwen_like(model_cls, cfg, sd, grids, in_dim, **kw):
         model = model_cls(cfg, **kw)
@@ -517,7 +517,8 @@ def main() -> None:
     import numpy as np
     import torch
 
-    from cornserve_amd import lib, ops, synth
+    from cornserve_amd import lib, ops
+    from tests import synth
     from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
 
     lib.load()

@@ -33,7 +33,7 @@ import torch
 HERE = Path(__file__).resolve().parent
 sys.path.insert(0, str(HERE.parent.parent))
 
-from cornserve_amd import synth  # noqa: E402
+from tests import synth  # noqa: E402
 
 INDEX_GRIDS = {
     "cfg1": [(1, 32, 32)],

@@ -11,7 +11,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from cornserve_amd import synth
+from tests import synth
 from cornserve_amd.eric.api import Modality
 from oracle import gemma3 as og
 from oracle import qwen2_5_vl as oq

@@ -6,7 +6,7 @@ import numpy as np
 import pytest
 import torch
 
-from cornserve_amd import synth
+from tests import synth
 from cornserve_amd.eric.api import Modality
 from cornserve_amd.eric.models import base, registry
 from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
@@ -118,7 +118,7 @@ def test_frame_processor_resize_and_table_match_the_hf_pil_processor():
 
 
 def test_qwen2_vl_class_surface():
-    from cornserve_amd import synth
+    from tests import synth
     from cornserve_amd.eric.models.qwen2_vl import Qwen2VisionTransformer
     from cornserve_amd.eric.models.registry import MODEL_REGISTRY
 
@@ -137,7 +137,7 @@ def test_qwen2_vl_class_surface():
 
 
 def test_qwen3_vl_class_surface():
-    from cornserve_amd import synth
+    from tests import synth
     from cornserve_amd.eric.models.qwen3_vl import Qwen3_VisionTransformer
     from cornserve_amd.eric.models.registry import MODEL_REGISTRY
 
@@ -221,7 +221,7 @@ def _write_checkpoint(directory, config, tensors: dict, shards: int = 2, with_in
 
 
 def test_load_model_from_local_checkpoint(tmp_path):
-    from cornserve_amd import synth
+    from tests import synth
     from cornserve_amd.eric.loader import load_model
     from cornserve_amd.eric.models.gemma3 import Gemma3VisionEncoder
     from cornserve_amd.eric.models.qwen2_5_vl import Qwen2_5_VisionTransformer
