@@ -5,7 +5,8 @@ The reference's router runs the Hugging Face image processor on the CPU and ship
 eric/router/processor.py:46-131).  With this format the router only RESIZES (the processor's `smart_resize` target
 size and its PIL bicubic resampling) and ships the uint8 frames, 8x fewer bytes; rescale, normalise and the patch
 layout happen on the GPU (`cs_qwen_patchify_u8`), reproducing the processor's float arithmetic exactly through a
-table of the 256 byte values per channel.
+table of the 256 byte values per channel.  The router can also ship the frames as decoded: the same resampling then
+runs on the GPU (`cs_resize_u8_pass`, Pillow's fixed-point bicubic bit for bit) at the target size computed here.
 """
 
 from __future__ import annotations
@@ -55,16 +56,22 @@ def byte_table(mean=CLIP_MEAN, std=CLIP_STD, scale: float = 1 / 255, arithmetic:
     raise ValueError(f"unknown arithmetic {arithmetic!r}")
 
 
+def as_frames(frames) -> np.ndarray:
+    """uint8 [H,W,3] or [T,H,W,3] -> contiguous uint8 [T,H,W,3]; anything else is refused."""
+    frames = np.asarray(frames)
+    if frames.ndim == 3:
+        frames = frames[None]
+    if frames.dtype != np.uint8 or frames.ndim != 4 or frames.shape[-1] != 3:
+        raise ValueError("frames must be uint8 [H,W,3] or [T,H,W,3] (RGB)")
+    return np.ascontiguousarray(frames)
+
+
 def resize_frames(frames: np.ndarray, factor: int = 28, min_pixels: int = 56 * 56,
                   max_pixels: int = 14 * 14 * 4 * 1280) -> np.ndarray:
     """uint8 [H,W,3] or [T,H,W,3] -> uint8 [T,H',W',3] at the processor's target size (PIL bicubic, as the
     processor's PIL backend resamples)."""
     from PIL import Image
 
-    frames = np.asarray(frames)
-    if frames.ndim == 3:
-        frames = frames[None]
-    if frames.dtype != np.uint8 or frames.ndim != 4 or frames.shape[-1] != 3:
-        raise ValueError("frames must be uint8 [H,W,3] or [T,H,W,3] (RGB)")
+    frames = as_frames(frames)
     h, w = target_size(frames.shape[1], frames.shape[2], factor, min_pixels, max_pixels)
     return np.stack([np.asarray(Image.fromarray(f).resize((w, h), resample=Image.Resampling.BICUBIC)) for f in frames])

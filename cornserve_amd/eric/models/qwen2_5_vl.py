@@ -168,11 +168,14 @@ class QwenVisionBase(EricModel):
     def _g(a: torch.Tensor, lin: dict, **kw) -> torch.Tensor:
         return ops.gemm(a, lin["w"], lin["b"], w_scale=lin["s"], **kw)
 
-    def patchify_frames(self, frames: list[torch.Tensor], arithmetic: str = "fused") -> tuple[torch.Tensor, np.ndarray]:
-        """uint8 frames of every item ([T,H,W,3] or [H,W,3], already at the processor's target size, on the host
-        or the device) -> (pixel_values [L, C*T*P*P] in the model dtype on the device, grid_thw int64 [n,3]): what
-        the Hugging Face processor the reference runs (:488-512) produces from the same frames, with rescale,
-        normalise and the patch layout done on the GPU."""
+    def patchify_frames(self, frames: list[torch.Tensor], arithmetic: str = "fused",
+                        pixel_budgets: list | None = None) -> tuple[torch.Tensor, np.ndarray]:
+        """uint8 frames of every item ([T,H,W,3] or [H,W,3], on the host or the device) -> (pixel_values
+        [L, C*T*P*P] in the model dtype on the device, grid_thw int64 [n,3]): what the Hugging Face processor the
+        reference runs (:488-512) produces from the same frames, with rescale, normalise and the patch layout done on
+        the GPU.  Without `pixel_budgets` the frames are already at the processor's target size; with it (one
+        (min_pixels, max_pixels) pair per item) they are as decoded and the processor's resize runs on the GPU too
+        (`frames.target_size`, then `ops.resize_bicubic_u8`: Pillow's bicubic, bit for bit)."""
         p, m, tps, dev = self.patch_size, self.spatial_merge_size, self.temporal_patch_size, self.device
         key = ("byte_table", arithmetic)   # (a model's mean / std are fixed)
         pk = self._ensure_packed()
@@ -185,10 +188,14 @@ class QwenVisionBase(EricModel):
                 f = f[None]
             if f.dtype != torch.uint8 or f.dim() != 4 or f.shape[-1] != 3:
                 raise ValueError("frames must be uint8 [T,H,W,3] or [H,W,3] (RGB)")
+            f = f.contiguous().to(dev, non_blocking=True)
+            if pixel_budgets is not None:
+                lo, hi = (int(v) for v in torch.as_tensor(pixel_budgets[len(items)]).reshape(-1).tolist())
+                f = ops.resize_bicubic_u8(f, *frame_ops.target_size(f.shape[1], f.shape[2], p * m, lo, hi))
             T, H, W, _ = f.shape
             if H % (p * m) or W % (p * m) or T < 1:
                 raise ValueError(f"frame size {H}x{W} is not a multiple of {p * m}: resize first (frames.resize_frames)")
-            items.append(f.contiguous().to(dev, non_blocking=True))
+            items.append(f)
             grids.append((-(-T // tps), H // p, W // p))
         grid = np.asarray(grids, dtype=np.int64).reshape(-1, 3)
         L = int((grid[:, 0] * grid[:, 1] * grid[:, 2]).sum())
@@ -232,13 +239,20 @@ class QwenVisionBase(EricModel):
         """See the reference docstring (:402-413): `pixel_values` + `image_grid_thw` for images,
         `pixel_values_videos` + `video_grid_thw` for videos.  In addition to the reference's format, a batch
         may carry `pixel_frames` / `pixel_frames_videos` instead: one uint8 [T,H,W,3] tensor of resized frames
-        per item (see `FrameModalityProcessor`); the grids follow from the shapes."""
+        per item (see `FrameModalityProcessor`); the grids follow from the shapes.  With `raw_frames` /
+        `raw_frames_videos` the frames are as decoded, and `raw_frames_budget` holds each item's
+        (min_pixels, max_pixels): the resize runs on the GPU as well."""
         if modality == Modality.IMAGE:
-            px_key, grid_key, frame_key = "pixel_values", "image_grid_thw", "pixel_frames"
+            px_key, grid_key, frame_key, raw_key = "pixel_values", "image_grid_thw", "pixel_frames", "raw_frames"
         elif modality == Modality.VIDEO:
-            px_key, grid_key, frame_key = "pixel_values_videos", "video_grid_thw", "pixel_frames_videos"
+            px_key, grid_key, frame_key, raw_key = ("pixel_values_videos", "video_grid_thw", "pixel_frames_videos",
+                                                    "raw_frames_videos")
         else:
             raise ValueError(f"Unsupported modality: {modality}")
+        if raw_key in batch:
+            if len(batch.get("raw_frames_budget", ())) != len(batch[raw_key]):
+                raise ValueError(f"`{raw_key}` needs one `raw_frames_budget` entry (min_pixels, max_pixels) per item")
+            return self.forward_device(*self.patchify_frames(batch[raw_key], pixel_budgets=batch["raw_frames_budget"]))
         if frame_key in batch:
             return self.forward_device(*self.patchify_frames(batch[frame_key]))
         pixel_values = ops.cat_to_device(batch[px_key], self.device, self.dtype)
@@ -531,21 +545,31 @@ class ModalityProcessor(BaseModalityProcessor):
 
 
 class FrameModalityProcessor(BaseModalityProcessor):
-    """Processor for the uint8-frame input format: resizes only (the Hugging Face processor's target size and
-    PIL bicubic resampling) and emits `pixel_frames` / `pixel_frames_videos`; rescale, normalise and the patch
-    layout run on the GPU inside the model's forward.  Needs no model files."""
+    """Processor for the uint8-frame input formats.  With `resize_on="router"` it resizes only (the Hugging Face
+    processor's target size and PIL bicubic resampling) and emits `pixel_frames` / `pixel_frames_videos`; rescale,
+    normalise and the patch layout run on the GPU inside the model's forward.  With `resize_on="gpu"` it only checks
+    the frames and emits them as decoded (`raw_frames` / `raw_frames_videos` plus the pixel budget); the model resizes
+    them on the GPU to the same bytes.  Needs no model files."""
 
     def __init__(self, model_id: str, min_pixels: int = 56 * 56, max_pixels: int = 14 * 14 * 4 * 1280,
-                 factor: int = 28) -> None:
+                 factor: int = 28, resize_on: str = "router") -> None:
         """`factor` = patch size x merge size of the encoder (28 for Qwen2-VL / Qwen2.5-VL, 32 for Qwen3-VL)."""
         super().__init__(model_id=model_id)
-        self.min_pixels, self.max_pixels, self.factor = min_pixels, max_pixels, factor
+        if resize_on not in ("router", "gpu"):
+            raise ValueError(f"resize_on must be 'router' or 'gpu', got {resize_on!r}")
+        self.min_pixels, self.max_pixels, self.factor, self.resize_on = min_pixels, max_pixels, factor, resize_on
 
-    def _resized(self, frames) -> torch.Tensor:
-        return torch.from_numpy(frame_ops.resize_frames(frames, self.factor, self.min_pixels, self.max_pixels))
+    def _frames(self, frames, key: str) -> dict[str, torch.Tensor]:
+        if self.resize_on == "router":
+            resized = frame_ops.resize_frames(frames, self.factor, self.min_pixels, self.max_pixels)
+            return {"pixel_frames" + key: torch.from_numpy(resized)}
+        raw = frame_ops.as_frames(frames)
+        frame_ops.target_size(raw.shape[1], raw.shape[2], self.factor, self.min_pixels, self.max_pixels)   # aspect check
+        return {"raw_frames" + key: torch.from_numpy(raw),
+                "raw_frames_budget": torch.tensor([self.min_pixels, self.max_pixels], dtype=torch.int64)}
 
     def get_image_processor(self) -> Callable | None:
-        return lambda image: {"pixel_frames": self._resized(image)}
+        return lambda image: self._frames(image, "")
 
     def get_video_processor(self) -> Callable | None:
-        return lambda video: {"pixel_frames_videos": self._resized(video)}
+        return lambda video: self._frames(video, "_videos")

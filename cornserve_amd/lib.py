@@ -17,7 +17,7 @@ CS_ERR_INVALID_ARG = 1
 CS_ERR_UNSUPPORTED = 2
 CS_ERR_LAUNCH = 3
 CS_ERR_TOO_LARGE = 4
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH, EPI_QUICK_GELU = range(6)
 
@@ -102,6 +102,8 @@ _SIGNATURES: dict[str, list] = {
     "cs_attn_work_host": [c_void_p, c_int32, c_int32, c_void_p, c_int32, POINTER(c_int32)],
     "cs_qwen_patchify_u8": [c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_int64,
                             c_int32, c_void_p],
+    "cs_resize_bicubic_taps_host": [c_int32, c_int32, c_void_p, c_void_p, c_int32, POINTER(c_int32)],
+    "cs_resize_u8_pass": [c_void_p, c_int64, c_int32, c_int32, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p],
     "cs_patchify_nchw": [c_void_p, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p, c_int64, c_void_p],
     "cs_avgpool_gemma_rmsnorm": [c_void_p, c_void_p, c_void_p, c_int32, c_int32, c_int32, c_int32, c_float, c_void_p],
     "cs_cast_f32_bf16": [c_void_p, c_void_p, c_int64, c_void_p],

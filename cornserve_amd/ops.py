@@ -14,6 +14,7 @@ from __future__ import annotations
 
 import ctypes
 import functools
+import math
 from dataclasses import dataclass
 
 import numpy as np
@@ -40,7 +41,7 @@ def host_to_device(a: np.ndarray, device: torch.device) -> torch.Tensor:
     a = np.ascontiguousarray(a)
     if a.size == 0:
         return torch.from_numpy(a.copy()).to(device)
-    staged = torch.empty(a.shape, dtype=torch.from_numpy(a[:0].reshape(-1)).dtype, pin_memory=True)
+    staged = torch.empty(a.shape, dtype=torch.from_numpy(np.empty(0, dtype=a.dtype)).dtype, pin_memory=True)
     staged.numpy()[...] = a
     return staged.to(device, non_blocking=True)
 
@@ -62,7 +63,7 @@ def host_to_device_packed(arrays: list[np.ndarray], device: torch.device) -> lis
     dev = staged.to(device, non_blocking=True)
     out = []
     for a, o in zip(arrays, offs):
-        dt = torch.from_numpy(a[:0].reshape(-1)).dtype
+        dt = torch.from_numpy(np.empty(0, dtype=a.dtype)).dtype
         out.append(dev[o : o + a.nbytes].view(dt).view(a.shape))
     return out
 
@@ -702,6 +703,69 @@ def attn_varlen_rotary_(qkv: torch.Tensor, plan: AttnPlan, heads: int, head_dim:
     return attn_varlen(q, k, v, plan, heads, head_dim, scale, out=out)
 
 
+@functools.lru_cache(maxsize=64)
+def resize_bicubic_taps_host(in_size: int, out_size: int) -> tuple[np.ndarray, np.ndarray]:
+    """Pillow's bicubic taps for one axis: (bounds int32 [out_size,2] = (first input position, tap count),
+    taps int32 [out_size,ksize] in 22-bit fixed point).  Host arithmetic only; no GPU call."""
+    lib = _l.load()
+    ksize = ctypes.c_int32(0)
+    _l.check(lib.cs_resize_bicubic_taps_host(in_size, out_size, None, None, 0, ctypes.byref(ksize)),
+             "cs_resize_bicubic_taps_host")
+    bounds = np.empty((out_size, 2), dtype=np.int32)
+    taps = np.empty((out_size, ksize.value), dtype=np.int32)
+    _l.check(lib.cs_resize_bicubic_taps_host(in_size, out_size, bounds.ctypes.data, taps.ctypes.data, ksize.value,
+                                             ctypes.byref(ksize)), "cs_resize_bicubic_taps_host")
+    bounds.setflags(write=False)
+    taps.setflags(write=False)
+    return bounds, taps
+
+
+def resize_bicubic_u8(frames: torch.Tensor, out_h: int, out_w: int) -> torch.Tensor:
+    """uint8 frames [T,H,W,C] on the device -> [T,out_h,out_w,C], bit for bit what Pillow's
+    `Image.resize((out_w, out_h), BICUBIC)` makes of every frame: a pass along x, then one along y, an axis that keeps
+    its size skipped (frames already at the target size come back as they are)."""
+    _req(frames, torch.uint8, "frames")
+    if frames.dim() != 4 or not frames.is_contiguous():
+        raise ValueError("frames must be contiguous uint8 [T,H,W,C]")
+    if out_h <= 0 or out_w <= 0:
+        raise ValueError(f"target size must be positive, got {out_h}x{out_w}")
+    T, H, W, C = frames.shape
+    todo = [(axis, a, b) for axis, a, b in ((2, W, out_w), (1, H, out_h)) if a != b]
+    if not todo:
+        return frames
+    host = [t for _, a, b in todo for t in resize_bicubic_taps_host(a, b)]
+    dev = host_to_device_packed(list(host), frames.device)
+    for i, (axis, a, b) in enumerate(todo):
+        shape = list(frames.shape)
+        shape[axis] = b
+        out = torch.empty(shape, dtype=torch.uint8, device=frames.device)
+        torch.ops.cornserve_amd.resize_u8_pass_(out, frames, dev[2 * i], dev[2 * i + 1], axis)
+        frames = out
+    return frames
+
+
+def _resize_u8_pass_impl(out, src, bounds, taps, axis) -> None:
+    lib = _l.load()
+    _req(src, torch.uint8, "src")
+    _req(out, torch.uint8, "out")
+    _req(bounds, torch.int32, "bounds")
+    _req(taps, torch.int32, "taps")
+    if src.dim() != out.dim() or not 0 <= axis < src.dim() or not src.is_contiguous() or not out.is_contiguous():
+        raise ValueError("src and out must be contiguous tensors of the same rank")
+    if any(a != b for i, (a, b) in enumerate(zip(src.shape, out.shape)) if i != axis):
+        raise ValueError(f"out {tuple(out.shape)} must match src {tuple(src.shape)} except along axis {axis}")
+    n_in, n_out = src.shape[axis], out.shape[axis]
+    if (tuple(bounds.shape) != (n_out, 2) or taps.dim() != 2 or taps.shape[0] != n_out or not bounds.is_contiguous()
+            or not taps.is_contiguous() or len({src.device, out.device, bounds.device, taps.device}) != 1):
+        raise ValueError(f"bounds must be int32 [{n_out},2] and taps int32 [{n_out},ksize] on the frames' device")
+    outer = math.prod(src.shape[:axis])
+    inner = math.prod(src.shape[axis + 1:])
+    if src.numel() == 0 or out.numel() == 0:
+        raise ValueError("empty frames")
+    _l.check(lib.cs_resize_u8_pass(src.data_ptr(), outer, n_in, n_out, inner, bounds.data_ptr(), taps.data_ptr(),
+                                   taps.shape[1], out.data_ptr(), _stream()), "cs_resize_u8_pass")
+
+
 def qwen_patchify_u8(frames: torch.Tensor, table: torch.Tensor, patch: int, merge: int, temporal: int, *,
                      out: torch.Tensor | None = None, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """uint8 frames [T,H,W,3] -> normalised patch rows [ceil(T/temporal)*(H/patch)*(W/patch), 3*temporal*patch^2]
@@ -894,6 +958,7 @@ _OPERATORS: dict[str, tuple[str, object]] = {
                      "int head_dim, float scale, Tensor? cos_sin, bool keys_rotated) -> ()", _attn_varlen_impl),
     "qwen_patchify_u8_": ("(Tensor(a!) out, Tensor frames, Tensor table, int patch, int merge, int temporal) -> ()",
                           _qwen_patchify_u8_impl),
+    "resize_u8_pass_": ("(Tensor(a!) out, Tensor src, Tensor bounds, Tensor taps, int axis) -> ()", _resize_u8_pass_impl),
     "patchify_nchw_": ("(Tensor(a!) out, Tensor pixels, int patch) -> ()", _patchify_nchw_impl),
     "qkv_window_attn_": ("(Tensor(a!) out, Tensor x, Tensor w_packed, Tensor b_packed, Tensor cos_sin, int heads, "
                          "float scale, Tensor? a_row_sumsq, float norm_eps) -> ()", _qkv_window_attn_impl),

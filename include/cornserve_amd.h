@@ -36,7 +36,7 @@ extern "C" {
 #define CS_ERR_TOO_LARGE 4
 
 /* ABI version of this header; cs_abi_version() returns the value the library was built with. */
-#define CS_ABI_VERSION 4
+#define CS_ABI_VERSION 5
 int cs_abi_version(void);
 
 /* ------------------------------------------------------------------------------------------------
@@ -309,6 +309,24 @@ int cs_patchify_nchw(const void* pixels, int32_t B, int32_t C, int32_t H, int32_
 int cs_qwen_patchify_u8(const void* frames, int32_t T, int32_t H, int32_t W, int32_t patch, int32_t merge,
                         int32_t temporal, const float* table, void* out, int64_t ldo, int32_t out_fp32,
                         void* stream);
+/* Bicubic resampling of uint8 frames on the device, bit for bit Pillow's Image.resize(size, BICUBIC): the
+ * resize the Hugging Face Qwen2-VL image processor (PIL backend) applies at its smart_resize target size
+ * before rescale + normalise.  The reference runs it on the router's CPU (ModalityProcessor,
+ * qwen2_5_vl.py:488-512, called from router/processor.py:46-131); with these two calls the router ships the
+ * frames as decoded and the resize runs in front of cs_qwen_patchify_u8.
+ * cs_resize_bicubic_taps_host (host only, no GPU call): the integer taps of one axis.  *ksize receives the taps
+ *   per output position; with bounds == taps == NULL that is all it does (size query).  Otherwise bounds
+ *   [out_size][2] receives (first input position, tap count) and taps [out_size][cap_ksize] the 22-bit
+ *   fixed-point weights, zero past the count; cap_ksize >= *ksize.
+ * cs_resize_u8_pass: one pass along the middle axis of src uint8 [outer, in_size, inner] -> dst
+ *   [outer, out_size, inner], bounds / taps on the device, ksize = the row stride of taps (the cap_ksize above).
+ *   Frames [T,H,W,3] -> [T,H2,W2,3] the way Pillow orders it: along x first (outer T*H, in W, out W2, inner 3)
+ *   into a temporary, then along y (outer T, in H, out H2, inner W2*3); an axis whose size does not change is
+ *   skipped.                                                                                         */
+int cs_resize_bicubic_taps_host(int32_t in_size, int32_t out_size, int32_t* bounds, int32_t* taps,
+                                int32_t cap_ksize, int32_t* ksize);
+int cs_resize_u8_pass(const void* src, int64_t outer, int32_t in_size, int32_t out_size, int64_t inner,
+                      const int32_t* bounds, const int32_t* taps, int32_t ksize, void* dst, void* stream);
 /* Gemma3MultiModalProjector front half, gemma3.py:36-46: AvgPool2d(k) over the side x side token grid
  * followed by GemmaRMSNorm.  x: bf16 [B, side*side, H] -> y: bf16 [B, (side/k)^2, H].             */
 int cs_avgpool_gemma_rmsnorm(const void* x, const void* w, void* y, int32_t B, int32_t side, int32_t k,

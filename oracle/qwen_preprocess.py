@@ -26,8 +26,17 @@ written independently (brute force over every output element of small cases); vi
 of repeated frames == the image"; the "fused" table entry by entry against an exact-rational evaluation of its four
 binary32 operations with IEEE round-to-nearest-even after each (what the standard fixes for that sequence; float64
 intermediates or the other order of operations fail it).  PARITY UNPINNED: that torchvision's normalize -- absent here
--- is exactly "subtract, then divide" in float32 (taken from its published source), and resampling (bicubic resize),
-which is not restated at all: it stays in the caller's CPU code.
+-- is exactly "subtract, then divide" in float32 (taken from its published source).
+
+* `pillow_bicubic_resize` the resampling the PIL processor applies before all of the above (`image.resize(size,
+                          resample=BICUBIC)`): the third-party package Pillow (the reference's pyproject lists it
+                          without a version; 12.2.0 is installed here), libImaging/Resample.c: per-axis taps
+                          (`precompute_coeffs` with the cubic a = -0.5 filter, `normalize_coeffs_8bpc`: 22 fractional
+                          bits) and the two 8-bit passes (`ImagingResampleHorizontal_8bpc`, then
+                          `ImagingResampleVertical_8bpc`, a uint8 image between them).  Pinned bit for bit against the
+                          installed Pillow itself on random, binary and smooth images over random size pairs (up- and
+                          down-scaling, one axis unchanged).  The torch processor resamples with torchvision (absent
+                          here, different integer weights): its resampling is PARITY UNPINNED and not restated.
 """
 
 from __future__ import annotations
@@ -91,3 +100,67 @@ def patchify_frames(frames: np.ndarray, table: np.ndarray, patch: int = 14, merg
     x = chw.reshape(grid_t, temporal, C, grid_h // merge, merge, patch, grid_w // merge, merge, patch)
     x = x.transpose(0, 3, 6, 4, 7, 2, 1, 5, 8)
     return np.ascontiguousarray(x.reshape(grid_t * grid_h * grid_w, C * temporal * patch * patch)), (grid_t, grid_h, grid_w)
+
+
+PILLOW_PRECISION_BITS = 32 - 8 - 2
+
+
+def _cubic(x: float) -> float:
+    a = -0.5
+    if x < 0.0:
+        x = -x
+    if x < 1.0:
+        return ((a + 2.0) * x - (a + 3.0)) * x * x + 1
+    if x < 2.0:
+        return (((x - 5) * x + 8) * x - 4) * a
+    return 0.0
+
+
+def pillow_bicubic_taps(in_size: int, out_size: int) -> tuple[np.ndarray, np.ndarray]:
+    """(bounds int32 [out_size,2] = (first input position, count), taps int32 [out_size,ksize]) of one axis:
+    Resample.c `precompute_coeffs` (doubles, the box [0, in_size) held as floats) + `normalize_coeffs_8bpc`."""
+    scale = float(np.float32(in_size) - np.float32(0.0)) / out_size
+    filterscale = max(scale, 1.0)
+    support = 2.0 * filterscale
+    ksize = int(math.ceil(support)) * 2 + 1
+    taps = np.zeros((out_size, ksize), dtype=np.int32)
+    bounds = np.zeros((out_size, 2), dtype=np.int32)
+    inv = 1.0 / filterscale
+    for i in range(out_size):
+        center = 0.0 + (i + 0.5) * scale
+        first = max(int(center - support + 0.5), 0)
+        n = max(min(int(center + support + 0.5), in_size) - first, 0)
+        w = [_cubic((x + first - center + 0.5) * inv) for x in range(n)]
+        total = 0.0
+        for v in w:
+            total += v
+        for x, v in enumerate(w):
+            if total != 0.0:
+                v = v / total
+            taps[i, x] = int(-0.5 + v * (1 << PILLOW_PRECISION_BITS)) if v < 0 else int(0.5 + v * (1 << PILLOW_PRECISION_BITS))
+        bounds[i] = (first, n)
+    return bounds, taps
+
+
+def _pillow_pass(img: np.ndarray, out_size: int, axis: int) -> np.ndarray:
+    img = np.moveaxis(img, axis, 0)
+    bounds, taps = pillow_bicubic_taps(img.shape[0], out_size)
+    out = np.empty((out_size,) + img.shape[1:], dtype=np.uint8)
+    for i in range(out_size):
+        first, n = bounds[i]
+        acc = np.tensordot(taps[i, :n].astype(np.int64), img[first:first + n].astype(np.int64), axes=(0, 0))
+        acc = (acc + (1 << (PILLOW_PRECISION_BITS - 1))).astype(np.int32)   # the C code accumulates in INT32
+        out[i] = np.clip(acc >> PILLOW_PRECISION_BITS, 0, 255)
+    return np.moveaxis(out, 0, axis)
+
+
+def pillow_bicubic_resize(frames: np.ndarray, out_h: int, out_w: int) -> np.ndarray:
+    """uint8 [..., H, W, C] -> [..., out_h, out_w, C]: along x first, then along y, an unchanged axis skipped."""
+    frames = np.asarray(frames)
+    if frames.dtype != np.uint8 or frames.ndim < 3:
+        raise ValueError("frames must be uint8 [..., H, W, C]")
+    if frames.shape[-2] != out_w:
+        frames = _pillow_pass(frames, out_w, frames.ndim - 2)
+    if frames.shape[-3] != out_h:
+        frames = _pillow_pass(frames, out_h, frames.ndim - 3)
+    return frames

@@ -123,3 +123,23 @@ def test_attention_work_list_host():
         cover[q0 : q0 + nq] += 1
     assert (cover == 1).all()
     assert l.cs_attn_work_host(cu.ctypes.data, 3, 128, work.ctypes.data, 2, ctypes.byref(n)) == lib.CS_ERR_TOO_LARGE
+
+
+def test_resize_taps_host_matches_the_oracle_bit_for_bit():
+    """cs_resize_bicubic_taps_host is host arithmetic (doubles, then 22-bit fixed point): no GPU needed."""
+    from oracle import qwen_preprocess as qp
+
+    for a, b in [(4000, 1344), (3000, 1008), (100, 250), (37, 37), (5, 3), (3, 300), (1080, 1092), (299, 28), (1, 7), (7, 1),
+                 (9000, 28)]:
+        bounds, taps = ops.resize_bicubic_taps_host(a, b)
+        rb, rt = qp.pillow_bicubic_taps(a, b)
+        assert bounds.dtype == np.int32 and taps.dtype == np.int32
+        assert np.array_equal(bounds, rb) and np.array_equal(taps, rt), (a, b)
+    dll = lib.load()
+    k = ctypes.c_int32(0)
+    assert dll.cs_resize_bicubic_taps_host(0, 5, None, None, 0, ctypes.byref(k)) == lib.CS_ERR_INVALID_ARG
+    assert dll.cs_resize_bicubic_taps_host(10, 5, None, None, 0, ctypes.byref(k)) == 0 and k.value == 9
+    small = np.zeros((5, 4), dtype=np.int32)
+    b = np.zeros((5, 2), dtype=np.int32)
+    assert dll.cs_resize_bicubic_taps_host(10, 5, b.ctypes.data, small.ctypes.data, 4, ctypes.byref(k)) == lib.CS_ERR_INVALID_ARG
+    assert dll.cs_resize_u8_pass(None, 1, 4, 4, 3, None, None, 5, None, None) == lib.CS_ERR_INVALID_ARG

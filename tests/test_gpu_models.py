@@ -198,6 +198,33 @@ def test_qwen_uint8_frames_equal_float_pixel_values(dev):
         model(Modality.IMAGE, "", {"pixel_frames": [torch.zeros((1, 30, 28, 3), dtype=torch.uint8)]})
 
 
+def test_qwen_raw_frames_resized_on_the_gpu_equal_router_resized_frames(dev):
+    """Frames as decoded + the pixel budget (`resize_on="gpu"`) give the same embedding bits as frames the router
+    resized with the processor's CPU resampling: target size and bicubic resampling on the GPU are the processor's."""
+    from cornserve_amd.eric.models.qwen2_5_vl import FrameModalityProcessor
+
+    model, _, _ = build_qwen(dev, 2, (1,), seed=9)
+    rng = np.random.default_rng(9)
+    budget = dict(min_pixels=56 * 56, max_pixels=28 * 28 * 48)
+    on_router = FrameModalityProcessor("unused", **budget)
+    on_gpu = FrameModalityProcessor("unused", resize_on="gpu", **budget)
+    images = [np.clip(np.cumsum(rng.integers(-20, 21, (h, w, 3)), axis=1) + 128, 0, 255).astype(np.uint8)
+              for h, w in [(301, 517), (40, 33), (112, 84), (700, 90)]]   # shrunk, grown, kept, clamped by the budget
+
+    def collate(parts):
+        return {k: [p[k] for p in parts] for k in parts[0]}
+
+    ref = model(Modality.IMAGE, "", collate([on_router.process(Modality.IMAGE, im) for im in images]))
+    got = model(Modality.IMAGE, "", collate([on_gpu.process(Modality.IMAGE, im) for im in images]))
+    assert len(got) == len(ref) == 4 and all(torch.equal(a, b) for a, b in zip(got, ref))
+    video = np.stack([images[0], images[0][::-1], images[0][:, ::-1]])
+    ref = model(Modality.VIDEO, "", collate([on_router.process(Modality.VIDEO, video)]))
+    got = model(Modality.VIDEO, "", collate([on_gpu.process(Modality.VIDEO, video)]))
+    assert torch.equal(got[0], ref[0])
+    with pytest.raises(ValueError):
+        model(Modality.IMAGE, "", {"raw_frames": [torch.from_numpy(images[0])]})   # no budget
+
+
 def test_qwen_multi_image_ragged_and_video(dev):
     """Ragged image grids (window padding at non-multiple-of-8 edges) and a video (per-frame segments)."""
     model, sd, ocfg = build_qwen(dev, 3, (1,), seed=2)

@@ -151,6 +151,50 @@ def test_attn_rotary_in_place_route_equals_fused_route(ops, dev, heads, d):
     assert torch.equal(got, ref) and torch.equal(buf, qkv[:320])
 
 
+def test_resize_bicubic_u8_bit_exact(ops, dev):
+    """GPU resize against the oracle's restatement of Pillow's bicubic (itself pinned against the package on the CPU)
+    and, where the package is importable, against the package directly: random, black/white (clamping) and smooth
+    frames; up- and down-scaling; one axis unchanged; both axes unchanged (returned as is); rows whose byte count is
+    not a multiple of 4 (the byte-wise form of the pass); frames that do not start at a 4-byte boundary."""
+    from oracle import qwen_preprocess as qp
+
+    rng = np.random.default_rng(3)
+    cases = [(1, 97, 64, 56, 140), (2, 600, 450, 196, 140), (1, 30, 45, 112, 168), (3, 37, 53, 37, 84), (1, 64, 64, 28, 64),
+             (1, 33, 35, 31, 29), (1, 1080, 1920, 588, 1036), (1, 5, 7, 56, 56), (1, 1500, 20, 28, 28)]
+    for i, (t, h, w, oh, ow) in enumerate(cases):
+        if i % 3 == 1:
+            frames = (rng.integers(0, 2, (t, h, w, 3)) * 255).astype(np.uint8)
+        elif i % 3 == 2:
+            frames = np.clip(np.cumsum(rng.integers(-9, 10, (t, h, w, 3)), axis=2) + 128, 0, 255).astype(np.uint8)
+        else:
+            frames = rng.integers(0, 256, (t, h, w, 3), dtype=np.uint8)
+        ref = qp.pillow_bicubic_resize(frames, oh, ow)
+        got = ops.resize_bicubic_u8(torch.from_numpy(frames).to(dev), oh, ow)
+        assert got.shape == (t, oh, ow, 3) and got.dtype == torch.uint8
+        assert np.array_equal(got.cpu().numpy(), ref), (t, h, w, oh, ow)
+    try:
+        from PIL import Image
+    except ImportError:
+        Image = None
+    frames = rng.integers(0, 256, (1, 301, 517, 3), dtype=np.uint8)
+    dbuf = torch.empty((frames.size + 3,), dtype=torch.uint8, device=dev)
+    dbuf[3:] = torch.from_numpy(frames).to(dev).reshape(-1)
+    got = ops.resize_bicubic_u8(dbuf[3:].view(1, 301, 517, 3), 308, 504).cpu().numpy()
+    assert np.array_equal(got, qp.pillow_bicubic_resize(frames, 308, 504))
+    if Image is not None:
+        assert np.array_equal(got[0], np.asarray(Image.fromarray(frames[0]).resize((504, 308), resample=Image.Resampling.BICUBIC)))
+    same = torch.from_numpy(frames).to(dev)
+    assert ops.resize_bicubic_u8(same, 301, 517) is same
+    grey = torch.from_numpy(frames[..., :1].copy()).to(dev)   # one channel: the pass takes any inner size
+    assert np.array_equal(ops.resize_bicubic_u8(grey, 100, 90).cpu().numpy(), qp.pillow_bicubic_resize(frames[..., :1], 100, 90))
+    with pytest.raises(ValueError):
+        ops.resize_bicubic_u8(same[0], 28, 28)
+    with pytest.raises(ValueError):
+        ops.resize_bicubic_u8(same, 0, 28)
+    with pytest.raises(ValueError):
+        ops.resize_bicubic_u8(same.float(), 28, 28)
+
+
 @pytest.mark.parametrize("patch", [14, 16])
 def test_qwen_patchify_u8_unaligned_frames(ops, dev, patch):
     """Frames that start at any byte offset of a 4-byte word (a view into a larger buffer), last frame at the very end

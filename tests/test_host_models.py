@@ -111,6 +111,16 @@ def test_frame_processor_resize_and_table_match_the_hf_pil_processor():
         px, grid = qp.patchify_frames(out.numpy(), table)
         assert grid == tuple(ref["image_grid_thw"][0]) and np.array_equal(px, ref["pixel_values"])
     assert np.array_equal(fr.byte_table(arithmetic="fused").numpy(), qp.normalization_table(arithmetic="fused"))
+    raw = FrameModalityProcessor("unused", min_pixels=3136, max_pixels=200704, resize_on="gpu")
+    img = rng.integers(0, 256, (301, 517, 3), dtype=np.uint8)
+    out = raw.process(Modality.IMAGE, img)
+    assert torch.equal(out["raw_frames"], torch.from_numpy(img[None])) and out["raw_frames_budget"].tolist() == [3136, 200704]
+    out = raw.process(Modality.VIDEO, np.stack([img, img]))
+    assert out["raw_frames_videos"].shape == (2, 301, 517, 3)
+    with pytest.raises(ValueError):
+        raw.process(Modality.IMAGE, np.zeros((1, 500, 3), np.uint8))   # aspect ratio beyond the processor's limit
+    with pytest.raises(ValueError):
+        FrameModalityProcessor("unused", resize_on="host")
     with pytest.raises(ValueError):
         fr.resize_frames(np.zeros((4, 4), np.uint8))
     with pytest.raises(ValueError):

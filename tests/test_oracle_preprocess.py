@@ -143,3 +143,44 @@ def test_rejects_bad_input():
         qp.patchify_frames(np.zeros((1, 30, 28, 3), np.uint8), qp.normalization_table())
     with pytest.raises(ValueError):
         qp.patchify_frames(np.zeros((1, 28, 28, 3), np.float32), qp.normalization_table())
+
+
+def _test_image(kind, h, w, rng):
+    if kind == 0:
+        return rng.integers(0, 256, (h, w, 3), dtype=np.uint8)
+    if kind == 1:   # black / white only: the negative lobes overshoot and the clamp at 0 and 255 is exercised
+        return (rng.integers(0, 2, (h, w, 3)) * 255).astype(np.uint8)
+    return np.clip(np.cumsum(rng.integers(-9, 10, (h, w, 3)), axis=1) + 128, 0, 255).astype(np.uint8)   # smooth
+
+
+def test_pillow_bicubic_resize_matches_the_package_bit_for_bit():
+    Image = pytest.importorskip("PIL.Image")
+    rng = np.random.default_rng(11)
+    sizes = [tuple(int(v) for v in rng.integers(3, 200, 4)) for _ in range(24)]
+    sizes += [(97, 64, 97, 140), (97, 64, 28, 64), (40, 40, 40, 40), (600, 450, 196, 140), (30, 45, 112, 168), (2, 2, 56, 56)]
+    for i, (h, w, oh, ow) in enumerate(sizes):
+        img = _test_image(i % 3, h, w, rng)
+        ref = np.asarray(Image.fromarray(img).resize((ow, oh), resample=Image.Resampling.BICUBIC))
+        got = qp.pillow_bicubic_resize(img, oh, ow)
+        assert got.shape == ref.shape and np.array_equal(got, ref), (h, w, oh, ow)
+    video = _test_image(0, 3 * 50, 70, rng).reshape(3, 50, 70, 3)
+    got = qp.pillow_bicubic_resize(video, 84, 112)
+    for f, g in zip(video, got):
+        assert np.array_equal(g, np.asarray(Image.fromarray(f).resize((112, 84), resample=Image.Resampling.BICUBIC)))
+
+
+def test_pillow_bicubic_taps_properties():
+    """What the construction fixes whatever the package: taps of a position sum to 2^22 within rounding, a pass over a
+    constant image returns the constant, and the same size in and out is the identity (centre tap 2^22, others 0)."""
+    for a, b in [(100, 37), (37, 100), (1000, 28), (5, 5), (3, 300)]:
+        bounds, taps = qp.pillow_bicubic_taps(a, b)
+        assert taps.shape[1] == int(np.ceil(2.0 * max(a / b, 1.0))) * 2 + 1
+        assert np.all(np.abs(taps.sum(axis=1) - (1 << 22)) <= taps.shape[1])
+        assert np.all(bounds[:, 0] >= 0) and np.all(bounds[:, 0] + bounds[:, 1] <= a) and np.all(bounds[:, 1] > 0)
+    bounds, taps = qp.pillow_bicubic_taps(5, 5)
+    for i in range(5):
+        row = np.zeros(5, dtype=np.int64)
+        row[bounds[i, 0]:bounds[i, 0] + bounds[i, 1]] = taps[i, :bounds[i, 1]]
+        assert row[i] == 1 << 22 and row.sum() == 1 << 22
+    flat = np.full((9, 13, 3), 201, dtype=np.uint8)
+    assert np.all(qp.pillow_bicubic_resize(flat, 31, 5) == 201)
