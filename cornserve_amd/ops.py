@@ -733,15 +733,20 @@ def resize_bicubic_u8(frames: torch.Tensor, out_h: int, out_w: int) -> torch.Ten
     todo = [(axis, a, b) for axis, a, b in ((2, W, out_w), (1, H, out_h)) if a != b]
     if not todo:
         return frames
-    host = [t for _, a, b in todo for t in resize_bicubic_taps_host(a, b)]
-    dev = host_to_device_packed(list(host), frames.device)
-    for i, (axis, a, b) in enumerate(todo):
+    for axis, a, b in todo:
+        bounds, taps = _resize_taps_device(a, b, frames.device)
         shape = list(frames.shape)
         shape[axis] = b
         out = torch.empty(shape, dtype=torch.uint8, device=frames.device)
-        torch.ops.cornserve_amd.resize_u8_pass_(out, frames, dev[2 * i], dev[2 * i + 1], axis)
+        torch.ops.cornserve_amd.resize_u8_pass_(out, frames, bounds, taps, axis)
         frames = out
     return frames
+
+
+@functools.lru_cache(maxsize=256)
+def _resize_taps_device(in_size: int, out_size: int, device: torch.device) -> list[torch.Tensor]:
+    """The taps of one axis on the device, kept for the next frame of the same size (a few KB per size pair)."""
+    return host_to_device_packed(list(resize_bicubic_taps_host(in_size, out_size)), device)
 
 
 def _resize_u8_pass_impl(out, src, bounds, taps, axis) -> None:

@@ -155,12 +155,15 @@ def test_resize_bicubic_u8_bit_exact(ops, dev):
     """GPU resize against the oracle's restatement of Pillow's bicubic (itself pinned against the package on the CPU)
     and, where the package is importable, against the package directly: random, black/white (clamping) and smooth
     frames; up- and down-scaling; one axis unchanged; both axes unchanged (returned as is); rows whose byte count is
-    not a multiple of 4 (the byte-wise form of the pass); frames that do not start at a 4-byte boundary."""
+    not a multiple of 4 (the byte-wise form of the pass); frames that do not start at a 4-byte boundary; along x every
+    tap-count class of the staged kernel, several tiles of 256 positions, row groups with a remainder, and windows too
+    wide for it (the general kernel)."""
     from oracle import qwen_preprocess as qp
 
     rng = np.random.default_rng(3)
     cases = [(1, 97, 64, 56, 140), (2, 600, 450, 196, 140), (1, 30, 45, 112, 168), (3, 37, 53, 37, 84), (1, 64, 64, 28, 64),
-             (1, 33, 35, 31, 29), (1, 1080, 1920, 588, 1036), (1, 5, 7, 56, 56), (1, 1500, 20, 28, 28)]
+             (1, 33, 35, 31, 29), (1, 1080, 1920, 588, 1036), (1, 5, 7, 56, 56), (1, 1500, 20, 28, 28), (2, 40, 2100, 56, 28),
+             (1, 19, 3000, 28, 420), (17, 50, 1300, 28, 300), (1, 64, 300, 64, 1100)]
     for i, (t, h, w, oh, ow) in enumerate(cases):
         if i % 3 == 1:
             frames = (rng.integers(0, 2, (t, h, w, 3)) * 255).astype(np.uint8)
