@@ -291,6 +291,25 @@ def hbm_kernels(dev, rows_list=(8192, 131072), reps: int = 20) -> dict:
         put("patchify_nchw (384x384 tiles, patch 14)", tiles * 3 * 378 * 378 * 2 + tiles * 729 * 592 * 2,
             lambda: ops.patchify_nchw(pxl, 14, 592))
         out[f"rows_{L}"] = res
+    # the processor's bicubic resize, pass by pass (x first, then y, as Pillow orders them), at the default pixel budget
+    from cornserve_amd.eric import frames as fr
+
+    res = {}
+    for name, shape in [("photo 1x3000x4000", (1, 3000, 4000, 3)), ("video 16x1080x1920", (16, 1080, 1920, 3)),
+                        ("frame 1x720x1280", (1, 720, 1280, 3))]:
+        f = torch.randint(0, 256, shape, dtype=torch.uint8).to(dev)
+        T, H, W, _ = shape
+        h, w = fr.target_size(H, W)
+        mid = torch.empty((T, H, w, 3), dtype=torch.uint8, device=dev)
+        fin = torch.empty((T, h, w, 3), dtype=torch.uint8, device=dev)
+        bx, tx = ops.host_to_device_packed(list(ops.resize_bicubic_taps_host(W, w)), dev)
+        by, ty = ops.host_to_device_packed(list(ops.resize_bicubic_taps_host(H, h)), dev)
+        for axis, src, dst, b, t in ((2, f, mid, bx, tx), (1, mid, fin, by, ty)):
+            dt = timed(lambda: torch.ops.cornserve_amd.resize_u8_pass_(dst, src, b, t, axis))
+            nbytes = src.numel() + dst.numel()
+            res[f"{name} -> {h}x{w}, pass along {'x' if axis == 2 else 'y'} ({t.shape[1]} taps)"] = {
+                "us": round(dt * 1e6, 2), "GB_per_s": round(nbytes / dt / 1e9, 1), "bytes": int(nbytes)}
+    out["resize_bicubic_u8"] = res
     return {"metric": "achieved GB/s of the HBM-bound kernels on 1 MI355X", "unit": "GB/s", "n_gpus": 1, "peak_GB_per_s": 8000,
             "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "hidden 1280, 16 heads of 80 (config 2's shapes); merged rows of 3584 for the row mixes"},
