@@ -310,6 +310,13 @@ def hbm_kernels(dev, rows_list=(8192, 131072), reps: int = 20) -> dict:
             res[f"{name} -> {h}x{w}, pass along {'x' if axis == 2 else 'y'} ({t.shape[1]} taps)"] = {
                 "us": round(dt * 1e6, 2), "GB_per_s": round(nbytes / dt / 1e9, 1), "bytes": int(nbytes)}
     out["resize_bicubic_u8"] = res
+    # a copy of known size at the end: what a counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) of this workload
+    # reads for 1 GiB read + 1 GiB written scales the counters of the kernels above
+    cal = torch.zeros(256 * 1024 * 1024, dtype=torch.int32, device=dev)
+    for _ in range(3):
+        cal2 = cal.clone()
+    torch.cuda.synchronize()
+    del cal, cal2
     return {"metric": "achieved GB/s of the HBM-bound kernels on 1 MI355X", "unit": "GB/s", "n_gpus": 1, "peak_GB_per_s": 8000,
             "higher_is_better": True, "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "hidden 1280, 16 heads of 80 (config 2's shapes); merged rows of 3584 for the row mixes"},

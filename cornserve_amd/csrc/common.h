@@ -90,6 +90,14 @@ CS_DEVICE float wave_max(float v) {
   return v;
 }
 
+// Workgroup b of a launch runs on XCD b mod 8, and every XCD has an L2 of its own.  This maps the launch index to a work
+// index (a bijection on 0..n-1) that gives every XCD one contiguous eighth of the work, so that work items that read
+// the same cache lines (neighbouring rows, neighbouring patches) meet in one L2 instead of fetching the lines eight times.
+CS_DEVICE unsigned xcd_contiguous(unsigned b, unsigned n) {
+  const unsigned k = b & 7u, q = n >> 3, r = n & 7u;
+  return k * q + min(k, r) + (b >> 3);
+}
+
 // Last launch error -> status code. Never aborts the process.
 static inline int cs_launch_status() {
   hipError_t e = hipGetLastError();

@@ -21,7 +21,7 @@ __global__ __launch_bounds__(256) void patchify_kernel(const bf16_t* __restrict_
   extern __shared__ bf16x2_t band[];   // [C*p][n*p/2] pixel pairs
   const int p = P ? P : p_any;
   const int hp = p >> 1;
-  unsigned wg = blockIdx.x;            // -> (image, patch row, run of patches)
+  unsigned wg = xcd_contiguous(blockIdx.x, gridDim.x);   // -> (image, patch row, run of patches); neighbours share an L2
   const int ch = wg % (unsigned)chunks;
   wg /= (unsigned)chunks;
   const int y = wg % (unsigned)gh, b = wg / (unsigned)gh;
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(256) void qwen_patchify_u8_kernel(const uint8_t* __
   const int pairs = 3 * tps * p * hp;
   // where each of this workgroup's rows sits in the frame: (first frame of the group, top pixel row, left pixel column)
   __shared__ int where[QP_ROWS][3];
-  const int row0 = blockIdx.x * QP_ROWS;
+  const int row0 = (int)xcd_contiguous(blockIdx.x, gridDim.x) * QP_ROWS;   // neighbouring rows share an L2
   const int n_rows = min(rows - row0, QP_ROWS);
   if (threadIdx.x < n_rows) {
     const int bw = W / (p * m), bh = H / (p * m);
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void qwen_patchify_u8_seg_kernel(const uint8_t
   __shared__ int where[ROWS][3];
   extern __shared__ __attribute__((aligned(16))) char dyn[];   // int64 segment offsets, then NDW words per segment
   for (int i = threadIdx.x; i < 3 * 256; i += 256) lut[i] = table[i];
-  const int row0 = blockIdx.x * ROWS;
+  const int row0 = (int)xcd_contiguous(blockIdx.x, gridDim.x) * ROWS;   // neighbouring rows (patches of one image row) share an L2
   const int n_rows = min(rows - row0, ROWS);
   if (threadIdx.x < n_rows) {
     const int bw = W / (P * m), bh = H / (P * m);

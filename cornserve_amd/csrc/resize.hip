@@ -88,7 +88,11 @@ __global__ __launch_bounds__(256) void resample_rows_kernel(const uint8_t* __res
                                                             int inner_w, int chunks, const int32_t* __restrict__ bounds,
                                                             const int32_t* __restrict__ taps, int ksize,
                                                             uint8_t* __restrict__ dst) {
-  const unsigned chunk = blockIdx.x % (unsigned)chunks, row = blockIdx.x / (unsigned)chunks;   // row = outer * out_size + pos
+  // work index -> (1024-byte column of the image, output row), rows fastest, a contiguous eighth of it per XCD: the
+  // workgroups that read the same input rows (neighbouring output rows of one column) share an L2
+  const unsigned v = xcd_contiguous(blockIdx.x, gridDim.x);
+  const unsigned n_rows = gridDim.x / (unsigned)chunks;   // outer * out_size
+  const unsigned chunk = v / n_rows, row = v % n_rows;
   const unsigned pos = row % (unsigned)out_size, outer = row / (unsigned)out_size;
   const int iw = (int)chunk * 256 + threadIdx.x;   // word of the row
   if (iw >= inner_w) return;
