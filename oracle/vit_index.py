@@ -8,8 +8,8 @@ A numpy restatement, step for step, of the reference's index code:
 * `full_cu_seqlens`       follows :445-448 (one segment per frame);
 * `rope_angles`           follows Qwen2_5_VisionRotaryEmbedding :236-259 and :352-354.
 
-Pinned by tests/test_oracle_index.py: the worked values the survey records (grid (1,32,32) and
-(8,24,42)), the independent closed form, permutation/monotonicity invariants on every even grid up to
+Pinned by tests/test_oracle_index.py: hand-worked values for two grids ((1,32,32): 16 windows of 64; and
+(8,24,42): 288 segments of 16 to 64), the independent closed form, permutation/monotonicity invariants on every even grid up to
 28x28 with t <= 3, the committed fixtures in tests/golden/index_*.json (written from the installed
 third-party `transformers.vision_utils`, which carries the same algorithm), and, when `transformers`
 is importable, a live comparison against it.
