@@ -62,6 +62,10 @@ constexpr int CS_EPI_BIAS_POS = 100;  // internal: CS_EPI_BIAS plus the (row % p
 // internal: the QKV projection of one head per column tile with rotary and window attention as its epilogue (see
 // cs_qkv_window_attn): the tile's 256 columns are the head's q (5 fragments), k (5), v (5) and one all-zero fragment
 constexpr int CS_EPI_QKV_WATTN = 101;
+// internal: the same with windows of 4 .. 64 rows, each in a 64-row slot of its own: the tile's rows are VIRTUAL rows,
+// slot v/64, place v%64; place >= the window's row count repeats the window's last row (operand loads), is masked
+// (keys) or not stored (queries)
+constexpr int CS_EPI_QKV_WATTN_RAGGED = 102;
 constexpr int NW = 4;                 // waves per workgroup, one per SIMD
 constexpr int LDS_BYTES = 160 * 1024;
 
@@ -162,6 +166,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   static_assert(WAVES_M * WAVES_N == NW, "four waves, one per SIMD");
   using Ring = RingShape<BM, BN, W_FP8>;
+  constexpr bool WATTN = EPI == CS_EPI_QKV_WATTN || EPI == CS_EPI_QKV_WATTN_RAGGED, RAGGED = EPI == CS_EPI_QKV_WATTN_RAGGED;
   constexpr int A_BYTES = Ring::A_BYTES, W_BYTES = Ring::W_BYTES;
   constexpr bool RING5 = Ring::FIVE_UNITS;
   // Byte offsets of operand tile slots.  Three-stage ring: slot s holds A at s*STAGE and W behind it.
@@ -236,7 +241,17 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     for (int j = 0; j < A_LD; ++j) {
       const int row = (j * NW + wave) * 8 + l_row;  // tile-local
       const int key = (row >> 1) & 7;
-      const int r = min(m0 + row, p.M - 1);
+      int r;
+      if constexpr (RAGGED) {
+        // the 8 rows of this load lie in one slot (8 divides 64): slot, start and count are wave-uniform
+        const int v0 = m0 + (j * NW + wave) * 8;
+        const int slot = min(v0 >> 6, p.attn_n_win - 1);
+        const int start = p.attn_win_start[slot];
+        const int cnt = min(max(p.attn_win_start[slot + 1] - start, 1), 64);
+        r = start + min((v0 & 63) + l_row, cnt - 1);
+      } else {
+        r = min(m0 + row, p.M - 1);
+      }
       a_src[j] = (uint32_t)(((int64_t)r * p.lda + ((l_slot ^ key) << 3)) * 2);
     }
 #pragma unroll
@@ -352,7 +367,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       // compiler pads that for its own MFMAs but cannot see into these.  Only the first MFMA after a
       // conversion can be that close.
       if constexpr (W_FP8 && I == 0) asm volatile("s_nop 3");
-      if constexpr (EPI == CS_EPI_QKV_WATTN && J >= 10) {
+      if constexpr (WATTN && J >= 10) {
         // The V fragments are computed TRANSPOSED (activation rows as the first operand): a lane then owns one
         // head dim and four consecutive keys, the operand layout of the P.V product.  Fragment 15 is padding.
         if constexpr (J < 15) {
@@ -588,7 +603,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     //      S^T's accumulators hold four consecutive keys per lane, the layout of the second product's operand, and
     //      the transposed V fragments hold four consecutive keys per head dim: O^T = V^T.P^T needs no transposition.
     auto wattn_epilogue = [&](auto) {   // (generic: only instantiated for the kernel that calls it)
-      static_assert(EPI != CS_EPI_QKV_WATTN || (BM == 256 && BN == 256 && WAVES_M == 4 && WAVES_N == 1 && !W_FP8),
+      static_assert(!WATTN || (BM == 256 && BN == 256 && WAVES_M == 4 && WAVES_N == 1 && !W_FP8),
                     "one 64-row window per wave, one head per column tile");
       constexpr int HD = 80, HALF = 40;
       // A register written by a vector instruction must not be read by an MFMA in the next few cycles.  The compiler
@@ -608,8 +623,16 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       auto lane_xchg = [](float v, int byte_addr) {
         return __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute(byte_addr, __builtin_bit_cast(int, v)));
       };
-      const int row0 = m0 + wm * 64;                 // first row of this wave's window
+      // first row and row count of this wave's window (RAGGED: the window of slot (m0 + 64 wm) / 64)
+      int row0 = m0 + wm * 64, cnt = 64;
       if (row0 >= p.M) return;                       // (no barrier below: waves may leave independently)
+      if constexpr (RAGGED) {
+        const int slot = row0 >> 6;
+        row0 = p.attn_win_start[slot];
+        cnt = min(max(p.attn_win_start[slot + 1] - row0, 1), 64);
+      }
+      // row of the window at place `local` (rows past the window's last repeat it: finite values that are never used)
+      auto row_at = [&](int local) { return RAGGED ? row0 + min(local, cnt - 1) : row0 + local; };
       const int head = n0 / BN;
       const bf16_t* const pBias = (const bf16_t*)p.bias + n0;
       const float sl2 = p.attn_scale_log2e;
@@ -619,7 +642,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       for (int I = 0; I < 4; ++I) {
         rstd[I] = 1.0f;
         if constexpr (NORM_A) {
-          const float* parts = p.a_row_sumsq + (int64_t)(row0 + 16 * I + lr) * CS_SUMSQ_PARTS;
+          const float* parts = p.a_row_sumsq + (int64_t)row_at(16 * I + lr) * CS_SUMSQ_PARTS;
           const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
           const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
           rstd[I] = rsqrtf(ss / (float)p.K + p.norm_eps);
@@ -634,7 +657,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       // q and k: scale, bias, rotary (fp32, one rounding), packed as operands
       static_for<4>([&](auto i_c) {
         constexpr int I = decltype(i_c)::value;
-        const float* cs = p.attn_cos_sin + (int64_t)(row0 + 16 * I + lr) * HD + 10 * kq;
+        const float* cs = p.attn_cos_sin + (int64_t)row_at(16 * I + lr) * HD + 10 * kq;
         float co[10], si[10];
 #pragma unroll
         for (int t = 0; t < 10; t += 2) {   // 8-byte aligned: 40 kq bytes into a 320-byte row
@@ -706,7 +729,9 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
           constexpr int E = decltype(e_c)::value, KB = E / 4, R = s_reg(KB * 4 + QB) + E % 4;
           float t;
           asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R));
-          sv[E] = t;
+          // (a lane's four keys of a block are keys 16 KB + 4 kq .. + 3, and a window's row count is a multiple of 4)
+          if constexpr (RAGGED) sv[E] = 16 * KB + 4 * kq < cnt ? t : -__builtin_inff();
+          else sv[E] = t;
         });
         float mx = sv[0];
 #pragma unroll
@@ -739,7 +764,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         for (int I = 0; I < 4; ++I) {
           float rs = 1.0f;
           if constexpr (NORM_A) {
-            const float* parts = p.a_row_sumsq + (int64_t)(row0 + 16 * I + lrv) * CS_SUMSQ_PARTS;
+            const float* parts = p.a_row_sumsq + (int64_t)row_at(16 * I + lrv) * CS_SUMSQ_PARTS;
             const f32x4_t s0 = *(const f32x4_t*)parts, s1 = *(const f32x4_t*)(parts + 4);
             const float ss = ((s0[0] + s0[1]) + (s0[2] + s0[3])) + ((s1[0] + s1[1]) + (s1[2] + s1[3]));
             rs = rsqrtf(ss / (float)p.K + p.norm_eps);
@@ -807,7 +832,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
             asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R + Rr));
             o[Rr] = f2bf(t * inv);
           });
-          *(bf16x4_t*)(out0 + (int64_t)(16 * QB) * p.ldc + 16 * Dd) = o;
+          if (!RAGGED || 16 * QB + lr < cnt) *(bf16x4_t*)(out0 + (int64_t)(16 * QB) * p.ldc + 16 * Dd) = o;
         });
       });
     };
@@ -1231,7 +1256,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       });
     };
     // (p.fast_epilogue: the host has checked that every matrix the epilogue touches lies within 32-bit byte offsets)
-    if constexpr (EPI == CS_EPI_QKV_WATTN) {
+    if constexpr (WATTN) {
       wattn_epilogue(0);
       // the next tile's source offsets and the fragment offsets are recomputed rather than kept in registers across
       // this epilogue (the lane number comes from the hardware again, not from a register held since the start)

@@ -262,17 +262,20 @@ class QwenVisionBase(EricModel):
 
 class Qwen2_5_VisionTransformer(QwenVisionBase):
     def __init__(self, config: Any, weight_format: str = "bf16", fold_norm: bool = True,
-                 split_residual: bool = True, fuse_window_attn: bool = True, fuse_min_rows: int = 0) -> None:
+                 split_residual: bool = True, fuse_window_attn: bool = True, fuse_min_rows: int = 0,
+                 fuse_min_fill: float = 0.75) -> None:
         """`fuse_window_attn`: run qkv projection + rotary + window attention of a block (:93-120) as ONE launch
-        (`ops.qkv_window_attn`: q, k and v stay in registers, the [L, 3*hidden] tensor is never written) for every ITEM
-        whose windows are all full 64-row windows -- images and videos with sides that are multiples of 8 patches.  Other
-        items of the same batch, fp8 weights and head dims other than 80 take the separate kernels.  The one launch
-        rounds q and k to bf16 once (after the rotation) instead of twice, so the two routes agree within the parity
-        tolerance, not bit for bit; since the route depends on the item alone, an item's embedding is the same bits
-        whatever it is batched with (setting the attribute to False afterwards selects the separate kernels for every
-        item).  `fuse_min_rows` > 0 is a deployment knob that gives this up for latency: a batch with fewer one-launch
-        rows than that takes the separate kernels throughout, whose GEMM has narrower tiles for few rows (one
-        1024-patch image alone: 3.99 against 4.28 ms; 3072 is where the one launch starts to pay).
+        (`ops.qkv_window_attn`: q, k and v stay in registers, the [L, 3*hidden] tensor is never written).  Every window
+        takes a 64-row slot of that launch, so an ITEM takes it when its windows fill their slots to `fuse_min_fill` or
+        more on average (an image whose sides are multiples of 8 patches fills them completely; edge windows of other
+        sizes are shorter, and a slot's empty rows cost the projection as much as full ones: below about 0.75 the
+        separate kernels are cheaper).  Other items of the same batch, fp8 weights and head dims other than 80 take the
+        separate kernels.  The one launch rounds q and k to bf16 once (after the rotation) instead of twice, so the two
+        routes agree within the parity tolerance, not bit for bit; since the route depends on the item alone, an item's
+        embedding is the same bits whatever it is batched with (setting the attribute to False afterwards selects the
+        separate kernels for every item).  `fuse_min_rows` > 0 is a deployment knob that gives this up for latency: a
+        batch with fewer one-launch rows than that takes the separate kernels throughout, whose GEMM has narrower tiles
+        for few rows (one 1024-patch image alone: 3.99 against 4.28 ms; 3072 is where the one launch starts to pay).
 
         `split_residual`: carry the residual stream (:175,177) with 16 significant bits -- the bf16 tensor every
         kernel reads plus a byte plane with the next 8 mantissa bits, joined and re-split inside the two residual GEMMs
@@ -293,6 +296,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         self.weight_format = weight_format
         self.split_residual = bool(split_residual)
         self.fuse_min_rows = int(fuse_min_rows)
+        self.fuse_min_fill = float(fuse_min_fill)
         self.hidden_size = vc.hidden_size
         self.out_hidden_size = vc.out_hidden_size
         self.num_heads = vc.num_heads
@@ -387,12 +391,13 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         (reference: rot_pos_emb :325-355, get_window_index :357-386, cu_seqlens :445-448), and the route of every item
         through the window blocks.
 
-        An item whose windows are all whole (both sides multiples of the window, i.e. of 8 patches) takes the one-launch
-        form of qkv + rotary + window attention, every other item the separate kernels.  The choice depends on the item
-        alone, so an item's embedding does not depend on what it is batched with.  The items are PROCESSED with the
-        one-launch items first (a stable reordering: their rows are then one leading block of the batch); the index
-        kernel takes each item's place in the caller's patch matrix separately from its place in the processing
-        order, and `order` maps processing position to the caller's item number."""
+        An item whose windows fill their 64-row slots well enough (`fuse_min_fill`; whole windows fill them completely)
+        takes the one-launch form of qkv + rotary + window attention, every other item the separate kernels.  The choice
+        depends on the item alone, so an item's embedding does not depend on what it is batched with.  The items are
+        PROCESSED with the one-launch items first (a stable reordering: their rows are then one leading block of the
+        batch); the index kernel takes each item's place in the caller's patch matrix separately from its place in the
+        processing order, and `order` maps processing position to the caller's item number.  `win_start` is None when
+        every one-launch window has 64 rows, else the starts of those windows on the device."""
         merge = self.spatial_merge_size
         win = self.window_size // merge // self.patch_size
         dev = self.device
@@ -400,14 +405,15 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         n = g.shape[0]
         units = g[:, 0] * (g[:, 1] // merge) * (g[:, 2] // merge)
         if self.fuse_window_attn and n:
-            whole = ((g[:, 1] // merge) % win == 0) & ((g[:, 2] // merge) % win == 0)
+            slots = g[:, 0] * -(-(g[:, 1] // merge) // win) * -(-(g[:, 2] // merge) // win)   # windows of the item
+            one_launch = units >= self.fuse_min_fill * slots * (win * win)
         else:
-            whole = np.zeros(n, dtype=bool)
-        fused_rows = int(units[whole].sum()) * merge * merge
+            one_launch = np.zeros(n, dtype=bool)
+        fused_rows = int(units[one_launch].sum()) * merge * merge
         if fused_rows < self.fuse_min_rows:
-            whole[:] = False
+            one_launch[:] = False
             fused_rows = 0
-        order = np.concatenate([np.flatnonzero(whole), np.flatnonzero(~whole)]) if n else np.zeros(0, np.int64)
+        order = np.concatenate([np.flatnonzero(one_launch), np.flatnonzero(~one_launch)]) if n else np.zeros(0, np.int64)
         sl = ops.vit_seqlens_host(g[order], merge, win)
         if n:
             caller_unit_base = np.concatenate([[0], np.cumsum(units)[:-1]])
@@ -416,11 +422,14 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         first_sep = int(np.searchsorted(sl.cu_window, fused_rows))
         work_win, max_win = ops.attn_work_host(sl.cu_window[first_sep:])
         work_full, max_full = ops.attn_work_host(sl.cu_full)
-        # one host-to-device copy for the three small arrays
-        meta, dwin, dfull = ops.host_to_device_packed([sl.item_meta, work_win, work_full], dev)
+        # the one-launch windows' starts, when any of them is short of 64 rows
+        cu_fused = np.ascontiguousarray(sl.cu_window[:first_sep + 1], dtype=np.int32)
+        ragged = bool(first_sep) and bool(np.any(np.diff(cu_fused) != ops.QKV_WATTN_WINDOW))
+        # one host-to-device copy for the small arrays
+        meta, dwin, dfull, dcu = ops.host_to_device_packed([sl.item_meta, work_win, work_full, cu_fused], dev)
         ix = ops.vit_index(meta, sl.total_patches, sl.max_units_per_item, merge, win, self._ensure_packed()["inv_freq"])
         return (ix, ops.AttnPlan(dwin, work_win.shape[0], max_win), ops.AttnPlan(dfull, work_full.shape[0], max_full),
-                sl.total_patches, fused_rows, order)
+                sl.total_patches, fused_rows, order, dcu if ragged else None)
 
     def forward_device(self, pixel_values: torch.Tensor, grid_thw: np.ndarray, mark=None) -> list[torch.Tensor]:
         """pixel_values: bf16 [L, C*T*P*P] already on the device; grid_thw: host int64 [n,3].
@@ -442,7 +451,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
             if len(groups) > 1:
                 return self._forward_in_groups(pixel_values, grid_thw, groups, mark)
         mark("index")
-        ix, plan_win, plan_full, L, fused_rows, order = self._index(grid_thw)
+        ix, plan_win, plan_full, L, fused_rows, order, win_start = self._index(grid_thw)
         if pixel_values.shape[0] != L:
             raise ValueError(f"pixel_values has {pixel_values.shape[0]} rows but grid_thw describes {L} patches")
 
@@ -471,12 +480,13 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 if fold:
                     mark("gemm_qkv_attn_window")
                     ops.qkv_window_attn(xf, wp, bp, ix.cos_sin[:fused_rows], nh, scale, a_row_sumsq=ss[:fused_rows], norm_eps=eps,
-                                        out=att[:fused_rows])
+                                        out=att[:fused_rows], win_start=win_start)
                 else:
                     mark("norm")
                     ops.rmsnorm(xf, b["n1"], eps, out=n[:fused_rows])
                     mark("gemm_qkv_attn_window")
-                    ops.qkv_window_attn(n[:fused_rows], wp, bp, ix.cos_sin[:fused_rows], nh, scale, out=att[:fused_rows])
+                    ops.qkv_window_attn(n[:fused_rows], wp, bp, ix.cos_sin[:fused_rows], nh, scale, out=att[:fused_rows],
+                                        win_start=win_start)
             if full or fused_rows < L:
                 lo = 0 if full else fused_rows           # first row the separate kernels work on in this block
                 if fold:

@@ -17,7 +17,7 @@ CS_ERR_INVALID_ARG = 1
 CS_ERR_UNSUPPORTED = 2
 CS_ERR_LAUNCH = 3
 CS_ERR_TOO_LARGE = 4
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH, EPI_QUICK_GELU = range(6)
 
@@ -63,6 +63,8 @@ class CsGemmArgs(ctypes.Structure):
         ("conv_patch", c_int32),
         ("attn_cos_sin", c_void_p),
         ("attn_scale_log2e", ctypes.c_float),
+        ("attn_win_start", c_void_p),
+        ("attn_n_win", c_int32),
     ]
 
 

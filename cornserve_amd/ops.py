@@ -881,20 +881,23 @@ def pack_qkv_window_attn(w: torch.Tensor, b: torch.Tensor, heads: int) -> tuple[
 
 def qkv_window_attn(x: torch.Tensor, w_packed: torch.Tensor, b_packed: torch.Tensor, cos_sin: torch.Tensor, heads: int,
                     scale: float, *, a_row_sumsq: torch.Tensor | None = None, norm_eps: float = 0.0,
-                    out: torch.Tensor | None = None) -> torch.Tensor:
-    """attention(rotary(x . Wq^T + bq), rotary(x . Wk^T + bk), x . Wv^T + bv) over windows of 64 rows, one launch.
+                    out: torch.Tensor | None = None, win_start: torch.Tensor | None = None) -> torch.Tensor:
+    """attention(rotary(x . Wq^T + bq), rotary(x . Wk^T + bk), x . Wv^T + bv) over windows of up to 64 rows, one launch.
 
-    Replaces qkv Linear -> split -> rotary -> flash_attn_varlen_func (qwen2_5_vl.py:93-120) for a sequence whose
-    attention segments are ALL 64 rows starting at multiples of 64.  `w_packed`, `b_packed` come from
-    `pack_qkv_window_attn`; with `a_row_sumsq` the rows of `x` are RMS-normalised on the way (the norm weight folded
-    into the packed weight's columns, as for `gemm`).  Raises ValueError for shapes the kernel does not take."""
+    Replaces qkv Linear -> split -> rotary -> flash_attn_varlen_func (qwen2_5_vl.py:93-120).  Without `win_start` the
+    attention segments are ALL 64 rows starting at multiples of 64; with it (int32 [windows + 1] on the device: the
+    leading entries of cu_window_seqlens, ending at the number of rows of `x`) a window has 4 .. 64 rows, a multiple of
+    4, which the caller guarantees.  `w_packed`, `b_packed` come from `pack_qkv_window_attn`; with `a_row_sumsq` the
+    rows of `x` are RMS-normalised on the way (the norm weight folded into the packed weight's columns, as for
+    `gemm`).  Raises ValueError for shapes the kernel does not take."""
     if out is None:
         out = torch.empty((x.shape[0], heads * QKV_WATTN_HEAD_DIM), dtype=torch.bfloat16, device=x.device)
-    torch.ops.cornserve_amd.qkv_window_attn_(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps)
+    torch.ops.cornserve_amd.qkv_window_attn_(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps,
+                                              win_start)
     return out
 
 
-def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps) -> None:
+def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps, win_start=None) -> None:
     lib = _l.load()
     _rows_2d(x, torch.bfloat16, "x")
     _rows_2d(w_packed, torch.bfloat16, "w_packed")
@@ -907,8 +910,15 @@ def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_r
         raise ValueError(f"w_packed must be [{heads}*{QKV_WATTN_TILE_ROWS}, {K}], got {tuple(w_packed.shape)}")
     if tuple(b_packed.shape) != (heads * QKV_WATTN_TILE_ROWS,) or not b_packed.is_contiguous():
         raise ValueError(f"b_packed must be a contiguous [{heads * QKV_WATTN_TILE_ROWS}] tensor")
-    if M % QKV_WATTN_WINDOW:
-        raise ValueError(f"the rows of x ({M}) must be a whole number of {QKV_WATTN_WINDOW}-row windows")
+    if win_start is None:
+        if M % QKV_WATTN_WINDOW:
+            raise ValueError(f"the rows of x ({M}) must be a whole number of {QKV_WATTN_WINDOW}-row windows")
+    else:
+        _req(win_start, torch.int32, "win_start")
+        n_win = win_start.numel() - 1
+        if win_start.dim() != 1 or not win_start.is_contiguous() or n_win < 1 or not 4 * n_win <= M <= QKV_WATTN_WINDOW * n_win or M % 4:
+            raise ValueError(f"win_start must be a contiguous int32 [windows + 1] tensor whose windows of 4 .. "
+                             f"{QKV_WATTN_WINDOW} rows add up to the {M} rows of x")
     if tuple(cos_sin.shape) != (M, d) or not cos_sin.is_contiguous():
         raise ValueError(f"cos_sin must be a contiguous fp32 [{M}, {d}] table")
     if out.shape[0] < M or out.shape[1] < heads * d:
@@ -917,7 +927,7 @@ def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_r
         _req(a_row_sumsq, torch.float32, "a_row_sumsq")
         if a_row_sumsq.dim() != 2 or a_row_sumsq.shape[1] != SUMSQ_PARTS or not a_row_sumsq.is_contiguous() or a_row_sumsq.shape[0] < M:
             raise ValueError(f"a_row_sumsq must be a contiguous fp32 [>=M, {SUMSQ_PARTS}] tensor")
-    on = {t.device for t in (out, x, w_packed, b_packed, cos_sin, a_row_sumsq) if t is not None}
+    on = {t.device for t in (out, x, w_packed, b_packed, cos_sin, a_row_sumsq, win_start) if t is not None}
     if len(on) != 1:
         raise ValueError(f"qkv_window_attn operands live on different devices: {sorted(map(str, on))}")
     args = _l.CsGemmArgs()
@@ -928,6 +938,8 @@ def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_r
     args.M, args.N, args.K = M, heads * QKV_WATTN_TILE_ROWS, K
     args.a_row_sumsq = _ptr(a_row_sumsq)
     args.norm_eps = norm_eps
+    if win_start is not None:
+        args.attn_win_start, args.attn_n_win = win_start.data_ptr(), win_start.numel() - 1
     _l.check(lib.cs_qkv_window_attn(ctypes.byref(args), cos_sin.data_ptr(), scale, heads, d, _stream()), "cs_qkv_window_attn")
 
 
@@ -966,7 +978,7 @@ _OPERATORS: dict[str, tuple[str, object]] = {
     "resize_u8_pass_": ("(Tensor(a!) out, Tensor src, Tensor bounds, Tensor taps, int axis) -> ()", _resize_u8_pass_impl),
     "patchify_nchw_": ("(Tensor(a!) out, Tensor pixels, int patch) -> ()", _patchify_nchw_impl),
     "qkv_window_attn_": ("(Tensor(a!) out, Tensor x, Tensor w_packed, Tensor b_packed, Tensor cos_sin, int heads, "
-                         "float scale, Tensor? a_row_sumsq, float norm_eps) -> ()", _qkv_window_attn_impl),
+                         "float scale, Tensor? a_row_sumsq, float norm_eps, Tensor? win_start=None) -> ()", _qkv_window_attn_impl),
 }
 
 

@@ -36,7 +36,7 @@ extern "C" {
 #define CS_ERR_TOO_LARGE 4
 
 /* ABI version of this header; cs_abi_version() returns the value the library was built with. */
-#define CS_ABI_VERSION 5
+#define CS_ABI_VERSION 6
 int cs_abi_version(void);
 
 /* ------------------------------------------------------------------------------------------------
@@ -126,6 +126,9 @@ typedef struct CsGemmArgs {
   /* filled in by cs_qkv_window_attn (the rotary table and softmax scale of its fused epilogue)                      */
   const float* attn_cos_sin;
   float attn_scale_log2e;
+  /* cs_qkv_window_attn only, set by the caller: windows of fewer than 64 rows (see there); NULL / 0 otherwise         */
+  const int32_t* attn_win_start;
+  int32_t attn_n_win;
 } CsGemmArgs;
 #define CS_SUMSQ_PARTS 8
 
@@ -277,6 +280,12 @@ int cs_attn_varlen_keys_rotated(const void* q, const void* k, const void* v, int
  *     (both halves of a rotary pair in one lane; eight consecutive slots of a lane = one MFMA operand)
  *   gemm->C, ldc: out [M, heads * 80] bf16;  gemm->N = heads * 256;  other fields zero
  *   cos_sin: the [M, 80] fp32 table of cs_vit_index;  scale = head_dim^-0.5;  head_dim must be 80.
+ * Windows of fewer than 64 rows (the edge windows of an image whose sides are not multiples of 8 patches): with
+ *   gemm->attn_win_start = the first attn_n_win + 1 entries of cu_window_seqlens on the device (int32; window w is rows
+ *   attn_win_start[w] .. attn_win_start[w+1] - 1 of A, of cos_sin and of C; every count a multiple of 4 in 4 .. 64, the
+ *   caller's to guarantee) every window takes a 64-row slot of its own: a workgroup loads a short window's last row in
+ *   place of the missing ones, masks their keys in the softmax and does not store their queries.  M is then the number
+ *   of real rows, attn_win_start[attn_n_win].  A window of 64 rows gives the same bits in both forms.
  * CS_ERR_UNSUPPORTED for any other shape (the caller then takes cs_gemm + cs_attn_varlen).                          */
 int cs_qkv_window_attn(const CsGemmArgs* gemm, const float* cos_sin, float scale, int32_t heads, int32_t head_dim,
                        void* stream);

@@ -87,8 +87,9 @@ def test_qwen_without_folded_norms(dev, golden_dir):
 @pytest.mark.parametrize("fold_norm", [True, False])
 def test_qwen_one_launch_window_attention_against_separate_kernels(dev, fold_norm):
     """Batches whose windows are all whole (sides multiples of 8 patches) run qkv + rotary + window attention of a
-    block as one launch; the same weights through the separate kernels, and both against the oracle.  A ragged batch
-    takes the separate kernels in either model."""
+    block as one launch; the same weights through the separate kernels, and both against the oracle.  An item with
+    short edge windows takes the one launch too when its windows fill their 64-row slots well enough, else the
+    separate kernels, whatever it is batched with."""
     fused, sd, ocfg = build_qwen(dev, 4, (3,), seed=5, fold_norm=fold_norm)
     plain, _, _ = build_qwen(dev, 4, (3,), seed=5, fold_norm=fold_norm, fuse_window_attn=False)
     assert fused.fuse_window_attn and not plain.fuse_window_attn
@@ -106,7 +107,9 @@ def test_qwen_one_launch_window_attention_against_separate_kernels(dev, fold_nor
     check(a, ref, REL_BF16, "one launch vs fp32 oracle")
     check(a, torch.cat(oq.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)), REL_BF16, "one launch vs bf16 oracle")
     # The route is chosen per item: an item with whole windows takes the one launch whatever the batch (a single image
-    # too), an item with partial windows at its edges the separate kernels -- inside one batch, both at once.
+    # too), and so does an item whose edge windows are short but fill their slots to fuse_min_fill (20 x 36 patches: 15
+    # windows for 180 merged units = 0.75); an item below that (2 frames of 6 x 10: 0.47) takes the separate kernels --
+    # inside one batch, both at once.
     px, grid = synth.qwen_inputs([(1, 32, 32)], seed=6)
     g = torch.cat(grid).numpy().astype(np.int64)
     pv = torch.cat(px).to(dev, torch.bfloat16)
@@ -125,11 +128,20 @@ def test_qwen_one_launch_window_attention_against_separate_kernels(dev, fold_nor
     assert [tuple(o.shape) for o in mixed] == [(t * h * w // 4, 3584) for t, h, w in grids]
     assert torch.equal(mixed[3], alone), "an item's bits do not depend on the batch"
     sep = plain.forward_device(pv, g)
-    for i in (0, 2):                                    # the items with partial windows ran the separate kernels: same bits
-        assert torch.equal(mixed[i], sep[i])
+    assert torch.equal(mixed[2], sep[2])                # the sparse item ran the separate kernels: same bits
+    assert not torch.equal(mixed[0], sep[0])            # the 0.75 item did not
+    stages.clear()
+    ragged_alone = fused.forward_device(px2[0].to(dev, torch.bfloat16), g[:1], mark=stages.append)[0]
+    assert stages.count("gemm_qkv_attn_window") == 3 and stages.count("attn_window") == 0
+    assert torch.equal(mixed[0], ragged_alone), "a ragged item's bits do not depend on the batch either"
     ref = oq.forward(sd, ocfg, px2, grid2, dtype=torch.float32)
     for i in range(len(grids)):
         check(mixed[i], ref[i], REL_BF16, f"mixed batch item {i} vs fp32 oracle")
+    # with the slots required to be full, only whole-window items take the one launch
+    fused.fuse_min_fill = 1.0
+    strict = fused.forward_device(pv, g)
+    assert torch.equal(strict[0], sep[0]) and torch.equal(strict[3], alone)
+    fused.fuse_min_fill = 0.75
     # the deployment knob: below `fuse_min_rows` one-launch rows a batch takes the separate kernels throughout
     fused.fuse_min_rows = 3072
     stages.clear()

@@ -1124,6 +1124,62 @@ def test_qkv_window_attn_against_fp32_and_the_unfused_chain(ops, dev, M, K, head
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("fold", [True, False])
+def test_qkv_window_attn_windows_of_fewer_than_64_rows(ops, dev, fold):
+    """Windows of 4 .. 64 rows, one 64-row slot each: against the fp32 restatement and the unfused chain on the same
+    segments, every row count a window can have (4 r c for r, c in 1..4) among them, a number of windows that is not a
+    multiple of the four a workgroup takes; a window of 64 rows comes out with the bits of the whole-window form; rows
+    past the last window's end are not written."""
+    d, heads, K = 80, 4, 1280
+    counts = [64, 48, 36, 64, 16, 4, 8, 12, 24, 32, 64, 64, 16, 48, 64, 36, 4]
+    cu = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    M = int(cu[-1])
+    x = rnd((M, K), 1.0, 21, dev)
+    w = rnd((3 * heads * d, K), K**-0.5, 22, dev)
+    b = rnd((3 * heads * d,), 0.5, 23, dev)
+    g = torch.Generator().manual_seed(24)
+    ang = torch.rand((M, d // 2), generator=g) * 6.0
+    cs = torch.cat([ang.cos(), ang.sin()], dim=1).float().contiguous().to(dev)
+    eps = 1e-6
+    sums = ops.row_sumsq(x) if fold else None
+    wp, bp = ops.pack_qkv_window_attn(w, b, heads)
+    out = torch.full((M + 8, heads * d), 7.0, dtype=torch.bfloat16, device=dev)
+    ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, a_row_sumsq=sums, norm_eps=eps, out=out[:M],
+                        win_start=torch.from_numpy(cu).to(dev))
+    assert torch.all(out[M:] == 7.0)
+    got = out[:M]
+    xf = x.float().cpu()
+    if fold:
+        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    qkv = xf @ w.float().cpu().T + b.float().cpu()
+    ref = attn_ref(qkv, cu.tolist(), heads, d, ang)
+    close(got, ref, 2**-6, f"fused qkv + ragged window attention fold={fold}")
+    qkv_dev = ops.gemm(x, w, b, a_row_sumsq=sums, norm_eps=eps)
+    H = heads * d
+    plan = ops.attn_plan(cu, dev)
+    chain = ops.attn_varlen(qkv_dev[:, :H], qkv_dev[:, H:2 * H], qkv_dev[:, 2 * H:], plan, heads, d, d**-0.5, cs)
+    err_fused = (got.float().cpu() - ref).abs().max().item()
+    err_chain = (chain.float().cpu() - ref).abs().max().item()
+    assert err_fused <= 1.5 * err_chain + 1e-3, (err_fused, err_chain)
+    # whole windows: the two forms of the launch give the same bits (what lets one batch hold both kinds of item)
+    for w0 in [i for i, c in enumerate(counts) if c == 64]:
+        lo = int(cu[w0])
+        alone = ops.qkv_window_attn(x[lo:lo + 64], wp, bp, cs[lo:lo + 64].contiguous(), heads, d**-0.5,
+                                    a_row_sumsq=None if sums is None else sums[lo:lo + 64].contiguous(), norm_eps=eps)
+        assert torch.equal(alone, got[lo:lo + 64]), w0
+    whole_cu = torch.arange(0, 64 * 6 + 1, 64, dtype=torch.int32, device=dev)
+    xs, css = x[:384], cs[:384].contiguous()
+    ss = None if sums is None else sums[:384].contiguous()
+    a = ops.qkv_window_attn(xs, wp, bp, css, heads, d**-0.5, a_row_sumsq=ss, norm_eps=eps)
+    r = ops.qkv_window_attn(xs, wp, bp, css, heads, d**-0.5, a_row_sumsq=ss, norm_eps=eps, win_start=whole_cu)
+    assert torch.equal(a, r)
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, win_start=torch.from_numpy(cu[:3].copy()).to(dev))   # 2 windows cannot hold M rows
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, win_start=torch.from_numpy(cu.astype(np.int64)).to(dev))
+
+
+@pytest.mark.gpu
 def test_qkv_window_attn_rejects_what_the_kernel_does_not_take(ops, dev):
     d, heads, K = 80, 2, 192
     x = rnd((128, K), 1.0, 1, dev)
