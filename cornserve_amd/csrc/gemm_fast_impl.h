@@ -603,7 +603,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
     //      S^T's accumulators hold four consecutive keys per lane, the layout of the second product's operand, and
     //      the transposed V fragments hold four consecutive keys per head dim: O^T = V^T.P^T needs no transposition.
     auto wattn_epilogue = [&](auto) {   // (generic: only instantiated for the kernel that calls it)
-      static_assert(!WATTN || (BM == 256 && BN == 256 && WAVES_M == 4 && WAVES_N == 1 && !W_FP8),
+      static_assert(!WATTN || (BM == 256 && BN == 256 && WAVES_M == 4 && WAVES_N == 1),
                     "one 64-row window per wave, one head per column tile");
       constexpr int HD = 80, HALF = 40;
       // A register written by a vector instruction must not be read by an MFMA in the next few cycles.  The compiler
@@ -635,6 +635,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
       auto row_at = [&](int local) { return RAGGED ? row0 + min(local, cnt - 1) : row0 + local; };
       const int head = n0 / BN;
       const bf16_t* const pBias = (const bf16_t*)p.bias + n0;
+      const float* const pScale = p.w_scale + n0;   // fp8 weights: the per-output-channel scales, packed like the bias
       const float sl2 = p.attn_scale_log2e;
       // per-row scale of the folded RMSNorm: rows row0 + 16I + lr
       float rstd[4];
@@ -649,9 +650,12 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         }
       }
       // bias of the lane's q / k slots (packed like the weight rows: fragment J, lane kq -> 4 consecutive entries)
+      // (fp8 weights: fetched per row block next to the scales instead, five at a time)
       bf16x4_t bias_qk[10];
+      if constexpr (!W_FP8) {
 #pragma unroll
-      for (int J = 0; J < 10; ++J) bias_qk[J] = *(const bf16x4_t*)(pBias + (J / 2) * 32 + kq * 8 + (J % 2) * 4);
+        for (int J = 0; J < 10; ++J) bias_qk[J] = *(const bf16x4_t*)(pBias + (J / 2) * 32 + kq * 8 + (J % 2) * 4);
+      }
       bf16x8_t qf8[4][2], kf8[4][2];
       bf16x4_t qf4[4], kf4[4];
       // q and k: scale, bias, rotary (fp32, one rounding), packed as operands
@@ -669,11 +673,25 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         }
         static_for<2>([&](auto which_c) {
           constexpr int WHICH = decltype(which_c)::value;   // 0: q (fragments 0..4), 1: k (fragments 5..9)
+          // fp8 weights: the scales of these 20 output channels, fetched for every row block anew (behind an opaque
+          // offset, so that the compiler does not keep all 40 registers of them across the row blocks)
+          f32x4_t wsc[W_FP8 ? 5 : 1];
+          if constexpr (W_FP8) {
+            int kq_s = kq * 8;
+            asm volatile("" : "+v"(kq_s));
+#pragma unroll
+            for (int J5 = 0; J5 < 5; ++J5) {
+              const int ch = ((WHICH * 5 + J5) / 2) * 32 + kq_s + ((WHICH * 5 + J5) % 2) * 4;
+              wsc[W_FP8 ? J5 : 0] = *(const f32x4_t*)(pScale + ch);
+              bias_qk[WHICH * 5 + J5] = *(const bf16x4_t*)(pBias + ch);
+            }
+          }
           float x[20];
           static_for<20>([&](auto s_c) {
             constexpr int S = decltype(s_c)::value, J = WHICH * 5 + S / 4, R = (I * NT + J) * 4 + S % 4;
             float t;
             asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R));
+            if constexpr (W_FP8) t *= wsc[W_FP8 ? S / 4 : 0][S % 4];
             x[S] = t * rstd[I] + bf2f(bias_qk[J][S % 4]);
           });
           float o[20];
@@ -754,9 +772,13 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
         int lane_v = __builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
         asm volatile("" : "+v"(lane_v));
         const int lrv = lane_v & 15;
-        float bias_v[5];   // fragment row lr of the transposed V fragments
+        float bias_v[5], scale_v[W_FP8 ? 5 : 1];   // fragment row lr of the transposed V fragments
 #pragma unroll
-        for (int d = 0; d < 5; ++d) bias_v[d] = bf2f(pBias[((10 + d) / 2) * 32 + (lrv >> 2) * 8 + ((10 + d) % 2) * 4 + (lrv & 3)]);
+        for (int d = 0; d < 5; ++d) {
+          const int ch = ((10 + d) / 2) * 32 + (lrv >> 2) * 8 + ((10 + d) % 2) * 4 + (lrv & 3);
+          bias_v[d] = bf2f(pBias[ch]);
+          if constexpr (W_FP8) scale_v[W_FP8 ? d : 0] = pScale[ch];
+        }
         // the folded norm's scale of rows 16I + 4kq + r: recomputed for rows 16I + lr (not kept in registers since the
         // q / k phase) and fetched from the lanes that hold them
         float rv[4][4];
@@ -781,6 +803,7 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
               constexpr int E = decltype(e_c)::value, I = 2 * T + E / 4, R = (I * NT + J) * 4 + E % 4;
               float t;
               asm volatile("v_accvgpr_read_b32 %0, a[%1]" : "=v"(t) : "n"(R));
+              if constexpr (W_FP8) t *= scale_v[W_FP8 ? Dd : 0];
               f[E] = f2bf(t * rv[I][E % 4] + bias_v[Dd]);
             });
             vf8[Dd][T] = f;

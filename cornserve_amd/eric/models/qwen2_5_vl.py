@@ -263,14 +263,15 @@ class QwenVisionBase(EricModel):
 class Qwen2_5_VisionTransformer(QwenVisionBase):
     def __init__(self, config: Any, weight_format: str = "bf16", fold_norm: bool = True,
                  split_residual: bool = True, fuse_window_attn: bool = True, fuse_min_rows: int = 0,
-                 fuse_min_fill: float = 0.75) -> None:
+                 fuse_min_fill: float | None = None) -> None:
         """`fuse_window_attn`: run qkv projection + rotary + window attention of a block (:93-120) as ONE launch
         (`ops.qkv_window_attn`: q, k and v stay in registers, the [L, 3*hidden] tensor is never written).  Every window
         takes a 64-row slot of that launch, so an ITEM takes it when its windows fill their slots to `fuse_min_fill` or
         more on average (an image whose sides are multiples of 8 patches fills them completely; edge windows of other
         sizes are shorter, and a slot's empty rows cost the projection as much as full ones: below about 0.75 the
-        separate kernels are cheaper).  Other items of the same batch, fp8 weights and head dims other than 80 take the
-        separate kernels.  The one launch rounds q and k to bf16 once (after the rotation) instead of twice, so the two
+        separate kernels are cheaper -- 0.92 with fp8 weights, whose projection costs more per row; None selects these
+        measured break-even points).  Other items of the same batch and head dims other than 80 take the separate
+        kernels.  The one launch rounds q and k to bf16 once (after the rotation) instead of twice, so the two
         routes agree within the parity tolerance, not bit for bit; since the route depends on the item alone, an item's
         embedding is the same bits whatever it is batched with (setting the attribute to False afterwards selects the
         separate kernels for every item).  `fuse_min_rows` > 0 is a deployment knob that gives this up for latency: a
@@ -296,7 +297,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         self.weight_format = weight_format
         self.split_residual = bool(split_residual)
         self.fuse_min_rows = int(fuse_min_rows)
-        self.fuse_min_fill = float(fuse_min_fill)
+        self.fuse_min_fill = float(fuse_min_fill) if fuse_min_fill is not None else (0.75 if weight_format == "bf16" else 0.92)
         self.hidden_size = vc.hidden_size
         self.out_hidden_size = vc.out_hidden_size
         self.num_heads = vc.num_heads
@@ -318,10 +319,10 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         self.fold_norm = (bool(fold_norm) and weight_format == "bf16" and H % 64 == 0 and 192 <= H <= 160 * ops.SUMSQ_PARTS
                           and _round_up(self.intermediate_size, 64) >= 192)
 
-        # (one launch for qkv + rotary + window attention: bf16 weights, heads of 80, K a multiple of 64 from 192 up,
+        # (one launch for qkv + rotary + window attention: heads of 80, K a multiple of 64 from 192 up,
         # windows of 64 rows)
         win_rows = (self.window_size // self.spatial_merge_size // self.patch_size) ** 2 * self.spatial_merge_unit
-        self.fuse_window_attn = (bool(fuse_window_attn) and weight_format == "bf16" and H % 64 == 0 and H >= 192
+        self.fuse_window_attn = (bool(fuse_window_attn) and H % 64 == 0 and H >= 192
                                  and self.head_dim == ops.QKV_WATTN_HEAD_DIM and win_rows == ops.QKV_WATTN_WINDOW)
 
         self.patch_embed = _PatchEmbed(self.in_channels, self.hidden_size, self.temporal_patch_size, self.patch_size)
@@ -365,7 +366,9 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 }
             )
             if self.fuse_window_attn and i not in self.fullatt_block_indexes:
-                blocks[-1]["qkv_wattn"] = ops.pack_qkv_window_attn(qkv_w, blk.attn.qkv.bias.to(self.dtype), self.num_heads)
+                # (fp8: the very bytes and scales of the plain form, reordered)
+                lin = blocks[-1]["qkv"]
+                blocks[-1]["qkv_wattn"] = ops.pack_qkv_window_attn(lin["w"], lin["b"].to(self.dtype), self.num_heads, w_scale=lin["s"])
         pk["blocks"] = blocks
         pk["ln_q"] = self.merger.ln_q.weight
         pk["fc1"] = self._lin(self.merger.mlp[0].weight, self.merger.mlp[0].bias)
@@ -476,7 +479,8 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         for i, b in enumerate(pk["blocks"]):
             full = i in self.fullatt_block_indexes
             if not full and fused_rows:
-                wp, bp = b["qkv_wattn"]
+                wp, bp, *sp = b["qkv_wattn"]      # (a third entry with fp8 weights: their scales)
+                wsc = sp[0] if sp else None
                 if fold:
                     mark("gemm_qkv_attn_window")
                     ops.qkv_window_attn(xf, wp, bp, ix.cos_sin[:fused_rows], nh, scale, a_row_sumsq=ss[:fused_rows], norm_eps=eps,
@@ -486,7 +490,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                     ops.rmsnorm(xf, b["n1"], eps, out=n[:fused_rows])
                     mark("gemm_qkv_attn_window")
                     ops.qkv_window_attn(n[:fused_rows], wp, bp, ix.cos_sin[:fused_rows], nh, scale, out=att[:fused_rows],
-                                        win_start=win_start)
+                                        win_start=win_start, w_scale=wsc)
             if full or fused_rows < L:
                 lo = 0 if full else fused_rows           # first row the separate kernels work on in this block
                 if fold:

@@ -867,21 +867,31 @@ def qkv_window_attn_row_order(heads: int) -> torch.Tensor:
     return _qkv_window_attn_row_order(int(heads)).clone()
 
 
-def pack_qkv_window_attn(w: torch.Tensor, b: torch.Tensor, heads: int) -> tuple[torch.Tensor, torch.Tensor]:
-    """The qkv weight [3*heads*80, K] and bias [3*heads*80] in the row order `qkv_window_attn` takes (done once, at load)."""
+def pack_qkv_window_attn(w: torch.Tensor, b: torch.Tensor, heads: int, w_scale: torch.Tensor | None = None):
+    """The qkv weight [3*heads*80, K] and bias [3*heads*80] in the row order `qkv_window_attn` takes (done once, at load).
+    fp8 weights (float8_e4m3fn or uint8 bytes, with `w_scale` fp32 [3*heads*80]): the bytes are reordered as they are,
+    and the result has a third entry, the scales in the same order (1 for the padding rows, whose bytes are zero)."""
     if w.dim() != 2 or w.shape[0] != 3 * heads * QKV_WATTN_HEAD_DIM or b.shape != (w.shape[0],):
         raise ValueError(f"qkv weight must be [3*{heads}*{QKV_WATTN_HEAD_DIM}, K] with a matching bias")
+    fp8 = w.dtype in (torch.float8_e4m3fn, torch.uint8)
+    if fp8 != (w_scale is not None) or (fp8 and (w_scale.shape != (w.shape[0],) or w_scale.dtype != torch.float32)):
+        raise ValueError("fp8 weights (float8_e4m3fn / uint8) come with an fp32 w_scale [3*heads*80]; bf16 weights without")
     order = qkv_window_attn_row_order(heads).to(w.device)
     keep = (order >= 0).unsqueeze(1)
     rows = order.clamp_min(0)
-    wp = torch.where(keep, w[rows], torch.zeros((), dtype=w.dtype, device=w.device)).contiguous()
+    wb = w.view(torch.uint8) if fp8 else w
+    wp = torch.where(keep, wb[rows], torch.zeros((), dtype=wb.dtype, device=w.device)).contiguous()
     bp = torch.where(keep[:, 0], b[rows], torch.zeros((), dtype=b.dtype, device=b.device)).contiguous()
-    return wp, bp
+    if not fp8:
+        return wp, bp
+    sp = torch.where(keep[:, 0], w_scale[rows], torch.ones((), dtype=torch.float32, device=w.device)).contiguous()
+    return wp, bp, sp
 
 
 def qkv_window_attn(x: torch.Tensor, w_packed: torch.Tensor, b_packed: torch.Tensor, cos_sin: torch.Tensor, heads: int,
                     scale: float, *, a_row_sumsq: torch.Tensor | None = None, norm_eps: float = 0.0,
-                    out: torch.Tensor | None = None, win_start: torch.Tensor | None = None) -> torch.Tensor:
+                    out: torch.Tensor | None = None, win_start: torch.Tensor | None = None,
+                    w_scale: torch.Tensor | None = None) -> torch.Tensor:
     """attention(rotary(x . Wq^T + bq), rotary(x . Wk^T + bk), x . Wv^T + bv) over windows of up to 64 rows, one launch.
 
     Replaces qkv Linear -> split -> rotary -> flash_attn_varlen_func (qwen2_5_vl.py:93-120).  Without `win_start` the
@@ -889,18 +899,27 @@ def qkv_window_attn(x: torch.Tensor, w_packed: torch.Tensor, b_packed: torch.Ten
     leading entries of cu_window_seqlens, ending at the number of rows of `x`) a window has 4 .. 64 rows, a multiple of
     4, which the caller guarantees.  `w_packed`, `b_packed` come from `pack_qkv_window_attn`; with `a_row_sumsq` the
     rows of `x` are RMS-normalised on the way (the norm weight folded into the packed weight's columns, as for
-    `gemm`).  Raises ValueError for shapes the kernel does not take."""
+    `gemm`).  fp8 weights: `w_packed` uint8 with `w_scale` (both from `pack_qkv_window_attn`), no folded norm.
+    Raises ValueError for shapes the kernel does not take."""
     if out is None:
         out = torch.empty((x.shape[0], heads * QKV_WATTN_HEAD_DIM), dtype=torch.bfloat16, device=x.device)
     torch.ops.cornserve_amd.qkv_window_attn_(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps,
-                                              win_start)
+                                              win_start, w_scale)
     return out
 
 
-def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps, win_start=None) -> None:
+def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps, win_start=None,
+                          w_scale=None) -> None:
     lib = _l.load()
     _rows_2d(x, torch.bfloat16, "x")
-    _rows_2d(w_packed, torch.bfloat16, "w_packed")
+    fp8 = w_scale is not None
+    _rows_2d(w_packed, torch.uint8 if fp8 else torch.bfloat16, "w_packed")
+    if fp8:
+        _req(w_scale, torch.float32, "w_scale")
+        if tuple(w_scale.shape) != (heads * QKV_WATTN_TILE_ROWS,) or not w_scale.is_contiguous():
+            raise ValueError(f"w_scale must be a contiguous fp32 [{heads * QKV_WATTN_TILE_ROWS}] tensor")
+        if a_row_sumsq is not None:
+            raise ValueError("the folded norm (a_row_sumsq) does not exist for fp8 weights")
     _rows_2d(out, torch.bfloat16, "out")
     _req(b_packed, torch.bfloat16, "b_packed")
     _req(cos_sin, torch.float32, "cos_sin")
@@ -927,7 +946,7 @@ def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_r
         _req(a_row_sumsq, torch.float32, "a_row_sumsq")
         if a_row_sumsq.dim() != 2 or a_row_sumsq.shape[1] != SUMSQ_PARTS or not a_row_sumsq.is_contiguous() or a_row_sumsq.shape[0] < M:
             raise ValueError(f"a_row_sumsq must be a contiguous fp32 [>=M, {SUMSQ_PARTS}] tensor")
-    on = {t.device for t in (out, x, w_packed, b_packed, cos_sin, a_row_sumsq, win_start) if t is not None}
+    on = {t.device for t in (out, x, w_packed, b_packed, cos_sin, a_row_sumsq, win_start, w_scale) if t is not None}
     if len(on) != 1:
         raise ValueError(f"qkv_window_attn operands live on different devices: {sorted(map(str, on))}")
     args = _l.CsGemmArgs()
@@ -940,6 +959,8 @@ def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_r
     args.norm_eps = norm_eps
     if win_start is not None:
         args.attn_win_start, args.attn_n_win = win_start.data_ptr(), win_start.numel() - 1
+    if fp8:
+        args.w_fp8, args.w_scale = 1, w_scale.data_ptr()
     _l.check(lib.cs_qkv_window_attn(ctypes.byref(args), cos_sin.data_ptr(), scale, heads, d, _stream()), "cs_qkv_window_attn")
 
 
@@ -978,7 +999,8 @@ _OPERATORS: dict[str, tuple[str, object]] = {
     "resize_u8_pass_": ("(Tensor(a!) out, Tensor src, Tensor bounds, Tensor taps, int axis) -> ()", _resize_u8_pass_impl),
     "patchify_nchw_": ("(Tensor(a!) out, Tensor pixels, int patch) -> ()", _patchify_nchw_impl),
     "qkv_window_attn_": ("(Tensor(a!) out, Tensor x, Tensor w_packed, Tensor b_packed, Tensor cos_sin, int heads, "
-                         "float scale, Tensor? a_row_sumsq, float norm_eps, Tensor? win_start=None) -> ()", _qkv_window_attn_impl),
+                         "float scale, Tensor? a_row_sumsq, float norm_eps, Tensor? win_start=None, Tensor? w_scale=None) -> ()",
+                         _qkv_window_attn_impl),
 }
 
 

@@ -286,6 +286,8 @@ int cs_attn_varlen_keys_rotated(const void* q, const void* k, const void* v, int
  *   caller's to guarantee) every window takes a 64-row slot of its own: a workgroup loads a short window's last row in
  *   place of the missing ones, masks their keys in the softmax and does not store their queries.  M is then the number
  *   of real rows, attn_win_start[attn_n_win].  A window of 64 rows gives the same bits in both forms.
+ * fp8 weights: gemm->w_fp8 = 1, W the e4m3 bytes of the same packed rows ([heads * 256, K], ldw % 16 == 0, zero bytes in
+ *   the padding rows), gemm->w_scale fp32 [heads * 256] packed like the bias (16-byte aligned); no a_row_sumsq.
  * CS_ERR_UNSUPPORTED for any other shape (the caller then takes cs_gemm + cs_attn_varlen).                          */
 int cs_qkv_window_attn(const CsGemmArgs* gemm, const float* cos_sin, float scale, int32_t heads, int32_t head_dim,
                        void* stream);

@@ -292,6 +292,16 @@ def test_qwen_fp8_weights(dev):
     out = model(Modality.VIDEO, "", {"pixel_values_videos": px, "video_grid_thw": grid})
     ref = oq.forward(sd_dq, ocfg, px, grid, dtype=torch.float32)
     check(out[0], ref[0], REL_FP8, "fp8 weights vs de-quantised fp32 oracle")
+    # whole windows take the one launch with fp8 weights too (short ones only above a slot fill of 0.92)
+    assert model.fuse_window_attn and model.fuse_min_fill == 0.92
+    px, grid = synth.qwen_inputs([(1, 16, 24), (2, 8, 16), (1, 18, 18)], seed=6)
+    g = torch.cat(grid).numpy().astype(np.int64)
+    stages: list[str] = []
+    out = model.forward_device(torch.cat(px).to(dev, torch.bfloat16), g, mark=stages.append)
+    assert stages.count("gemm_qkv_attn_window") == 2 and stages.count("attn_window") == 2   # the 18 x 18 image: separate
+    ref = oq.forward(sd_dq, ocfg, px, grid, dtype=torch.float32)
+    for i in range(3):
+        check(out[i], ref[i], REL_FP8, f"fp8 weights, one launch, item {i} vs de-quantised fp32 oracle")
 
 
 def test_full_size_configs_through_properties(dev):

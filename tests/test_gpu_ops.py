@@ -1180,6 +1180,48 @@ def test_qkv_window_attn_windows_of_fewer_than_64_rows(ops, dev, fold):
 
 
 @pytest.mark.gpu
+def test_qkv_window_attn_fp8_weights(ops, dev):
+    """The one launch with e4m3 weights and per-output-channel scales (the bytes and scales of the plain fp8 GEMM,
+    reordered): whole windows and short ones against the fp32 restatement on the de-quantised weights, and no further
+    from it than the unfused fp8 chain."""
+    from cornserve_amd.eric.models.qwen2_5_vl import quantize_fp8_rows
+
+    d, heads, K = 80, 4, 1280
+    w = rnd((3 * heads * d, K), K**-0.5, 32, dev)
+    b = rnd((3 * heads * d,), 0.5, 33, dev)
+    q, sc = quantize_fp8_rows(w)
+    w_deq = q.float().cpu() * sc.float().cpu()[:, None]
+    wp, bp, sp = ops.pack_qkv_window_attn(q, b, heads, w_scale=sc)
+    assert wp.dtype == torch.uint8 and sp.dtype == torch.float32 and sp.shape == (heads * 256,)
+    for counts in ([64] * 9, [64, 48, 36, 16, 4, 64, 24, 32, 12, 8]):
+        cu = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+        M = int(cu[-1])
+        x = rnd((M, K), 1.0, 31, dev)
+        g = torch.Generator().manual_seed(34)
+        ang = torch.rand((M, d // 2), generator=g) * 6.0
+        cs = torch.cat([ang.cos(), ang.sin()], dim=1).float().contiguous().to(dev)
+        ragged = any(c != 64 for c in counts)
+        got = ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, w_scale=sp,
+                                  win_start=torch.from_numpy(cu).to(dev) if ragged else None)
+        qkv = x.float().cpu() @ w_deq.T + b.float().cpu()
+        ref = attn_ref(qkv, cu.tolist(), heads, d, ang)
+        close(got, ref, 2**-6, f"fused fp8 qkv + window attention, ragged={ragged}")
+        qkv_dev = ops.gemm(x, q, b, w_scale=sc)
+        H = heads * d
+        chain = ops.attn_varlen(qkv_dev[:, :H], qkv_dev[:, H:2 * H], qkv_dev[:, 2 * H:], ops.attn_plan(cu, dev), heads, d,
+                                d**-0.5, cs)
+        err_fused = (got.float().cpu() - ref).abs().max().item()
+        err_chain = (chain.float().cpu() - ref).abs().max().item()
+        assert err_fused <= 1.5 * err_chain + 1e-3, (err_fused, err_chain)
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5)                      # fp8 bytes without their scales
+    with pytest.raises(ValueError):
+        ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, w_scale=sp, a_row_sumsq=ops.row_sumsq(x))
+    with pytest.raises(ValueError):
+        ops.pack_qkv_window_attn(q, b, heads)
+
+
+@pytest.mark.gpu
 def test_qkv_window_attn_rejects_what_the_kernel_does_not_take(ops, dev):
     d, heads, K = 80, 2, 192
     x = rnd((128, K), 1.0, 1, dev)
