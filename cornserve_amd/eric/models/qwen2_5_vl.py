@@ -168,6 +168,16 @@ class QwenVisionBase(EricModel):
     def _g(a: torch.Tensor, lin: dict, **kw) -> torch.Tensor:
         return ops.gemm(a, lin["w"], lin["b"], w_scale=lin["s"], **kw)
 
+    def _plain_qkv(self, block: dict) -> dict:
+        """The qkv layer of a block in the form the separate kernels take.  A window block keeps only the per-head
+        packed form of its weight (one copy in HBM); the plain rows are the same bits in another order and are put back
+        together the first time an item takes the separate kernels."""
+        if block["qkv"] is None:
+            wp, bp, *sp = block["qkv_wattn"]
+            w, b, *s = ops.unpack_qkv_window_attn(wp, bp, self.num_heads, w_scale=sp[0] if sp else None)
+            block["qkv"] = {"w": w, "b": b, "s": s[0] if s else None}
+        return block["qkv"]
+
     def patchify_frames(self, frames: list[torch.Tensor], arithmetic: str = "fused",
                         pixel_budgets: list | None = None) -> tuple[torch.Tensor, np.ndarray]:
         """uint8 frames of every item ([T,H,W,3] or [H,W,3], on the host or the device) -> (pixel_values
@@ -369,6 +379,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 # (fp8: the very bytes and scales of the plain form, reordered)
                 lin = blocks[-1]["qkv"]
                 blocks[-1]["qkv_wattn"] = ops.pack_qkv_window_attn(lin["w"], lin["b"].to(self.dtype), self.num_heads, w_scale=lin["s"])
+                blocks[-1]["qkv"] = None   # the plain form comes back from the packed one if a batch ever needs it
         pk["blocks"] = blocks
         pk["ln_q"] = self.merger.ln_q.weight
         pk["fc1"] = self._lin(self.merger.mlp[0].weight, self.merger.mlp[0].bias)
@@ -495,12 +506,12 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 lo = 0 if full else fused_rows           # first row the separate kernels work on in this block
                 if fold:
                     mark("gemm_qkv")
-                    self._g(x[lo:], b["qkv"], out=qkv[lo:], a_row_sumsq=ss[lo:], norm_eps=eps)
+                    self._g(x[lo:], self._plain_qkv(b), out=qkv[lo:], a_row_sumsq=ss[lo:], norm_eps=eps)
                 else:
                     mark("norm")
                     ops.rmsnorm(x[lo:], b["n1"], eps, out=n[lo:])
                     mark("gemm_qkv")
-                    self._g(n[lo:], b["qkv"], out=qkv[lo:])
+                    self._g(n[lo:], self._plain_qkv(b), out=qkv[lo:])
                 mark("attn_full" if full else "attn_window")
                 ops.attn_varlen_rotary_(qkv, plan_full if full else plan_win, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")

@@ -888,6 +888,19 @@ def pack_qkv_window_attn(w: torch.Tensor, b: torch.Tensor, heads: int, w_scale: 
     return wp, bp, sp
 
 
+def unpack_qkv_window_attn(w_packed: torch.Tensor, b_packed: torch.Tensor, heads: int, w_scale: torch.Tensor | None = None):
+    """The inverse of `pack_qkv_window_attn`: the plain [3*heads*80, K] weight, bias (and scales) back from the packed
+    form, bit for bit (fp8 weights come back as uint8 bytes)."""
+    order = qkv_window_attn_row_order(heads).to(w_packed.device)
+    if w_packed.dim() != 2 or w_packed.shape[0] != order.numel() or b_packed.shape != (order.numel(),):
+        raise ValueError(f"packed qkv weight must be [{heads}*{QKV_WATTN_TILE_ROWS}, K] with a matching bias")
+    place = torch.empty(3 * heads * QKV_WATTN_HEAD_DIM, dtype=torch.int64, device=w_packed.device)
+    packed_rows = torch.arange(order.numel(), device=w_packed.device)
+    place[order[order >= 0]] = packed_rows[order >= 0]
+    out = (w_packed[place].contiguous(), b_packed[place].contiguous())
+    return out if w_scale is None else out + (w_scale[place].contiguous(),)
+
+
 def qkv_window_attn(x: torch.Tensor, w_packed: torch.Tensor, b_packed: torch.Tensor, cos_sin: torch.Tensor, heads: int,
                     scale: float, *, a_row_sumsq: torch.Tensor | None = None, norm_eps: float = 0.0,
                     out: torch.Tensor | None = None, win_start: torch.Tensor | None = None,

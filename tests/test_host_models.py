@@ -471,3 +471,24 @@ def test_qkv_window_attn_row_order_is_a_permutation_with_padding():
     for d in range(40):
         a, b = pos[80 + d], pos[80 + d + 40]      # q rows of head 1
         assert (a % 32) // 8 == (b % 32) // 8
+
+
+def test_qkv_window_attn_pack_and_unpack_are_inverse():
+    """The per-head packed qkv weight (the only copy a window block keeps) gives back the plain rows bit for bit."""
+    from cornserve_amd import ops
+
+    heads, K = 3, 64
+    g = torch.Generator().manual_seed(3)
+    w = torch.randn((3 * heads * 80, K), generator=g).to(torch.bfloat16)
+    b = torch.randn((3 * heads * 80,), generator=g).to(torch.bfloat16)
+    wp, bp = ops.pack_qkv_window_attn(w, b, heads)
+    assert wp.shape == (heads * 256, K) and int((wp.float().abs().sum(1) == 0).sum()) >= heads * 16   # 16 zero rows per head
+    w2, b2 = ops.unpack_qkv_window_attn(wp, bp, heads)
+    assert torch.equal(w2, w) and torch.equal(b2, b)
+    q = torch.randint(0, 256, (3 * heads * 80, K), generator=g, dtype=torch.uint8)
+    sc = torch.rand((3 * heads * 80,), generator=g) + 0.5
+    qp, bp, sp = ops.pack_qkv_window_attn(q, b, heads, w_scale=sc)
+    q2, b2, s2 = ops.unpack_qkv_window_attn(qp, bp, heads, w_scale=sp)
+    assert torch.equal(q2, q) and torch.equal(b2, b) and torch.equal(s2, sc)
+    with pytest.raises(ValueError):
+        ops.unpack_qkv_window_attn(wp[:-1], bp, heads)
