@@ -581,6 +581,13 @@ def test_worker_upload_ahead(dev):
         pending = nxt
     out = worker.execute_model(worker.upload(wb(Modality.IMAGE, {"pixel_frames": frames}, 1)))
     assert torch.equal(out[0], direct_frames[0])
+    # frames as decoded, resized on the GPU: the frames travel as bytes, the pixel budget stays on the host
+    raw = {"raw_frames": [torch.randint(0, 256, (1, 90, 131, 3), dtype=torch.uint8, generator=torch.Generator().manual_seed(4))],
+           "raw_frames_budget": [torch.tensor([56 * 56, 28 * 28 * 12])]}
+    direct_raw = model(Modality.IMAGE, "", raw)
+    up = worker.upload(wb(Modality.IMAGE, dict(raw), 1))
+    assert up.data["raw_frames"][0].is_cuda and not up.data["raw_frames_budget"][0].is_cuda
+    assert torch.equal(worker.execute_model(up)[0], direct_raw[0])
 
     gmodel, _, _ = build_gemma(dev, 2, 224, 640, 16, seed=2)
     px, crops = synth.gemma3_inputs(2, 224, seed=2)
