@@ -83,6 +83,7 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
       const int n1 = best_cols * 256;
       CsGemmArgs lo = a, hi = a;
       lo.N = n1;
+      lo.prefetch = nullptr;  // the tail launch is the one with idle compute units
       hi.N = a.N - n1;
       hi.W = (const char*)a.W + (int64_t)n1 * a.ldw * (a.w_fp8 ? 1 : 2);
       if (a.w_scale) hi.w_scale = a.w_scale + n1;

@@ -202,6 +202,27 @@ __global__ __launch_bounds__(64 * NW) void gemm_fast_kernel(const CsGemmArgs p) 
   //      then bands of 8 tile-rows walked column-major so the 32 workgroups resident on one XCD share
   //      8 A panels and 4 W panels through that XCD's L2.
   const int ntiles = p.tiles_m * p.tiles_n;
+  // ---- workgroups past the computing ones (a launch with few tiles and a prefetch hint): read the hinted bytes once,
+  //      16 per lane and four loads in flight, and leave.  They take no part in barriers or in the tile loop.
+  if ((int)blockIdx.x >= ntiles) {
+    const int pw = (int)blockIdx.x - ntiles, npw = (int)gridDim.x - ntiles;
+    const char* const base = (const char*)p.prefetch;
+    const int64_t n16 = p.prefetch_bytes >> 4, stride = (int64_t)npw * (64 * NW);
+    u32x4_t sink = {0u, 0u, 0u, 0u};
+    for (int64_t i = (int64_t)pw * (64 * NW) + threadIdx.x; i < n16; i += 4 * stride) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int64_t j = i + u * stride;
+        if (j < n16) {
+          const u32x4_t v = *(const u32x4_t*)(base + 16 * j);
+          sink[0] |= v[0] & v[1] & v[2] & v[3];
+        }
+      }
+    }
+    // (a store that never happens -- M is positive -- keeps the loads alive)
+    if (sink[0] == 0xFFFFFFFFu && p.M < 0) *(volatile uint32_t*)p.C = sink[0];
+    return;
+  }
   auto tile_origin = [&](int vb, int& m0, int& n0) {
     const int per = ntiles >> 3;
     if (vb < per * 8) vb = (vb & 7) * per + (vb >> 3);
@@ -1320,7 +1341,10 @@ int launch(const CsGemmArgs& a, hipStream_t stream) {
   }
   const int tiles = p.tiles_m * p.tiles_n;
   // One resident workgroup per CU (LDS-bound); with more tiles than CUs the kernel is persistent.
-  const int grid = tiles <= 256 ? tiles : 256;
+  int grid = tiles <= 256 ? tiles : 256;
+  // few tiles and a prefetch hint: the idle compute units read the hinted bytes (see the kernel)
+  if (p.prefetch && p.prefetch_bytes >= 16 && tiles <= 192) grid = tiles + (256 - tiles < 128 ? 256 - tiles : 128);
+  else p.prefetch = nullptr;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, p);
   return cs_launch_status();
 }

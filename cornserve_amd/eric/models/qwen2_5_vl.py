@@ -308,6 +308,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         self.split_residual = bool(split_residual)
         self.fuse_min_rows = int(fuse_min_rows)
         self.fuse_min_fill = float(fuse_min_fill) if fuse_min_fill is not None else (0.75 if weight_format == "bf16" else 0.92)
+        self.prefetch_rows = 6144   # batches of at most this many patches pass the kernels a weight-prefetch hint (0: never)
         self.hidden_size = vc.hidden_size
         self.out_hidden_size = vc.out_hidden_size
         self.num_heads = vc.num_heads
@@ -487,15 +488,29 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         scale = d**-0.5
         # rows [0, fused_rows) belong to the items whose window blocks run as one launch, the rest to the others
         xf = x[:fused_rows]
+        # A batch of few rows leaves most compute units idle in the N = hidden GEMMs, and what bounds those launches is
+        # the latency of weights that nothing has touched since the previous forward pass: the one-launch window block
+        # has its idle units read the gate|up weights, the attention-output projection the down-projection's, the
+        # down-projection the next block's qkv weights.
+        hint = L <= self.prefetch_rows
+
+        def next_qkv(i: int) -> torch.Tensor | None:
+            if i + 1 >= len(pk["blocks"]):
+                return pk["fc1"]["w"]
+            nb = pk["blocks"][i + 1]
+            return nb["qkv"]["w"] if nb["qkv"] is not None else nb["qkv_wattn"][0]
+
         for i, b in enumerate(pk["blocks"]):
             full = i in self.fullatt_block_indexes
+            pf_proj = b["down"]["w"] if hint else None
+            pf_down = next_qkv(i) if hint else None
             if not full and fused_rows:
                 wp, bp, *sp = b["qkv_wattn"]      # (a third entry with fp8 weights: their scales)
                 wsc = sp[0] if sp else None
                 if fold:
                     mark("gemm_qkv_attn_window")
                     ops.qkv_window_attn(xf, wp, bp, ix.cos_sin[:fused_rows], nh, scale, a_row_sumsq=ss[:fused_rows], norm_eps=eps,
-                                        out=att[:fused_rows], win_start=win_start)
+                                        out=att[:fused_rows], win_start=win_start, prefetch=b["gu"]["w"] if hint else None)
                 else:
                     mark("norm")
                     ops.rmsnorm(xf, b["n1"], eps, out=n[:fused_rows])
@@ -516,19 +531,19 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 ops.attn_varlen_rotary_(qkv, plan_full if full else plan_win, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")
             if fold:
-                self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss, **res)
+                self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss, prefetch=pf_proj, **res)
                 mark("gemm_gate_up")
                 self._g(x, b["gu"], epilogue=ops.EPI_SWIGLU, out=hmid, a_row_sumsq=ss, norm_eps=eps)
                 mark("gemm_down")
-                self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss, **res)
+                self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, c_row_sumsq=ss, prefetch=pf_down, **res)
             else:
-                self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **res)
+                self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, prefetch=pf_proj, **res)
                 mark("norm")
                 ops.rmsnorm(x, b["n2"], eps, out=n)
                 mark("gemm_gate_up")
                 self._g(n, b["gu"], epilogue=ops.EPI_SWIGLU, out=hmid)
                 mark("gemm_down")
-                self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **res)
+                self._g(hmid, b["down"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, prefetch=pf_down, **res)
 
         mark("norm")
         ops.rmsnorm(x, pk["ln_q"], self.norm_eps, out=n)

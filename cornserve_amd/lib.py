@@ -17,7 +17,7 @@ CS_ERR_INVALID_ARG = 1
 CS_ERR_UNSUPPORTED = 2
 CS_ERR_LAUNCH = 3
 CS_ERR_TOO_LARGE = 4
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 EPI_BIAS, EPI_RESIDUAL, EPI_SWIGLU, EPI_GELU_ERF, EPI_GELU_TANH, EPI_QUICK_GELU = range(6)
 
@@ -65,6 +65,8 @@ class CsGemmArgs(ctypes.Structure):
         ("attn_scale_log2e", ctypes.c_float),
         ("attn_win_start", c_void_p),
         ("attn_n_win", c_int32),
+        ("prefetch", c_void_p),
+        ("prefetch_bytes", c_int64),
     ]
 
 

@@ -123,8 +123,13 @@ def gemm(
     residual_lo: torch.Tensor | None = None,
     out_lo: torch.Tensor | None = None,
     conv_patch: int = 0,
+    prefetch: torch.Tensor | None = None,
 ) -> torch.Tensor:
     """out[M,N] = epilogue(a[M,K] @ w[N,K]^T).  `w` is bf16, or float8_e4m3fn/uint8 with `w_scale`.
+
+    `prefetch`: a contiguous tensor (the weights of the launch that follows) that a launch with few rows has its idle
+    compute units read once, so that it sits in the last-level cache when the next launch asks for it; no effect on
+    the result, ignored by launches that fill the chip.
 
     `conv_patch` > 0: `a` is NCHW pixels [B,C,H,W] (bf16, contiguous) and the product is the convolution with kernel =
     stride = conv_patch as a strided-gather GEMM: row m is patch (b, py, px), its K elements are the patch's pixels in
@@ -143,15 +148,24 @@ def gemm(
     exactly).  A zero-filled plane next to any bf16 tensor is a valid pair.
 
     Dispatches to `torch.ops.cornserve_amd.gemm_` (or the functional `gemm` when nothing is written in place)."""
-    if out is None and c_row_sumsq is None and c_row_sum is None and out_lo is None and residual_lo is None:
+    if out is None and c_row_sumsq is None and c_row_sum is None and out_lo is None and residual_lo is None and prefetch is None:
         return torch.ops.cornserve_amd.gemm(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k,
                                             a_row_sumsq, norm_eps, a_row_sum, w_col_sum, conv_patch)
     if out is None:  # (with c_rows: a permutation of the M rows; anything else needs the caller's `out`)
         out = torch.empty((_gemm_rows(a, a_rows, conv_patch), w.shape[0] // 2 if epilogue == EPI_SWIGLU else w.shape[0]),
                           dtype=torch.bfloat16, device=a.device)
     torch.ops.cornserve_amd.gemm_(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq,
-                                  c_row_sumsq, norm_eps, a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo, conv_patch)
+                                  c_row_sumsq, norm_eps, a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo, conv_patch,
+                                  prefetch)
     return out
+
+
+def _set_prefetch(args, prefetch: torch.Tensor | None, device: torch.device) -> None:
+    if prefetch is None:
+        return
+    if not prefetch.is_cuda or prefetch.device != device or not prefetch.is_contiguous() or prefetch.data_ptr() % 16:
+        raise ValueError("prefetch must be a contiguous, 16-byte aligned tensor on the operands' device")
+    args.prefetch, args.prefetch_bytes = prefetch.data_ptr(), prefetch.numel() * prefetch.element_size()
 
 
 def _gemm_rows(a, a_rows, conv_patch) -> int:
@@ -177,7 +191,7 @@ def _gemm_functional(a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_row
 
 
 def _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows, k, a_row_sumsq, c_row_sumsq, norm_eps,
-               a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo, conv_patch=0) -> None:
+               a_row_sum, c_row_sum, w_col_sum, residual_lo, out_lo, conv_patch=0, prefetch=None) -> None:
     """Implementation of cornserve_amd::gemm_: argument checks, then cs_gemm on the current stream."""
     lib = _l.load()
     _req(a, torch.bfloat16, "a")
@@ -290,6 +304,7 @@ def _gemm_impl(out, a, w, bias, epilogue, residual, w_scale, pos, a_rows, c_rows
     args.w_col_sum = _ptr(w_col_sum)
     args.residual_lo = _ptr(residual_lo)
     args.c_lo = _ptr(out_lo)
+    _set_prefetch(args, prefetch, a.device)
     _l.check(lib.cs_gemm(ctypes.byref(args), _stream()), "cs_gemm")
 
 
@@ -904,7 +919,7 @@ def unpack_qkv_window_attn(w_packed: torch.Tensor, b_packed: torch.Tensor, heads
 def qkv_window_attn(x: torch.Tensor, w_packed: torch.Tensor, b_packed: torch.Tensor, cos_sin: torch.Tensor, heads: int,
                     scale: float, *, a_row_sumsq: torch.Tensor | None = None, norm_eps: float = 0.0,
                     out: torch.Tensor | None = None, win_start: torch.Tensor | None = None,
-                    w_scale: torch.Tensor | None = None) -> torch.Tensor:
+                    w_scale: torch.Tensor | None = None, prefetch: torch.Tensor | None = None) -> torch.Tensor:
     """attention(rotary(x . Wq^T + bq), rotary(x . Wk^T + bk), x . Wv^T + bv) over windows of up to 64 rows, one launch.
 
     Replaces qkv Linear -> split -> rotary -> flash_attn_varlen_func (qwen2_5_vl.py:93-120).  Without `win_start` the
@@ -913,16 +928,17 @@ def qkv_window_attn(x: torch.Tensor, w_packed: torch.Tensor, b_packed: torch.Ten
     4, which the caller guarantees.  `w_packed`, `b_packed` come from `pack_qkv_window_attn`; with `a_row_sumsq` the
     rows of `x` are RMS-normalised on the way (the norm weight folded into the packed weight's columns, as for
     `gemm`).  fp8 weights: `w_packed` uint8 with `w_scale` (both from `pack_qkv_window_attn`), no folded norm.
+    `prefetch` as for `gemm`.
     Raises ValueError for shapes the kernel does not take."""
     if out is None:
         out = torch.empty((x.shape[0], heads * QKV_WATTN_HEAD_DIM), dtype=torch.bfloat16, device=x.device)
     torch.ops.cornserve_amd.qkv_window_attn_(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps,
-                                              win_start, w_scale)
+                                              win_start, w_scale, prefetch)
     return out
 
 
 def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_row_sumsq, norm_eps, win_start=None,
-                          w_scale=None) -> None:
+                          w_scale=None, prefetch=None) -> None:
     lib = _l.load()
     _rows_2d(x, torch.bfloat16, "x")
     fp8 = w_scale is not None
@@ -974,6 +990,7 @@ def _qkv_window_attn_impl(out, x, w_packed, b_packed, cos_sin, heads, scale, a_r
         args.attn_win_start, args.attn_n_win = win_start.data_ptr(), win_start.numel() - 1
     if fp8:
         args.w_fp8, args.w_scale = 1, w_scale.data_ptr()
+    _set_prefetch(args, prefetch, x.device)
     _l.check(lib.cs_qkv_window_attn(ctypes.byref(args), cos_sin.data_ptr(), scale, heads, d, _stream()), "cs_qkv_window_attn")
 
 
@@ -990,7 +1007,7 @@ _OPERATORS: dict[str, tuple[str, object]] = {
     "gemm_": ("(Tensor(a!) out, Tensor a, Tensor w, Tensor? bias, int epilogue, Tensor? residual, Tensor? w_scale, "
               "Tensor? pos, Tensor? a_rows, Tensor? c_rows, int? k, Tensor? a_row_sumsq, Tensor(b!)? c_row_sumsq, "
               "float norm_eps, Tensor? a_row_sum, Tensor(c!)? c_row_sum, Tensor? w_col_sum, Tensor? residual_lo, "
-              "Tensor(d!)? out_lo, int conv_patch=0) -> ()", _gemm_impl),
+              "Tensor(d!)? out_lo, int conv_patch=0, Tensor? prefetch=None) -> ()", _gemm_impl),
     "row_stats_": ("(Tensor(a!) sumsq_out, Tensor(b!)? sum_out, Tensor x) -> ()", _row_stats_impl),
     "rmsnorm_": ("(Tensor(a!) out, Tensor x, Tensor w, float eps, bool gemma) -> ()", _rmsnorm_impl),
     "layernorm_": ("(Tensor(a!) out, Tensor x, Tensor w, Tensor b, float eps) -> ()", _layernorm_impl),
@@ -1012,7 +1029,8 @@ _OPERATORS: dict[str, tuple[str, object]] = {
     "resize_u8_pass_": ("(Tensor(a!) out, Tensor src, Tensor bounds, Tensor taps, int axis) -> ()", _resize_u8_pass_impl),
     "patchify_nchw_": ("(Tensor(a!) out, Tensor pixels, int patch) -> ()", _patchify_nchw_impl),
     "qkv_window_attn_": ("(Tensor(a!) out, Tensor x, Tensor w_packed, Tensor b_packed, Tensor cos_sin, int heads, "
-                         "float scale, Tensor? a_row_sumsq, float norm_eps, Tensor? win_start=None, Tensor? w_scale=None) -> ()",
+                         "float scale, Tensor? a_row_sumsq, float norm_eps, Tensor? win_start=None, Tensor? w_scale=None, "
+                         "Tensor? prefetch=None) -> ()",
                          _qkv_window_attn_impl),
 }
 

@@ -36,7 +36,7 @@ extern "C" {
 #define CS_ERR_TOO_LARGE 4
 
 /* ABI version of this header; cs_abi_version() returns the value the library was built with. */
-#define CS_ABI_VERSION 6
+#define CS_ABI_VERSION 7
 int cs_abi_version(void);
 
 /* ------------------------------------------------------------------------------------------------
@@ -129,6 +129,14 @@ typedef struct CsGemmArgs {
   /* cs_qkv_window_attn only, set by the caller: windows of fewer than 64 rows (see there); NULL / 0 otherwise         */
   const int32_t* attn_win_start;
   int32_t attn_n_win;
+  /* Optional hint for launches that leave compute units idle (at most 192 workgroups of the fast path's tile forms and
+   * of cs_qkv_window_attn): prefetch_bytes bytes at prefetch (16-byte aligned) -- typically the weights of the NEXT
+   * launch, which no kernel has touched since the previous forward pass -- are read once by up to 128 workgroups
+   * started next to the computing ones, so that they sit in the last-level cache when the next launch asks for them
+   * (a few-row launch is bound by operand latency, not by arithmetic).  Results are not affected; the hint is ignored
+   * by launches that fill the chip and by the general kernel.  NULL / 0: no hint.                                  */
+  const void* prefetch;
+  int64_t prefetch_bytes;
 } CsGemmArgs;
 #define CS_SUMSQ_PARTS 8
 

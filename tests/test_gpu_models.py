@@ -281,6 +281,11 @@ def test_qwen_batch_items_are_independent(dev):
         assert torch.equal(alone, together[i])
     again = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
     assert all(torch.equal(a, b) for a, b in zip(again, together))  # deterministic
+    # small batches pass the kernels a weight-prefetch hint: the same bits with the hint switched off
+    assert model.prefetch_rows >= 2048
+    model.prefetch_rows = 0
+    unhinted = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+    assert all(torch.equal(a, b) for a, b in zip(unhinted, together))
 
 
 def test_qwen_fp8_weights(dev):

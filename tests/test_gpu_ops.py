@@ -414,6 +414,39 @@ def test_gemm_fast_path_forms(ops, dev, M, N, K):
     assert torch.equal(scat, ref)
 
 
+def test_gemm_prefetch_hint_leaves_the_result_alone(ops, dev):
+    """A launch with few tiles and a `prefetch` tensor starts extra workgroups that only read that tensor: the product
+    has the bits it has without the hint, whatever the hinted size (odd, shorter than one 16-byte piece, many MB), on
+    every tile form, and a launch that fills the chip ignores the hint."""
+    hints = [torch.zeros(n, dtype=torch.uint8, device=dev) for n in (8, 16, 1000003, 24 << 20)]
+    hints.append(rnd((3420, 1280), 0.05, 5, dev))
+    for M, N, K in [(1000, 1280, 320), (300, 520, 448), (2100, 1280, 192), (8192, 1280, 192), (700, 2304, 256)]:
+        a, w, b = rnd((M, K), 1.0, 11, dev), rnd((N, K), 0.05, 12, dev), rnd((N,), 0.02, 13, dev)
+        res = rnd((M, N), 1.0, 14, dev)
+        plain = ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res)
+        ss0 = torch.zeros((M, ops.SUMSQ_PARTS), device=dev) if N <= 1280 else None   # (parts past N's are not written)
+        plain_ss = ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res, c_row_sumsq=ss0) if ss0 is not None else None
+        for h in hints:
+            assert torch.equal(ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res, prefetch=h), plain), (M, N, K, h.shape)
+            if ss0 is not None:
+                ss1 = torch.zeros_like(ss0)
+                got = ops.gemm(a, w, b, epilogue=ops.EPI_RESIDUAL, residual=res, c_row_sumsq=ss1, prefetch=h)
+                assert torch.equal(got, plain_ss) and torch.equal(ss1, ss0)
+    # fp8 weights (their own tile forms)
+    a, b = rnd((520, 448), 1.0, 21, dev), rnd((640,), 0.02, 23, dev)
+    wq = torch.randn(640, 448, generator=torch.Generator().manual_seed(22)) * 0.05
+    sc = wq.abs().amax(dim=1) / 448.0
+    q, sc = (wq / sc[:, None]).to(torch.float8_e4m3fn).to(dev), sc.to(dev)
+    assert torch.equal(ops.gemm(a, q, b, w_scale=sc, prefetch=hints[2]), ops.gemm(a, q, b, w_scale=sc))
+    # the hint has to be readable device memory in whole 16-byte pieces from its start
+    with pytest.raises(ValueError):
+        ops.gemm(a, q, b, w_scale=sc, prefetch=hints[2][1:])
+    with pytest.raises(ValueError):
+        ops.gemm(a, q, b, w_scale=sc, prefetch=hints[4][:, :64])
+    with pytest.raises((ValueError, RuntimeError)):
+        ops.gemm(a, q, b, w_scale=sc, prefetch=torch.zeros(64))
+
+
 @pytest.mark.parametrize("M,N,K", [
     (8192, 3072, 192),    # 256x256 (three-stage ring with byte-wide W tiles) + 256x128 remainder, 3 K tiles
     (8192, 2304, 256),    # 256x256 + 128x192 remainder
@@ -1173,6 +1206,11 @@ def test_qkv_window_attn_windows_of_fewer_than_64_rows(ops, dev, fold):
     a = ops.qkv_window_attn(xs, wp, bp, css, heads, d**-0.5, a_row_sumsq=ss, norm_eps=eps)
     r = ops.qkv_window_attn(xs, wp, bp, css, heads, d**-0.5, a_row_sumsq=ss, norm_eps=eps, win_start=whole_cu)
     assert torch.equal(a, r)
+    # a prefetch hint (extra workgroups that only read it) changes no bit of either form
+    hint = rnd((3420, 1280), 0.05, 25, dev)
+    assert torch.equal(ops.qkv_window_attn(xs, wp, bp, css, heads, d**-0.5, a_row_sumsq=ss, norm_eps=eps, prefetch=hint), a)
+    assert torch.equal(ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, a_row_sumsq=sums, norm_eps=eps,
+                                           win_start=torch.from_numpy(cu).to(dev), prefetch=hint), got)
     with pytest.raises(ValueError):
         ops.qkv_window_attn(x, wp, bp, cs, heads, d**-0.5, win_start=torch.from_numpy(cu[:3].copy()).to(dev))   # 2 windows cannot hold M rows
     with pytest.raises(ValueError):
