@@ -116,6 +116,10 @@ class QwenVisionBase(EricModel):
     `forward_device`, `chunk_shape` and the attributes patch_size, temporal_patch_size, spatial_merge_size,
     in_channels, weight_format and patch_embed."""
 
+    # Batches of at most this many patches pass the GEMM launches a weight-prefetch hint (0: never): such launches
+    # leave compute units idle, and those read the weights a later launch of the block needs into the last-level cache.
+    prefetch_rows = 6144
+
     # what the checkpoint's image processor normalises with (preprocessor_config.json): CLIP statistics for
     # Qwen2-VL and Qwen2.5-VL; subclasses override
     # carry the residual stream with 16 significant bits (see Qwen2_5_VisionTransformer.__init__)
@@ -308,7 +312,6 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
         self.split_residual = bool(split_residual)
         self.fuse_min_rows = int(fuse_min_rows)
         self.fuse_min_fill = float(fuse_min_fill) if fuse_min_fill is not None else (0.75 if weight_format == "bf16" else 0.92)
-        self.prefetch_rows = 6144   # batches of at most this many patches pass the kernels a weight-prefetch hint (0: never)
         self.hidden_size = vc.hidden_size
         self.out_hidden_size = vc.out_hidden_size
         self.num_heads = vc.num_heads

@@ -175,29 +175,38 @@ class Qwen2VisionTransformer(QwenVisionBase):
             ops.row_stats(x, ss, sm)
             stats_in = lambda lin: {"a_row_sumsq": ss, "a_row_sum": sm, "w_col_sum": lin["colsum"], "norm_eps": eps}  # noqa: E731
             stats_out = {"c_row_sumsq": ss, "c_row_sum": sm}
-        for b in pk["blocks"]:
+        # few rows: each launch names the weights of the launch after next for its idle compute units to read
+        hint = L <= self.prefetch_rows
+        for i, b in enumerate(pk["blocks"]):
+            after = pk["blocks"][i + 1]["qkv"] if i + 1 < len(pk["blocks"]) else pk["m1"]
+            after_proj = pk["blocks"][i + 1]["proj"]["w"] if i + 1 < len(pk["blocks"]) else None
+            pf_qkv, pf_proj, pf_fc1, pf_fc2 = ((b["fc1"]["w"], b["fc2"]["w"], after["w"], after_proj) if hint
+                                               else (None, None, None, None))
             if fold:
                 mark("gemm_qkv")
-                ops.gemm(x, b["qkv"]["w"], b["qkv"]["b"], out=qkv, **stats_in(b["qkv"]))
+                ops.gemm(x, b["qkv"]["w"], b["qkv"]["b"], out=qkv, prefetch=pf_qkv, **stats_in(b["qkv"]))
             else:
                 mark("norm")
                 ops.layernorm(x, *b["n1"], eps, out=n)
                 mark("gemm_qkv")
-                self._g(n, b["qkv"], out=qkv)
+                self._g(n, b["qkv"], out=qkv, prefetch=pf_qkv)
             mark("attn_full")
             ops.attn_varlen_rotary_(qkv, plan, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")
-            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **res, **(stats_out if fold else {}))
+            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, prefetch=pf_proj, **res,
+                    **(stats_out if fold else {}))
             if fold:
                 mark("gemm_fc1")
-                ops.gemm(x, b["fc1"]["w"], b["fc1"]["b"], epilogue=ops.EPI_QUICK_GELU, out=hmid, **stats_in(b["fc1"]))
+                ops.gemm(x, b["fc1"]["w"], b["fc1"]["b"], epilogue=ops.EPI_QUICK_GELU, out=hmid, prefetch=pf_fc1,
+                         **stats_in(b["fc1"]))
             else:
                 mark("norm")
                 ops.layernorm(x, *b["n2"], eps, out=n)
                 mark("gemm_fc1")
-                self._g(n, b["fc1"], epilogue=ops.EPI_QUICK_GELU, out=hmid)
+                self._g(n, b["fc1"], epilogue=ops.EPI_QUICK_GELU, out=hmid, prefetch=pf_fc1)
             mark("gemm_fc2")
-            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **res, **(stats_out if fold else {}))
+            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, prefetch=pf_fc2, **res,
+                    **(stats_out if fold else {}))
         mark("norm")
         ops.layernorm(x, *pk["ln_q"], eps, out=n)
         mark("gemm_merger")

@@ -233,15 +233,21 @@ class Qwen3_VisionTransformer(QwenVisionBase):
         if self.split_residual:   # the byte plane of the residual stream; zero = "x is exact".  It is updated in place
             lo = torch.zeros(x.shape, dtype=torch.uint8, device=dev)   # even when the bf16 plane moves to a new buffer
             stats_out = dict(stats_out, residual_lo=lo, out_lo=lo)
+        # few rows: each launch names the weights of the launch after next for its idle compute units to read
+        hint = L <= self.prefetch_rows
         for i, b in enumerate(pk["blocks"]):
+            after = pk["blocks"][i + 1]["qkv"] if i + 1 < len(pk["blocks"]) else pk["merger"]["fc1"]
+            after_proj = pk["blocks"][i + 1]["proj"]["w"] if i + 1 < len(pk["blocks"]) else None
+            pf_qkv, pf_proj, pf_fc1, pf_fc2 = ((b["fc1"]["w"], b["fc2"]["w"], after["w"], after_proj) if hint
+                                               else (None, None, None, None))
             if fold:
                 mark("gemm_qkv")
-                ops.gemm(x, b["qkv"]["w"], b["qkv"]["b"], out=qkv, **stats_in(b["qkv"]))
+                ops.gemm(x, b["qkv"]["w"], b["qkv"]["b"], out=qkv, prefetch=pf_qkv, **stats_in(b["qkv"]))
             else:
                 mark("norm")
                 ops.layernorm(x, *b["n1"], eps, out=n)
                 mark("gemm_qkv")
-                self._g(n, b["qkv"], out=qkv)
+                self._g(n, b["qkv"], out=qkv, prefetch=pf_qkv)
             mark("rope")
             ops.rope_qk_(qkv, ix.cos_sin, nh, d)
             mark("attn_full")
@@ -249,18 +255,19 @@ class Qwen3_VisionTransformer(QwenVisionBase):
             mark("gemm_proj")
             # a hidden state kept for a deepstack merger must survive: the next update goes to a new buffer
             x_next = torch.empty_like(x) if kept and kept[-1] is x else x
-            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x_next, **stats_out)
+            self._g(att, b["proj"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x_next, prefetch=pf_proj, **stats_out)
             x = x_next
             if fold:
                 mark("gemm_fc1")
-                ops.gemm(x, b["fc1"]["w"], b["fc1"]["b"], epilogue=self.act_epilogue, out=hmid, **stats_in(b["fc1"]))
+                ops.gemm(x, b["fc1"]["w"], b["fc1"]["b"], epilogue=self.act_epilogue, out=hmid, prefetch=pf_fc1,
+                         **stats_in(b["fc1"]))
             else:
                 mark("norm")
                 ops.layernorm(x, *b["n2"], eps, out=n)
                 mark("gemm_fc1")
-                self._g(n, b["fc1"], epilogue=self.act_epilogue, out=hmid)
+                self._g(n, b["fc1"], epilogue=self.act_epilogue, out=hmid, prefetch=pf_fc1)
             mark("gemm_fc2")
-            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, **stats_out)
+            self._g(hmid, b["fc2"], epilogue=ops.EPI_RESIDUAL, residual=x, out=x, prefetch=pf_fc2, **stats_out)
             if i in self.deepstack_visual_indexes:
                 kept.append(x)
 

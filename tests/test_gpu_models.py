@@ -697,6 +697,8 @@ def test_qwen2_vl_against_oracle_and_golden(dev, golden_dir):
     assert img[0].shape == (64, 3584) and vid[0].shape == (48, 3584) and img[0].dtype == torch.bfloat16
     both = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
     assert torch.equal(both[0], img[0]) and torch.equal(both[1], vid[0])        # items are independent
+    model.prefetch_rows = 0                                                     # the weight-prefetch hint changes no bit
+    assert all(torch.equal(a, b) for a, b in zip(model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid}), both))
     ref16 = o2.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
     ref32 = o2.forward(sd, ocfg, px, grid, dtype=torch.float32)
     for i in range(2):
@@ -756,6 +758,8 @@ def test_qwen3_vl_against_oracle_and_golden(dev, golden_dir):
     assert [tuple(o.shape) for o in out] == [(60, 3072), (32, 3072)] and out[0].dtype == torch.bfloat16
     vid = model(Modality.VIDEO, "", {"pixel_values_videos": px[1:], "video_grid_thw": grid[1:]})
     assert torch.equal(vid[0], out[1])                                   # items are independent
+    model.prefetch_rows = 0                                              # the weight-prefetch hint changes no bit
+    assert all(torch.equal(a, b) for a, b in zip(model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid}), out))
     ref16 = o3.forward(sd, ocfg, px, grid, dtype=torch.bfloat16)
     ref32 = o3.forward(sd, ocfg, px, grid, dtype=torch.float32)
     for i in range(2):
