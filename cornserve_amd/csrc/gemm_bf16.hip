@@ -284,6 +284,7 @@ extern "C" int cs_gemm(const CsGemmArgs* args, void* stream_) {
   if (((uintptr_t)a.A | (uintptr_t)a.W) & 15) return CS_ERR_INVALID_ARG;
   if (((uintptr_t)a.C | (uintptr_t)a.bias | (uintptr_t)a.residual | (uintptr_t)a.pos) & 7) return CS_ERR_INVALID_ARG;
   if ((uintptr_t)a.w_scale & 15) return CS_ERR_INVALID_ARG;
+  if (a.prefetch ? (((uintptr_t)a.prefetch & 15) || a.prefetch_bytes < 0) : a.prefetch_bytes != 0) return CS_ERR_INVALID_ARG;
   if (((uintptr_t)a.a_row_sumsq | (uintptr_t)a.c_row_sumsq | (uintptr_t)a.a_row_sum | (uintptr_t)a.c_row_sum |
        (uintptr_t)a.w_col_sum) & 15)
     return CS_ERR_INVALID_ARG;

@@ -24,6 +24,7 @@ extern "C" int cs_qkv_window_attn(const CsGemmArgs* gemm, const float* cos_sin, 
   if (a.lda % 8 || a.ldw % (a.w_fp8 ? 16 : 8) || a.ldc % 4 || a.ldc < heads * 80) return CS_ERR_INVALID_ARG;
   if (((uintptr_t)a.A | (uintptr_t)a.W | (uintptr_t)cos_sin | (uintptr_t)a.a_row_sumsq) & 15) return CS_ERR_INVALID_ARG;
   if (((uintptr_t)a.C | (uintptr_t)a.bias) & 7) return CS_ERR_INVALID_ARG;
+  if (a.prefetch ? (((uintptr_t)a.prefetch & 15) || a.prefetch_bytes < 0) : a.prefetch_bytes != 0) return CS_ERR_INVALID_ARG;
   // per-lane source offsets of the direct loads are 32-bit byte offsets from the matrix bases
   if ((int64_t)a.M * a.lda * 2 >= (int64_t)UINT32_MAX || (int64_t)a.N * a.ldw * (a.w_fp8 ? 1 : 2) >= (int64_t)UINT32_MAX)
     return CS_ERR_UNSUPPORTED;

@@ -77,6 +77,18 @@ def test_invalid_arguments_are_rejected_without_a_gpu():
     assert l.cs_gemm_rmsnorm_noalloc(ctypes.byref(na), None) == lib.CS_ERR_UNSUPPORTED      # no folded form of it
     na.epilogue, na.M = lib.EPI_BIAS, 65537
     assert l.cs_gemm_rmsnorm_noalloc(ctypes.byref(na), None) == lib.CS_ERR_TOO_LARGE
+    # a prefetch hint must start on a 16-byte boundary and carry a size (and no size without an address)
+    pa = lib.CsGemmArgs()
+    pa.A, pa.W, pa.C = 0x1000, 0x2000, 0x3000
+    pa.lda = pa.ldw = pa.K = 1280
+    pa.ldc = pa.N = 3840
+    pa.M, pa.epilogue = 256, lib.EPI_BIAS
+    pa.prefetch, pa.prefetch_bytes = 0x4008, 4096
+    assert l.cs_gemm(ctypes.byref(pa), None) == lib.CS_ERR_INVALID_ARG
+    pa.prefetch, pa.prefetch_bytes = 0x4000, -1
+    assert l.cs_gemm(ctypes.byref(pa), None) == lib.CS_ERR_INVALID_ARG
+    pa.prefetch, pa.prefetch_bytes = None, 4096
+    assert l.cs_gemm(ctypes.byref(pa), None) == lib.CS_ERR_INVALID_ARG
     g = np.array([[1, 3, 4]], np.int64)  # odd height cannot be merged 2x2
     with pytest.raises(ValueError):
         ops.vit_seqlens_host(g, 2, 4)
