@@ -53,6 +53,15 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
     return narrow();
   }
   if (a.a_row_sum) return narrow();   // see dispatch_epi_w
+  // Few rows and many columns: when 256x128 tiles fit in one round they put more compute units to work than the
+  // forms above (1024 rows x 6912 columns: 216 workgroups against 176 of 256x160 or 108 of 256x256), and a launch
+  // of one round is bound by what a single compute unit pulls in per K tile, not by the chip's throughput.  The
+  // accumulation order of an output element is the same in every tile form, so the choice changes no bit.
+  {
+    const int64_t t128 = (int64_t)((a.M + 255) / 256) * ((a.N + 127) / 128);
+    const double c128 = rounds_cost(a.M, a.N, 256, 128) * 1.10;
+    if (t128 <= 256 && !few_rows && c128 < c160 - 0.05 && c128 < c256 - 0.05) return cs_gemm_fast_tile_256x128(a, stream);
+  }
   if (c160 < c256) return narrow();
   // Column split.  When the last round of 256x256 tiles would leave most CUs idle, the leading columns
   // that fill whole rounds go to one launch and the remaining columns to a second launch with smaller

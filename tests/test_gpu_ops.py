@@ -392,6 +392,8 @@ def _epilogue_ref(ops, epi, base, res):
     (1000, 1280, 320),    # 256x160, row tail, 5 K tiles
     (300, 520, 448),      # 256x256 with row and column tails, 7 K tiles
     (8192, 1280, 192),    # 256x160, one tile per CU, 3 K tiles
+    (1000, 6912, 256),    # few rows, many columns: 256x128 over the whole width (216 workgroups in one round)
+    (2048, 3840, 192),    # the same choice at 240 workgroups
 ])
 def test_gemm_fast_path_forms(ops, dev, M, N, K):
     a, w, b = rnd((M, K), 1.0, 11, dev), rnd((N, K), 0.05, 12, dev), rnd((N,), 0.02, 13, dev)
@@ -407,6 +409,9 @@ def test_gemm_fast_path_forms(ops, dev, M, N, K):
     first = ops.gemm(a, w, b)
     for _ in range(3):
         assert torch.equal(ops.gemm(a, w, b), first)
+    # the tile form follows the row count; an output element's bits do not (same accumulation order in every form)
+    for lo, hi in ((0, min(M, 256)), (M // 2, min(M, M // 2 + 100))):
+        assert torch.equal(ops.gemm(a[lo:hi], w, b), first[lo:hi]), (lo, hi)
     perm = torch.randperm(M, generator=torch.Generator().manual_seed(2)).int().to(dev)
     scat = ops.gemm(a, w, b, c_rows=perm)
     ref = torch.empty_like(first)
