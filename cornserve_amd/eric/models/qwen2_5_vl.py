@@ -505,6 +505,7 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
 
         for i, b in enumerate(pk["blocks"]):
             full = i in self.fullatt_block_indexes
+            pf_qkv = b["gu"]["w"] if hint else None
             pf_proj = b["down"]["w"] if hint else None
             pf_down = next_qkv(i) if hint else None
             if not full and fused_rows:
@@ -513,23 +514,23 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 if fold:
                     mark("gemm_qkv_attn_window")
                     ops.qkv_window_attn(xf, wp, bp, ix.cos_sin[:fused_rows], nh, scale, a_row_sumsq=ss[:fused_rows], norm_eps=eps,
-                                        out=att[:fused_rows], win_start=win_start, prefetch=b["gu"]["w"] if hint else None)
+                                        out=att[:fused_rows], win_start=win_start, prefetch=pf_qkv)
                 else:
                     mark("norm")
                     ops.rmsnorm(xf, b["n1"], eps, out=n[:fused_rows])
                     mark("gemm_qkv_attn_window")
                     ops.qkv_window_attn(n[:fused_rows], wp, bp, ix.cos_sin[:fused_rows], nh, scale, out=att[:fused_rows],
-                                        win_start=win_start, w_scale=wsc)
+                                        win_start=win_start, w_scale=wsc, prefetch=pf_qkv)
             if full or fused_rows < L:
                 lo = 0 if full else fused_rows           # first row the separate kernels work on in this block
                 if fold:
                     mark("gemm_qkv")
-                    self._g(x[lo:], self._plain_qkv(b), out=qkv[lo:], a_row_sumsq=ss[lo:], norm_eps=eps)
+                    self._g(x[lo:], self._plain_qkv(b), out=qkv[lo:], a_row_sumsq=ss[lo:], norm_eps=eps, prefetch=pf_qkv)
                 else:
                     mark("norm")
                     ops.rmsnorm(x[lo:], b["n1"], eps, out=n[lo:])
                     mark("gemm_qkv")
-                    self._g(n[lo:], self._plain_qkv(b), out=qkv[lo:])
+                    self._g(n[lo:], self._plain_qkv(b), out=qkv[lo:], prefetch=pf_qkv)
                 mark("attn_full" if full else "attn_window")
                 ops.attn_varlen_rotary_(qkv, plan_full if full else plan_win, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")

@@ -286,6 +286,14 @@ def test_qwen_batch_items_are_independent(dev):
     model.prefetch_rows = 0
     unhinted = model(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
     assert all(torch.equal(a, b) for a, b in zip(unhinted, together))
+    # ... on the other routes of the window blocks as well (separate kernels, unfolded norms, fp8 weights)
+    for kw in ({"fuse_window_attn": False}, {"fold_norm": False}, {"weight_format": "fp8_e4m3"},
+               {"weight_format": "fp8_e4m3", "fuse_window_attn": False}):
+        other, _, _ = build_qwen(dev, 2, (1,), seed=4, **kw)
+        hinted = other(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+        other.prefetch_rows = 0
+        plain = other(Modality.IMAGE, "", {"pixel_values": px, "image_grid_thw": grid})
+        assert all(torch.equal(a, b) for a, b in zip(hinted, plain)), kw
 
 
 def test_qwen_fp8_weights(dev):
