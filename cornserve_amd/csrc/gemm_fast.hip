@@ -56,8 +56,10 @@ int cs_gemm_fast(const CsGemmArgs& a, hipStream_t stream, bool* handled) {
   // Few rows and many columns: when 256x128 tiles fit in one round they put more compute units to work than the
   // forms above (1024 rows x 6912 columns: 216 workgroups against 176 of 256x160 or 108 of 256x256), and a launch
   // of one round is bound by what a single compute unit pulls in per K tile, not by the chip's throughput.  The
-  // accumulation order of an output element is the same in every tile form, so the choice changes no bit.
-  {
+  // accumulation order of an output element is the same in every tile form, so the choice changes no bit.  Taken
+  // for the SwiGLU epilogue only, where it measures faster inside the model (gate|up of one image); the QKV
+  // projection of two images (240 workgroups against 192) is faster alone and slower in the model.
+  if (a.epilogue == CS_EPI_SWIGLU) {
     const int64_t t128 = (int64_t)((a.M + 255) / 256) * ((a.N + 127) / 128);
     const double c128 = rounds_cost(a.M, a.N, 256, 128) * 1.10;
     if (t128 <= 256 && !few_rows && c128 < c160 - 0.05 && c128 < c256 - 0.05) return cs_gemm_fast_tile_256x128(a, stream);

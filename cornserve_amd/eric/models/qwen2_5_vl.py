@@ -505,7 +505,8 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
 
         for i, b in enumerate(pk["blocks"]):
             full = i in self.fullatt_block_indexes
-            pf_qkv = b["gu"]["w"] if hint else None
+            pf_qkv = b["gu"]["w"] if hint else None   # (from the one-launch window block only: the plain QKV GEMM of a
+            # small batch leaves too few compute units idle to read 18 MB in its own time -- measured slower)
             pf_proj = b["down"]["w"] if hint else None
             pf_down = next_qkv(i) if hint else None
             if not full and fused_rows:
@@ -525,12 +526,12 @@ class Qwen2_5_VisionTransformer(QwenVisionBase):
                 lo = 0 if full else fused_rows           # first row the separate kernels work on in this block
                 if fold:
                     mark("gemm_qkv")
-                    self._g(x[lo:], self._plain_qkv(b), out=qkv[lo:], a_row_sumsq=ss[lo:], norm_eps=eps, prefetch=pf_qkv)
+                    self._g(x[lo:], self._plain_qkv(b), out=qkv[lo:], a_row_sumsq=ss[lo:], norm_eps=eps)
                 else:
                     mark("norm")
                     ops.rmsnorm(x[lo:], b["n1"], eps, out=n[lo:])
                     mark("gemm_qkv")
-                    self._g(n[lo:], self._plain_qkv(b), out=qkv[lo:], prefetch=pf_qkv)
+                    self._g(n[lo:], self._plain_qkv(b), out=qkv[lo:])
                 mark("attn_full" if full else "attn_window")
                 ops.attn_varlen_rotary_(qkv, plan_full if full else plan_win, nh, d, scale, ix.cos_sin, out=att)
             mark("gemm_proj")

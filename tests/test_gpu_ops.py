@@ -392,8 +392,8 @@ def _epilogue_ref(ops, epi, base, res):
     (1000, 1280, 320),    # 256x160, row tail, 5 K tiles
     (300, 520, 448),      # 256x256 with row and column tails, 7 K tiles
     (8192, 1280, 192),    # 256x160, one tile per CU, 3 K tiles
-    (1000, 6912, 256),    # few rows, many columns: 256x128 over the whole width (216 workgroups in one round)
-    (2048, 3840, 192),    # the same choice at 240 workgroups
+    (1000, 6912, 256),    # few rows, many columns: the SwiGLU epilogue takes 256x128 over the whole width (216 workgroups)
+    (2048, 3840, 192),    # 256x160 in one round of 192 workgroups
 ])
 def test_gemm_fast_path_forms(ops, dev, M, N, K):
     a, w, b = rnd((M, K), 1.0, 11, dev), rnd((N, K), 0.05, 12, dev), rnd((N,), 0.02, 13, dev)
