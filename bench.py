@@ -48,9 +48,9 @@ if str(ROOT) not in sys.path:
 PEAK_BF16_TFLOPS = 2500.0   # MI355X dense bf16 MFMA peak (2.5 PFLOP/s, the published figure at 2.4 GHz)
 N_IMAGES = 8
 # HBM-side bytes per gate|up call (its two launches together), measured with rocprofv3 --pmc (not live):
-# FETCH_SIZE 93,147 + 18,179 KiB scaled by 2.00 (what the same counter reads for a plain 1 GiB copy) +
+# FETCH_SIZE 93,158 + 18,189 KiB scaled by 2.00 (what the same counter reads for a plain 1 GiB copy) +
 # WRITE_SIZE 49,152 + 6,144 KiB scaled by 1.00.
-GATE_UP_HBM_BYTES_PER_LAUNCH = int(((93147 + 18179) * 2.00 + (49152 + 6144) * 1.00) * 1024)
+GATE_UP_HBM_BYTES_PER_LAUNCH = int(((93158 + 18189) * 2.00 + (49152 + 6144) * 1.00) * 1024)
 GATE_UP_TRAFFIC_SOURCE = ("profiles/qwen2_5_vl_cfg2_bench_kernels_and_traffic.md (rocprofv3 --pmc runs of this script; a "
                           "constant read from that file, not a live measurement)")
 GRID = (1, 32, 32)          # 448 x 448, patch 14
